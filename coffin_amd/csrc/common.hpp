@@ -1,0 +1,79 @@
+// Shared device helpers and host-side status plumbing for the gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/coffin_mi355.h"
+
+namespace cmi {
+
+// ---------------------------------------------------------------- host status
+void set_error(const char *fmt, ...);
+int fail(int code, const char *fmt, ...);
+int check_launch(const char *what);
+
+#define CMI_REQUIRE(cond, code, ...)                 \
+    do {                                             \
+        if (!(cond)) return cmi::fail(code, __VA_ARGS__); \
+    } while (0)
+
+static inline bool aligned(const void *p, uintptr_t a) {
+    return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
+}
+
+// ------------------------------------------------------------- device helpers
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef int v4i32 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t v) {
+    return __uint_as_float(v << 16);
+}
+
+// fp32 -> bf16 bit pattern, round to nearest even (finite inputs).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK,
+                                                      0xf, false));
+}
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp_i32(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xf, false);
+}
+
+// Sum over the 64 lanes of a wavefront in a fixed order; the total lands in
+// lane 63 (other lanes hold partial sums).
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+    v += dpp_f32<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
+    v += dpp_f32<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
+    v += dpp_f32<0x141, 0xf>(v);  // row_half_mirror
+    v += dpp_f32<0x140, 0xf>(v);  // row_mirror
+    v += dpp_f32<0x142, 0xa>(v);  // row_bcast15 into rows 1 and 3
+    v += dpp_f32<0x143, 0xc>(v);  // row_bcast31 into rows 2 and 3
+    return v;
+}
+
+// Max over the 64 lanes; every lane of row 3 ends with the wave maximum, lane
+// 63 included.  Inputs must be >= 0 (masked lanes contribute 0).
+__device__ __forceinline__ float wave_max_to_lane63(float v) {
+    v = fmaxf(v, dpp_f32<0xB1, 0xf>(v));
+    v = fmaxf(v, dpp_f32<0x4E, 0xf>(v));
+    v = fmaxf(v, dpp_f32<0x141, 0xf>(v));
+    v = fmaxf(v, dpp_f32<0x140, 0xf>(v));
+    v = fmaxf(v, dpp_f32<0x142, 0xa>(v));
+    v = fmaxf(v, dpp_f32<0x143, 0xc>(v));
+    return v;
+}
+
+__device__ __forceinline__ float lane63(float v) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
+}  // namespace cmi

@@ -1,0 +1,260 @@
+// W4A8 GEMV for 1..16 activation rows on the re-laid-out int4 weight.
+//
+//   sum_g  = sum_{k in group g} xq[m,k] * (code(n,k) - 8)     int32, exact
+//   total  = fma((float)sum_g, ws[n,g], total)                 g = 0,1,.. from 0.f
+//   y[m,n] = bf16(total * xs[m])
+//
+// HBM-bound on the packed weight (half a byte per element), read once with
+// 16-byte loads; a half-wavefront (32 lanes, 512 contiguous bytes) walks one
+// output row so that 2560-wide rows (1280 B) fill whole loads.  No MFMA:
+// nibbles are split with two AND/shift ops per word into the byte operands of
+// v_dot4_i32_i8, whose accumulator starts at -8 * sum(xq) so the unsigned
+// codes never need re-biasing.  Four adjacent lanes own one group of 128 k;
+// their int32 partials are added with two DPP quad permutes.  The fp32 part of
+// the arithmetic is a strict chain over the groups and is order sensitive, so
+// group sums go through LDS and one lane per (row, m) walks them in order:
+// the result does not depend on how K was split over wavefronts or trips.
+#include "common.hpp"
+
+namespace {
+
+using namespace cmi;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int GS = 128;  // group size the kernels are built for
+
+struct W4Args {
+    const uint8_t *w4;
+    const float *ws;
+    const int8_t *xq;
+    const float *xs;
+    uint16_t *y;
+    int32_t *group_acc;
+    int M, N, K;
+    int G;        // K / 128
+    int nchunks;  // K / 32: 16-byte chunks per row
+    int KW, teams, iters;
+};
+
+template <int M, int R2, int CH>
+__global__ void __launch_bounds__(256)
+gemv_w4a8_kernel(const W4Args a) {
+    constexpr int ROWS = 2 * R2;
+    extern __shared__ int32_t sums[];  // [teams][iters*KW*CH*8 groups][ROWS*M]
+    const int lane = threadIdx.x & 63;
+    const int half = lane >> 5, hl = lane & 31;
+    const int wave = threadIdx.x >> 6;
+    const int team = wave / a.KW;
+    const int kw = wave - team * a.KW;
+    const int n0 = (blockIdx.x * a.teams + team) * ROWS;
+    int32_t *team_sums = sums + (size_t)team * (a.iters * a.KW * CH * 8) * (ROWS * M);
+    const int row_bytes = a.K / 2;
+
+    const u32x4 *wrow[R2];
+#pragma unroll
+    for (int rr = 0; rr < R2; ++rr) {
+        int n = n0 + 2 * rr + half;
+        n = n < a.N ? n : a.N - 1;
+        wrow[rr] = reinterpret_cast<const u32x4 *>(a.w4 + (size_t)n * row_bytes);
+    }
+
+    for (int it = 0; it < a.iters; ++it) {
+        const int hs0 = (it * a.KW + kw) * CH;
+        int chunk[CH];
+        bool live[CH];
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+            chunk[j] = (hs0 + j) * 32 + hl;
+            live[j] = chunk[j] < a.nchunks;
+        }
+
+        u32x4 wr[R2][CH];
+#pragma unroll
+        for (int rr = 0; rr < R2; ++rr)
+#pragma unroll
+            for (int j = 0; j < CH; ++j)
+                wr[rr][j] = live[j] ? __builtin_nontemporal_load(wrow[rr] + chunk[j]) : u32x4{0, 0, 0, 0};
+
+        // Activations of this lane's chunks: 32 int8 per (m, chunk), and the
+        // accumulator start value -8 * sum of those 32.
+        uint4 xr[M][CH][2];
+        int xinit[M][CH];
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            const int mrow = m < a.M ? m : a.M - 1;
+            const uint4 *xp = reinterpret_cast<const uint4 *>(a.xq + (size_t)mrow * a.K);
+#pragma unroll
+            for (int j = 0; j < CH; ++j) {
+                if (live[j]) {
+                    xr[m][j][0] = xp[2 * chunk[j]];
+                    xr[m][j][1] = xp[2 * chunk[j] + 1];
+                } else {
+                    xr[m][j][0] = make_uint4(0, 0, 0, 0);
+                    xr[m][j][1] = make_uint4(0, 0, 0, 0);
+                }
+                const uint32_t xv[8] = {xr[m][j][0].x, xr[m][j][0].y, xr[m][j][0].z, xr[m][j][0].w,
+                                        xr[m][j][1].x, xr[m][j][1].y, xr[m][j][1].z, xr[m][j][1].w};
+                int s = 0;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) s = __builtin_amdgcn_sdot4((int)xv[i], 0x01010101, s, false);
+                xinit[m][j] = -8 * s;
+            }
+        }
+
+#pragma unroll
+        for (int rr = 0; rr < R2; ++rr) {
+#pragma unroll
+            for (int j = 0; j < CH; ++j) {
+                const uint32_t w[4] = {wr[rr][j].x, wr[rr][j].y, wr[rr][j].z, wr[rr][j].w};
+                uint32_t op[8];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    op[2 * i] = w[i] & 0x0F0F0F0Fu;
+                    op[2 * i + 1] = (w[i] >> 4) & 0x0F0F0F0Fu;
+                }
+                const int group = chunk[j] >> 2;
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    const uint32_t xv[8] = {xr[m][j][0].x, xr[m][j][0].y, xr[m][j][0].z,
+                                            xr[m][j][0].w, xr[m][j][1].x, xr[m][j][1].y,
+                                            xr[m][j][1].z, xr[m][j][1].w};
+                    int acc = xinit[m][j];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i)
+                        acc = __builtin_amdgcn_sdot4((int)op[i], (int)xv[i], acc, false);
+                    acc += dpp_i32<0xB1, 0xf>(acc);  // quad_perm [1,0,3,2]
+                    acc += dpp_i32<0x4E, 0xf>(acc);  // quad_perm [2,3,0,1]
+                    if ((hl & 3) == 0 && live[j])
+                        team_sums[group * (ROWS * M) + (2 * rr + half) * M + m] = acc;
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    if (kw == 0 && lane < ROWS * M) {
+        const int r = lane / M, m = lane - r * M;
+        const int n = n0 + r;
+        if (n < a.N && m < a.M) {
+            const float *wsn = a.ws + (size_t)n * a.G;
+            float total = 0.f;
+            for (int g = 0; g < a.G; ++g) {
+                const int s = team_sums[g * (ROWS * M) + lane];
+                if (a.group_acc) a.group_acc[((size_t)m * a.G + g) * a.N + n] = s;
+                total = fmaf((float)s, wsn[g], total);
+            }
+            a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * a.xs[m]);
+        }
+    }
+}
+
+struct Plan {
+    int mt, r2, ch, kw, teams, iters;
+};
+
+Plan make_plan(int M, int N, int K) {
+    Plan p;
+    p.mt = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
+    const int chmax = p.mt <= 4 ? 4 : p.mt <= 8 ? 2 : 1;
+    const int nhseg = (K / 32 + 31) / 32;
+    // Up to a quarter of padding is accepted for fewer trips (more loads in
+    // flight); then least padding, then fewest wavefronts per team.
+    long best = -1;
+    p.kw = 1; p.ch = 1; p.iters = nhseg;
+    for (int kw = 1; kw <= 4; kw *= 2) {
+        for (int ch = 1; ch <= chmax; ++ch) {
+            const int per_trip = kw * ch;
+            const int iters = (nhseg + per_trip - 1) / per_trip;
+            const int waste = iters * per_trip - nhseg;
+            if (waste * 4 > nhseg && waste > 1) continue;
+            const long cost = (long)iters * 10000 + waste * 100 + kw;
+            if (best < 0 || cost < best) {
+                best = cost;
+                p.kw = kw; p.ch = ch; p.iters = iters;
+            }
+        }
+    }
+    p.teams = 4 / p.kw;
+    int r2 = 2;
+    const long target_waves = 256L * 8;
+    while (r2 > 1 && (long)((N + 2 * r2 - 1) / (2 * r2)) * p.kw < target_waves) r2 >>= 1;
+    while (2 * r2 * p.mt > 64) r2 >>= 1;
+    p.r2 = r2 < 1 ? 1 : r2;
+    // Group sums of a whole team live in LDS; shrink the team count, then the
+    // row block, until they fit comfortably.
+    auto lds_bytes = [&]() {
+        return (size_t)4 * p.teams * (p.iters * p.kw * p.ch * 8) * (2 * p.r2 * p.mt);
+    };
+    while (lds_bytes() > 48 * 1024 && p.teams > 1) p.teams >>= 1;
+    while (lds_bytes() > 48 * 1024 && p.r2 > 1) p.r2 >>= 1;
+    return p;
+}
+
+template <int M, int R2, int CH>
+int launch(const W4Args &a, hipStream_t st) {
+    const int rows_per_block = 2 * R2 * a.teams;
+    const dim3 grid((a.N + rows_per_block - 1) / rows_per_block);
+    const size_t lds = sizeof(int32_t) * a.teams * (a.iters * a.KW * CH * 8) * (2 * R2 * M);
+    if (lds > 64 * 1024)
+        return fail(CMI_E_UNSUPPORTED, "cmi_gemv_w4a8: K=%d needs %zu bytes of LDS", a.K, lds);
+    gemv_w4a8_kernel<M, R2, CH><<<grid, dim3(64 * a.KW * a.teams), lds, st>>>(a);
+    return check_launch("cmi_gemv_w4a8");
+}
+
+template <int M, int R2>
+int dispatch_ch(const W4Args &a, int ch, hipStream_t st) {
+    constexpr int CHMAX = M <= 4 ? 4 : M <= 8 ? 2 : 1;
+    if (ch == 1) return launch<M, R2, 1>(a, st);
+    if constexpr (CHMAX >= 2) if (ch == 2) return launch<M, R2, 2>(a, st);
+    if constexpr (CHMAX >= 4) {
+        if (ch == 3) return launch<M, R2, 3>(a, st);
+        if (ch == 4) return launch<M, R2, 4>(a, st);
+    }
+    return fail(CMI_E_UNSUPPORTED, "cmi_gemv_w4a8: no kernel for M-tile %d with %d chunks", M, ch);
+}
+
+template <int M>
+int dispatch_r(const W4Args &a, const Plan &p, hipStream_t st) {
+    if (p.r2 == 1) return dispatch_ch<M, 1>(a, p.ch, st);
+    if constexpr (4 * M <= 64) if (p.r2 == 2) return dispatch_ch<M, 2>(a, p.ch, st);
+    return fail(CMI_E_UNSUPPORTED, "cmi_gemv_w4a8: no kernel for %d row pairs", p.r2);
+}
+
+}  // namespace
+
+extern "C" int cmi_gemv_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs,
+                             void *y, int32_t *group_acc, int M, int N, int K, int gs,
+                             void *stream) {
+    CMI_REQUIRE(w4 && ws && xq && xs && y, CMI_E_ARG, "cmi_gemv_w4a8: null pointer");
+    CMI_REQUIRE(M >= 1 && M <= 16, CMI_E_UNSUPPORTED, "cmi_gemv_w4a8: M=%d outside 1..16", M);
+    CMI_REQUIRE(N >= 1 && K >= GS, CMI_E_ARG, "cmi_gemv_w4a8: bad shape N=%d K=%d", N, K);
+    CMI_REQUIRE(gs == GS, CMI_E_UNSUPPORTED, "cmi_gemv_w4a8: group size %d, kernels are built for %d", gs, GS);
+    CMI_REQUIRE(K % GS == 0, CMI_E_UNSUPPORTED, "cmi_gemv_w4a8: K=%d is not a multiple of %d", K, GS);
+    CMI_REQUIRE(aligned(w4, 16) && aligned(xq, 16), CMI_E_ARG,
+                "cmi_gemv_w4a8: w4 and xq must be 16-byte aligned");
+    const Plan p = make_plan(M, N, K);
+    W4Args a;
+    a.w4 = w4;
+    a.ws = ws;
+    a.xq = xq;
+    a.xs = xs;
+    a.y = static_cast<uint16_t *>(y);
+    a.group_acc = group_acc;
+    a.M = M;
+    a.N = N;
+    a.K = K;
+    a.G = K / GS;
+    a.nchunks = K / 32;
+    a.KW = p.kw;
+    a.teams = p.teams;
+    a.iters = p.iters;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (p.mt) {
+        case 1: return dispatch_r<1>(a, p, st);
+        case 2: return dispatch_r<2>(a, p, st);
+        case 4: return dispatch_r<4>(a, p, st);
+        case 8: return dispatch_r<8>(a, p, st);
+        default: return dispatch_r<16>(a, p, st);
+    }
+}

@@ -1,0 +1,102 @@
+/*
+ * C ABI of the MI355X (gfx950) quantized-linear kernels.
+ *
+ * This is the whole boundary between the host adapter and the device code:
+ * plain device pointers, sizes and a HIP stream, `int` status out.  Each entry
+ * point names the reference interface it stands in for (paths relative to the
+ * MuWinds/coffin tree).  The reference binds its kernels with pybind11 and
+ * torch types; a maintainer replaces those bindings with the ctypes stub in
+ * coffin_amd/_native.py.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer valid on the current HIP device;
+ *   - bf16 tensors are passed as `const void*` / `void*` (16-bit patterns);
+ *   - all tensors are dense row-major unless a leading dimension is given;
+ *   - `stream` is a hipStream_t (NULL = the legacy default stream; callers on
+ *     torch pass torch.cuda.current_stream().cuda_stream);
+ *   - nothing synchronises, allocates or reads device memory on the host;
+ *   - return 0 on success, otherwise one of CMI_E_* and a message retrievable
+ *     with cmi_last_error() (thread-local).
+ */
+#ifndef COFFIN_MI355_H
+#define COFFIN_MI355_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CMI_OK 0
+#define CMI_E_ARG 1         /* null pointer, non-positive size, misalignment */
+#define CMI_E_UNSUPPORTED 2 /* shape outside what the kernels are built for   */
+#define CMI_E_HIP 3         /* a HIP runtime call failed                       */
+
+/* ABI version; bumped when a signature changes. */
+int cmi_abi_version(void);
+
+/* Message for the last non-zero status returned on this thread ("" if none). */
+const char *cmi_last_error(void);
+
+/* Per-token symmetric int8 quantisation, x bf16 [M,K] -> q int8 [M,K], s fp32 [M]:
+ *   s = max(amax_k |x|, 1e-5) / 127 ;  q = clamp(rne(x / s), -127, 127)
+ * with an IEEE fp32 division.  Replaces Ops.kv_quant
+ * (backends/protocol.py:252-258, spec backends/reference/__init__.py:367-390)
+ * and the native quant_act_i8 (backends/corex/kernels/w8a8.cu:75-107,
+ * bound at backends/corex/kernels/w8a8.cu:213-240). */
+int cmi_quant_act_i8(const void *x, int8_t *q, float *s, int M, int K, void *stream);
+
+/* int8 weight-only GEMV, 1 <= M <= 16:
+ *   y[m,n] = bf16( ws[n] * sum_k wq[n,k] * x[m,k] ),  fp32 accumulation,
+ * wq int8 [N,K], ws fp32 [N], x bf16 [M,K], y bf16 [M,N].  K % 16 == 0.
+ * Row m of a batched call is bit-identical to the M=1 call on x[m].
+ * Replaces gemv_nk_i8 / gemv_nk_i8_m (backends/corex/kernels/gemv.cu:838-990,
+ * called from backends/corex/__init__.py:424,533) and gemv_w8a16*
+ * (backends/hip/kernels/gemv_int8.cu:61-212). */
+int cmi_gemv_w8a16(const int8_t *wq, const float *ws, const void *x, void *y,
+                   int M, int N, int K, void *stream);
+
+/* One-time re-layout of a W4A8Weight for the device kernels.
+ *   in : packed u8 [ceil(K/2), N] (low nibble = even k, code = q+8) and
+ *        scale fp32 [K/gs, N]      (w4a8_weights.py:14-20,28-53)
+ *   out: w4 u8 [N, K/2] with, inside every 32-bit word, nibble 2i = code of
+ *        k0+i and nibble 2i+1 = code of k0+4+i (k0 = 8*word index), and
+ *        ws fp32 [N, K/gs].
+ * K % 32 == 0, gs % 32 == 0, K % gs == 0.  Plays the role of the load-time
+ * repack a backend may do at its own cost (backends/protocol.py:118-126,
+ * backends/corex/pack.py:323-359). */
+int cmi_w4_repack(const uint8_t *packed, const float *scale, uint8_t *w4, float *ws,
+                  int N, int K, int gs, void *stream);
+
+/* W4A8 GEMV, 1 <= M <= 16, on the re-laid-out weight:
+ *   sum_g = sum_{k in g} xq[m,k]*(code-8)           (int32, exact)
+ *   total = fma((float)sum_g, ws[n,g], total)        (g ascending, from 0)
+ *   y[m,n] = bf16(total * xs[m])
+ * Replaces w4a8_gemv = w4a8_dot + w4a8_finish
+ * (backends/corex/kernels/w4a8.cu:56-195, called from
+ * backends/corex/__init__.py:649).  group_acc (nullable) receives the int32
+ * sums as [M, K/gs, N] for parity checks. */
+int cmi_gemv_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs,
+                  void *y, int32_t *group_acc, int M, int N, int K, int gs, void *stream);
+
+/* W8A8 GEMM with fused epilogue:
+ *   acc[m,n] = sum_k xq[m,k]*wq[n,k]  (int32) ; y[m,n] = bf16((float)acc*xs[m]*ws[n])
+ * xq int8 [M,K], wq int8 [N,K], y bf16 with row stride ldy >= N.  K % 64 == 0.
+ * acc_out (nullable) receives the int32 accumulators as [M,N].
+ * Replaces w8a8_gemm + w8a8_epilogue (backends/corex/kernels/w8a8.cu:195-211,
+ * 289-336) and w8a8_gemm_tcu (backends/corex/kernels/w8a8_tcu.cu:276-384),
+ * called from backends/corex/__init__.py:1587-1608. */
+int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws,
+                  void *y, int32_t *acc_out, int M, int N, int K, int ldy, void *stream);
+
+/* W4A8 GEMM on the re-laid-out weight; same arithmetic as cmi_gemv_w4a8 for
+ * any M.  K % 128 == 0, gs == 128.  Replaces w4a8_gemm_tcu
+ * (backends/corex/kernels/w8a8_tcu.cu:453-574, called from
+ * backends/corex/__init__.py:647). group_acc as in cmi_gemv_w4a8. */
+int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs,
+                  void *y, int32_t *group_acc, int M, int N, int K, int gs, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COFFIN_MI355_H */
