@@ -1,0 +1,294 @@
+"""Adapters behind the ``linear*`` / ``kv_quant`` table entries on MI355X.
+
+Each module-level function whose name is a contract name is that op's native
+entry (the name-is-registration rule of backends/protocol.py:582-612); the
+vendor file collects them into the ``Ops`` table.  Signatures, return shapes
+and error behaviour follow backends/protocol.py:143-159,252-258 and the corex
+adapters they stand in for (backends/corex/__init__.py:396-425 ``linear``,
+:495-546 ``_gemv_rows``, :576-651 ``_w4_rows``, :1557-1609 ``_w8a8_rows``,
+:1612-1670 ``linear_prefill``).
+
+Routing, by storage type first (never by op name), then by row count:
+
+=================  ==========================  =================================
+weight             rows                        kernel
+=================  ==========================  =================================
+QWeight (int8)     1..16 (any entry)           int8 weight-only GEMV
+QWeight            > 16, linear / linear_m /   weight-only GEMV, 16 rows at a
+                   linear_m_verify             time (numerics stay weight-only)
+QWeight            >= 64, linear_prefill       per-token quant + W8A8 MFMA GEMM
+W4A8Weight         1..16                       per-token quant + W4A8 GEMV
+W4A8Weight         > 16                        per-token quant + W4A8 MFMA GEMM
+plain tensor       any                         torch ``F.linear`` (not quantized,
+                                               outside this backend's scope)
+=================  ==========================  =================================
+
+Everything launches on torch's current stream; nothing synchronises or reads
+device memory on the host.  Outputs are fresh tensors; ``xq``/``xs`` scratch is
+private and cached by shape; weights are borrowed and never modified (the int4
+re-layout is a private copy made once per weight).
+"""
+
+from __future__ import annotations
+
+import ctypes
+import weakref
+
+import torch
+import torch.nn.functional as F
+
+from coffin_amd import _native
+
+#: Widest batch the GEMV kernels take in one launch.
+GEMV_MAX_ROWS = 16
+#: From this many rows ``linear_prefill`` quantizes activations and runs the
+#: int8 MFMA GEMM (the reference's corex backend draws the same line at 64,
+#: backends/corex/__init__.py:633,1655-1659).
+PREFILL_MIN_ROWS = 64
+#: W4A8 switches from the GEMV to the MFMA GEMM above this many rows.
+W4_GEMM_MIN_ROWS = 17
+
+_vp = ctypes.c_void_p
+
+
+def _ptr(t: torch.Tensor | None) -> ctypes.c_void_p:
+    return _vp(t.data_ptr()) if t is not None else _vp(0)
+
+
+def _stream() -> ctypes.c_void_p:
+    return _vp(torch.cuda.current_stream().cuda_stream)
+
+
+def _is_w4(w) -> bool:
+    return hasattr(w, "packed") and hasattr(w, "group_size")
+
+
+def _is_q8(w) -> bool:
+    return hasattr(w, "wq") and hasattr(w, "scale")
+
+
+def _on_gpu(t: torch.Tensor) -> bool:
+    return t.device.type == "cuda"
+
+
+# --------------------------------------------------------------- private state
+
+#: (rows, k, device) -> (xq int8 [rows,k], xs fp32 [rows]); single-threaded caller
+#: by contract (backends/corex/__init__.py:654-690 keeps the same kind of pool).
+_SCRATCH: dict = {}
+_SCRATCH_MAX = 32
+
+
+def _scratch(rows: int, k: int, device: torch.device):
+    key = (rows, k, device)
+    hit = _SCRATCH.get(key)
+    if hit is None:
+        if len(_SCRATCH) >= _SCRATCH_MAX:
+            _SCRATCH.clear()
+        hit = (torch.empty((rows, k), dtype=torch.int8, device=device),
+               torch.empty(rows, dtype=torch.float32, device=device))
+        _SCRATCH[key] = hit
+    return hit
+
+
+#: id(source tensor) -> device-layout copy, dropped when the source dies
+#: (same ownership rule as backends/corex/pack.py:323-359).
+_REPACKED: dict = {}
+
+
+def _memo(source: torch.Tensor, make):
+    key = id(source)
+    hit = _REPACKED.get(key)
+    if hit is not None and hit[0]() is source:
+        return hit[1]
+    value = make()
+    ref = weakref.ref(source, lambda _r, key=key: _REPACKED.pop(key, None))
+    _REPACKED[key] = (ref, value)
+    return value
+
+
+def _q8_operands(w):
+    """``(wq int8 [N,K] contiguous, scale fp32 [N] contiguous)`` for a QWeight-like."""
+    wq, scale = w.wq, w.scale
+    if wq.dtype != torch.int8 or wq.dim() != 2:
+        raise ValueError(f"int8 weight must be 2-D int8, got {tuple(wq.shape)} {wq.dtype}")
+    if not wq.is_contiguous():
+        # e.g. a [K,N]-stored weight exposed as a transposed view: one private
+        # row-major copy, made once.
+        wq = _memo(w.wq, lambda: w.wq.contiguous())
+    if scale.dtype != torch.float32 or not scale.is_contiguous():
+        scale = _memo(w.scale, lambda: w.scale.to(torch.float32).contiguous())
+    return wq, scale
+
+
+def _w4_operands(w):
+    """Device layout ``(w4 uint8 [N,K/2], ws fp32 [N,G])`` of a W4A8Weight-like, built once."""
+    def make():
+        n, k, gs = int(w.n), int(w.k), int(w.group_size)
+        w4 = torch.empty((n, k // 2), dtype=torch.uint8, device=w.packed.device)
+        ws = torch.empty((n, k // gs), dtype=torch.float32, device=w.packed.device)
+        lib = _native.load()
+        with torch.cuda.device(w.packed.device):
+            _native.check(lib.cmi_w4_repack(_ptr(w.packed), _ptr(w.scale), _ptr(w4), _ptr(ws),
+                                            n, k, gs, _stream()), "w4 re-layout")
+        return w4, ws
+    return _memo(w.packed, make)
+
+
+# ------------------------------------------------------------------- kernels
+
+def _quantize_rows(act: torch.Tensor, xq: torch.Tensor, xs: torch.Tensor) -> None:
+    rows, k = act.shape
+    _native.check(_native.load().cmi_quant_act_i8(_ptr(act), _ptr(xq), _ptr(xs), rows, k,
+                                                  _stream()), "quant_act_i8")
+
+
+def _gemv_q8(w, act: torch.Tensor) -> torch.Tensor:
+    wq, scale = _q8_operands(w)
+    n, k = wq.shape
+    rows = act.shape[0]
+    out = torch.empty((rows, n), dtype=torch.bfloat16, device=act.device)
+    lib = _native.load()
+    stream = _stream()
+    for lo in range(0, rows, GEMV_MAX_ROWS):
+        m = min(GEMV_MAX_ROWS, rows - lo)
+        _native.check(lib.cmi_gemv_w8a16(_ptr(wq), _ptr(scale), _vp(act.data_ptr() + lo * k * 2),
+                                         _vp(out.data_ptr() + lo * n * 2), m, n, k, stream),
+                      "gemv_w8a16")
+    return out
+
+
+def _gemm_q8(w, act: torch.Tensor) -> torch.Tensor:
+    wq, scale = _q8_operands(w)
+    n, k = wq.shape
+    rows = act.shape[0]
+    xq, xs = _scratch(rows, k, act.device)
+    out = torch.empty((rows, n), dtype=torch.bfloat16, device=act.device)
+    _quantize_rows(act, xq, xs)
+    _native.check(_native.load().cmi_gemm_w8a8(_ptr(xq), _ptr(wq), _ptr(xs), _ptr(scale),
+                                               _ptr(out), _vp(0), rows, n, k, n, _stream()),
+                  "gemm_w8a8")
+    return out
+
+
+def _rows_w4(w, act: torch.Tensor) -> torch.Tensor:
+    n, k, gs = int(w.n), int(w.k), int(w.group_size)
+    rows = act.shape[0]
+    w4, ws = _w4_operands(w)
+    xq, xs = _scratch(rows, k, act.device)
+    out = torch.empty((rows, n), dtype=torch.bfloat16, device=act.device)
+    if rows == 0:
+        return out
+    _quantize_rows(act, xq, xs)
+    lib = _native.load()
+    fn, what = ((lib.cmi_gemm_w4a8, "gemm_w4a8") if rows >= W4_GEMM_MIN_ROWS
+                else (lib.cmi_gemv_w4a8, "gemv_w4a8"))
+    _native.check(fn(_ptr(w4), _ptr(ws), _ptr(xq), _ptr(xs), _ptr(out), _vp(0), rows, n, k, gs,
+                     _stream()), what)
+    return out
+
+
+# ------------------------------------------------------------------ dispatch
+
+def _dense(w, x: torch.Tensor) -> torch.Tensor:
+    """Unquantized or non-bf16 call: the torch statement of the op, on x's device.
+
+    Same arithmetic as backends/reference/__init__.py:93-95; used for plain
+    tensors and for activation dtypes the kernels are not built for.
+    """
+    compute = torch.promote_types(x.dtype, torch.bfloat16)
+    if _is_q8(w):
+        dense = (w.wq.to(torch.float32) * w.scale.unsqueeze(1)).to(compute)
+    elif _is_w4(w):
+        dense = w.to(compute)
+    else:
+        dense = w.to(compute)
+    return F.linear(x.to(compute), dense).to(x.dtype)
+
+
+def _project(w, x: torch.Tensor, prefill: bool) -> torch.Tensor:
+    if not (_is_w4(w) or _is_q8(w)):
+        return _dense(w, x)
+    if not _on_gpu(x):
+        # A CPU tensor cannot reach the kernels and this backend has no CPU
+        # path for quantized weights: refuse instead of answering slowly.
+        raise ValueError("coffin_amd: quantized weights need activations on the GPU, "
+                         f"got {x.device}")
+    if x.dtype != torch.bfloat16:
+        return _dense(w, x)
+    k = int(w.k)
+    if x.dim() not in (1, 2) or x.shape[-1] != k:
+        raise ValueError(f"projection expects [K] or [M, K] activations with K={k}, "
+                         f"got {tuple(x.shape)}")
+    wdev = (w.packed if _is_w4(w) else w.wq).device
+    if x.device != wdev:
+        raise ValueError(f"weight on {wdev} and activation on {x.device} must share a device")
+    act = x if x.dim() == 2 else x.unsqueeze(0)
+    if not act.is_contiguous():
+        act = act.contiguous()
+    rows = act.shape[0]
+    if torch.cuda.current_device() != x.device.index:
+        with torch.cuda.device(x.device):
+            return _project(w, x, prefill)
+    if _is_w4(w):
+        out = _rows_w4(w, act)
+    elif rows == 0:
+        out = torch.empty((0, int(w.n)), dtype=x.dtype, device=x.device)
+    elif prefill and rows >= PREFILL_MIN_ROWS:
+        out = _gemm_q8(w, act)
+    else:
+        out = _gemv_q8(w, act)
+    return out[0] if x.dim() == 1 else out
+
+
+def linear(w, x: torch.Tensor) -> torch.Tensor:
+    """``linear(w, x) -> y``: ``x`` ``[K]`` or ``[C, K]``, ``y`` ``[N]`` or ``[C, N]``, dtype of ``x``."""
+    return _project(w, x, prefill=False)
+
+
+def linear_m(w, x: torch.Tensor) -> torch.Tensor:
+    """``linear_m(w, x[M, K]) -> [M, N]``: one weight read serves all rows."""
+    return _project(w, x, prefill=False)
+
+
+def linear_m_verify(w, x: torch.Tensor) -> torch.Tensor:
+    """Speculative-verify batches; same numerics as :func:`linear_m` on this backend."""
+    return _project(w, x, prefill=False)
+
+
+def linear_prefill(w, x: torch.Tensor) -> torch.Tensor:
+    """``linear_prefill(w, x[C, K]) -> [C, N]``: the GEMM regime (W8A8 from 64 rows up)."""
+    return _project(w, x, prefill=True)
+
+
+def kv_quant(x: torch.Tensor, out_q: torch.Tensor, out_s: torch.Tensor) -> torch.Tensor:
+    """Per-row symmetric int8 quantisation into caller-owned ``out_q`` / ``out_s``.
+
+    ``s = max(amax|x|, 1e-5)/127``, ``q = clamp(rne(x/s), -127, 127)``
+    (backends/reference/__init__.py:386-389).  bf16 rows on the GPU run the
+    kernel; other inputs take the same formula in torch.
+    """
+    if x.dim() != 2 or tuple(out_q.shape) != tuple(x.shape) or out_s.numel() != x.shape[0]:
+        raise ValueError("kv_quant expects x [M, N], out_q [M, N], out_s [M]")
+    native_ok = (_on_gpu(x) and x.dtype == torch.bfloat16 and x.is_contiguous()
+                 and out_q.dtype == torch.int8 and out_q.is_contiguous()
+                 and out_s.dtype == torch.float32 and out_s.is_contiguous()
+                 and out_q.device == x.device and out_s.device == x.device)
+    if not native_ok:
+        xf = x.to(torch.float32)
+        s = xf.abs().amax(dim=-1).clamp_min(1e-5) / 127.0
+        out_s.copy_(s.reshape(out_s.shape))
+        out_q.copy_(torch.round(xf / s.unsqueeze(-1)).clamp_(-127, 127).to(torch.int8))
+        return out_q
+    with torch.cuda.device(x.device):
+        _quantize_rows(x, out_q, out_s)
+    return out_q
+
+
+#: Contract names this module answers natively.
+NATIVE_NAMES = ("linear", "linear_m", "linear_m_verify", "linear_prefill", "kv_quant")
+
+
+def native_table() -> dict:
+    """``{contract name: adapter}`` for the vendor file's ``build_ops``."""
+    return {name: globals()[name] for name in NATIVE_NAMES}

@@ -305,13 +305,13 @@ int launch(GemmArgs &a, hipStream_t st, const char *what) {
 extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws,
                              void *y, int32_t *acc_out, int M, int N, int K, int ldy,
                              void *stream) {
-    CMI_REQUIRE(xq && wq && xs && ws && y, CMI_E_ARG, "cmi_gemm_w8a8: null pointer");
     CMI_REQUIRE(M >= 0 && N >= 1 && K >= 16, CMI_E_ARG, "cmi_gemm_w8a8: bad shape M=%d N=%d K=%d", M, N, K);
+    if (M == 0) return CMI_OK;  // an empty batch has no storage to point at
+    CMI_REQUIRE(xq && wq && xs && ws && y, CMI_E_ARG, "cmi_gemm_w8a8: null pointer");
     CMI_REQUIRE(ldy >= N, CMI_E_ARG, "cmi_gemm_w8a8: ldy=%d is smaller than N=%d", ldy, N);
     CMI_REQUIRE(K % 16 == 0, CMI_E_UNSUPPORTED, "cmi_gemm_w8a8: K=%d is not a multiple of 16", K);
     CMI_REQUIRE(aligned(xq, 16) && aligned(wq, 16), CMI_E_ARG,
                 "cmi_gemm_w8a8: xq and wq must be 16-byte aligned");
-    if (M == 0) return CMI_OK;
     GemmArgs a;
     a.xq = xq;
     a.w = wq;
@@ -330,13 +330,13 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
 extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs,
                              void *y, int32_t *group_acc, int M, int N, int K, int gs,
                              void *stream) {
-    CMI_REQUIRE(w4 && ws && xq && xs && y, CMI_E_ARG, "cmi_gemm_w4a8: null pointer");
     CMI_REQUIRE(M >= 0 && N >= 1 && K >= BK, CMI_E_ARG, "cmi_gemm_w4a8: bad shape M=%d N=%d K=%d", M, N, K);
+    if (M == 0) return CMI_OK;  // an empty batch has no storage to point at
+    CMI_REQUIRE(w4 && ws && xq && xs && y, CMI_E_ARG, "cmi_gemm_w4a8: null pointer");
     CMI_REQUIRE(gs == BK, CMI_E_UNSUPPORTED, "cmi_gemm_w4a8: group size %d, kernels are built for %d", gs, BK);
     CMI_REQUIRE(K % BK == 0, CMI_E_UNSUPPORTED, "cmi_gemm_w4a8: K=%d is not a multiple of %d", K, BK);
     CMI_REQUIRE(aligned(xq, 16) && aligned(w4, 16), CMI_E_ARG,
                 "cmi_gemm_w4a8: xq and w4 must be 16-byte aligned");
-    if (M == 0) return CMI_OK;
     GemmArgs a;
     a.xq = xq;
     a.w = w4;

@@ -114,9 +114,9 @@ quant_act_i8_scalar(const uint16_t *__restrict__ x, int8_t *__restrict__ q,
 
 extern "C" int cmi_quant_act_i8(const void *x, int8_t *q, float *s, int M, int K,
                                 void *stream) {
-    CMI_REQUIRE(x && q && s, CMI_E_ARG, "cmi_quant_act_i8: null pointer");
     CMI_REQUIRE(M >= 0 && K > 0, CMI_E_ARG, "cmi_quant_act_i8: bad shape M=%d K=%d", M, K);
-    if (M == 0) return CMI_OK;
+    if (M == 0) return CMI_OK;  // an empty batch has no storage to point at
+    CMI_REQUIRE(x && q && s, CMI_E_ARG, "cmi_quant_act_i8: null pointer");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 grid(M), block(QUANT_THREADS);
     if (K % 8 == 0 && aligned(x, 16) && aligned(q, 8)) {

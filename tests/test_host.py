@@ -1,0 +1,238 @@
+"""CPU-side checks: the contract mirror, weight containers, caller dispatch, the
+vendor declaration and the C-ABI library (load + symbols + argument checks; no
+kernel is launched here)."""
+
+from __future__ import annotations
+
+import ctypes
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from coffin_amd import _native, backend, contract, gemv, synth
+from coffin_amd.weights import (QWeight, W4A8Weight, dequantize_projection,
+                                quantize_projection)
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+# ------------------------------------------------------------------ contract
+
+def test_ops_table_names_and_errors():
+    assert contract.Ops.NAMES == ("linear", "linear_m", "linear_m_verify", "linear_prefill",
+                                  "kv_quant")
+    t = contract.Ops.from_mapping({"linear": lambda w, x: x})
+    assert t.implemented() == ("linear",) and "kv_quant" in t.missing()
+    with pytest.raises(ValueError, match="unknown op"):
+        contract.Ops.from_mapping({"linear_fast": lambda: None})
+    with pytest.raises(TypeError, match="callable or None"):
+        contract.Ops(linear=3)
+
+
+def test_vendor_spec_validation_and_declaration():
+    from coffin_amd.vendors import mi355x
+    spec = mi355x.SPEC
+    spec.validate()
+    assert spec.name == "mi355x" and spec.weight_layout == "nk" and spec.int8_weights
+    assert spec.has_kernels and callable(spec.build_ops)
+    assert spec.detection.namespace == "cuda" and spec.detection.hip
+    assert all(m == m.lower() for m in spec.detection.name_markers)
+    with pytest.raises(ValueError, match="weight_layout"):
+        contract.VendorSpec(name="x", detection=contract.Detection("cuda"),
+                            weight_layout="kk").validate()
+    with pytest.raises(ValueError, match="has_kernels"):
+        contract.VendorSpec(name="x", detection=contract.Detection("cuda"),
+                            has_kernels=True).validate()
+    if not torch.cuda.is_available():
+        # no card: claim is "not mine" and build_ops degrades to an empty table
+        assert contract.detect(spec.detection) == contract.CLAIM_NONE
+        assert mi355x.build_ops().implemented() == ()
+
+
+# ------------------------------------------------------------------- weights
+
+def test_qweight_matches_oracle_and_surface(orc):
+    g = synth.generator()
+    w = synth.dense_weight(70, 300, g)
+    q = QWeight.quantize(w, chunk_rows=32)                 # exercises the chunked path
+    wq, scale = orc.qweight_quantize(w.numpy())
+    assert (q.wq.numpy() == wq).all() and (q.scale.numpy() == scale).all()
+    assert (q.n, q.k) == (70, 300) and q.wq.is_contiguous()
+    assert q.nbytes() == 70 * 300 + 4 * 70
+    d = q.dequant(torch.bfloat16)
+    assert (d.view(torch.int16).numpy().view(np.uint16) == orc.qweight_dequant_bf16(wq, scale)).all()
+    rows, s = q.rows(torch.tensor([3, 0]))
+    assert (rows == q.wq[[3, 0]]).all() and (s == q.scale[[3, 0]]).all()
+    z = QWeight.quantize(torch.zeros(2, 8))
+    assert (z.wq == 0).all() and torch.isfinite(z.scale).all()
+
+
+def test_w4_weight_matches_oracle_and_validates(orc):
+    g = synth.generator()
+    w = synth.dense_weight(20, 200, g)                     # K not a multiple of the group
+    packed, scale = quantize_projection(w, 128)
+    p2, s2 = orc.w4_quantize(w.numpy(), 128)
+    assert (packed.numpy() == p2).all() and (scale.numpy() == s2).all()
+    dense = dequantize_projection(packed, scale, k=200)
+    assert (dense.numpy() == orc.w4_dequant_f32(p2, s2, 200, 128)).all()
+    W = W4A8Weight(packed, scale, k=200)
+    assert W.shape == (20, 200) and (W.to(torch.float32) == dense).all()
+    assert (W.rows(torch.tensor([5, 1])) == dense[[5, 1]]).all()
+    with pytest.raises(ValueError):
+        W4A8Weight(packed.t(), scale, k=200)               # not contiguous [K/2, N]
+    with pytest.raises(ValueError):
+        W4A8Weight(packed, scale[:1].contiguous(), k=200)  # scale rows do not match groups
+    with pytest.raises(ValueError):
+        W4A8Weight(packed, scale, k=0)
+    with pytest.raises(ValueError):
+        quantize_projection(w[0])
+    a = W4A8Weight.quantize(synth.dense_weight(6, 256, g))
+    b = W4A8Weight.quantize(synth.dense_weight(10, 256, g))
+    fused = W4A8Weight.cat_output([a, b])
+    assert fused.n == 16 and (fused.to(torch.float32) ==
+                              torch.cat([a.to(torch.float32), b.to(torch.float32)])).all()
+    with pytest.raises(ValueError, match="share K"):
+        W4A8Weight.cat_output([a, W4A8Weight.quantize(synth.dense_weight(4, 128, g))])
+
+
+def test_synth_scales_are_fp16_representable():
+    g = synth.generator()
+    q = synth.int8_weight(32, 256, g)
+    w4 = synth.int4_weight(16, 256, g)
+    assert (q.scale.half().float() == q.scale).all()
+    assert (w4.scale.half().float() == w4.scale).all()
+    assert q.wq.abs().max() <= 127 and w4.packed.shape == (128, 16)
+    x = synth.activations(4, 256, g, outliers=True)
+    assert x.dtype == torch.bfloat16 and x.shape == (4, 256)
+    assert sum(synth.gemv_bytes(1, n, k) for _, n, k in synth.DECODE_LAYER) == 101_101_568
+    assert sum(synth.gemv_bytes(1, n, k) for _, n, k in synth.DECODE_LAYER_FUSED) == 101_086_208
+    assert synth.gemv_bytes(1, *synth.LM_HEAD[1:]) == 389_569_024
+    assert synth.w4_gemv_bytes(1, 9728, 2560) == 12_865_536
+    assert synth.gemm_ops(2048, 9728, 2560) == 2 * 2048 * 9728 * 2560 == 102_005_473_280
+
+
+# ------------------------------------------------------------ caller dispatch
+
+class Recorder:
+    """Fake op table: remembers which entry saw which row count."""
+
+    def __init__(self):
+        self.calls = []
+
+    def _make(name):
+        def fn(self, w, x):
+            self.calls.append((name, tuple(x.shape)))
+            n = w.shape[0] if isinstance(w, torch.Tensor) else w.n
+            return torch.zeros((n,) if x.dim() == 1 else (x.shape[0], n))
+        return fn
+
+    linear = _make("linear")
+    linear_m = _make("linear_m")
+    linear_m_verify = _make("linear_m_verify")
+    linear_prefill = _make("linear_prefill")
+
+
+def test_gemv_regimes_follow_row_count():
+    rec = Recorder()
+    op = gemv.GEMV(torch.zeros(6, 4), ops=rec)
+    assert (op.N, op.K) == (6, 4)
+    assert op(torch.zeros(4)).shape == (6,)
+    assert op.linear_m(torch.zeros(1, 4)).shape == (1, 6)      # one row -> linear on x[0]
+    assert op.linear_m(torch.zeros(5, 4)).shape == (5, 6)
+    assert op.linear_m_verify(torch.zeros(1, 4)).shape == (1, 6)
+    op.linear_m_verify(torch.zeros(3, 4))
+    assert op.prefill(torch.zeros(1, 4)).shape == (1, 6)
+    op.prefill(torch.zeros(2, 4)); op.prefill(torch.zeros(8, 4)); op.prefill(torch.zeros(9, 4))
+    assert rec.calls == [
+        ("linear", (4,)), ("linear", (4,)), ("linear_m", (5, 4)), ("linear", (4,)),
+        ("linear_m_verify", (3, 4)), ("linear", (4,)), ("linear_m", (2, 4)),
+        ("linear_m", (8, 4)), ("linear_prefill", (9, 4))]
+
+
+def test_gemv_group_fuses_and_splits():
+    g = synth.generator()
+    qa, qb = synth.int8_weight(6, 32, g), synth.int8_weight(10, 32, g)
+    rec = Recorder()
+    grp = gemv.GEMVGroup([qa, qb], ops=rec)
+    assert grp.sizes == [6, 10] and grp.g.N == 16 and grp.g.q is not None
+    assert (grp.g.w.wq[:6] == qa.wq).all() and (grp.g.w.scale[6:] == qb.scale).all()
+    a, b = grp(torch.zeros(32))
+    assert a.shape == (6,) and b.shape == (10,)
+    a, b = grp.linear_m(torch.zeros(1, 32))
+    assert a.shape == (1, 6) and b.shape == (1, 10)
+    a, b = grp.prefill(torch.zeros(12, 32))
+    assert a.shape == (12, 6) and b.shape == (12, 10)
+    wa, wb = synth.int4_weight(4, 128, g), synth.int4_weight(8, 128, g)
+    g4 = gemv.GEMVGroup([wa, wb], ops=rec)
+    assert g4.g.q4 is not None and g4.g.N == 12
+    with pytest.raises(ValueError, match="same weight format"):
+        gemv.GEMVGroup([qa, wa], ops=rec)
+    dense = gemv.GEMVGroup([torch.ones(2, 4), torch.zeros(3, 4)], ops=rec)
+    assert dense.g.w.shape == (5, 4)
+
+
+# --------------------------------------------------------------- adapters, CPU
+
+def test_adapter_answers_dense_and_refuses_cpu_quantized():
+    torch.manual_seed(1234)
+    w, x = torch.randn(8, 6), torch.randn(6)
+    # the reference's own dense assertion, tests/test_backends.py:451-457
+    assert torch.allclose(backend.linear(w, x), x @ w.t(), rtol=1e-5, atol=1e-6)
+    X = torch.randn(5, 6)
+    for fn in (backend.linear_m, backend.linear_m_verify, backend.linear_prefill):
+        assert torch.allclose(fn(w, X), X @ w.t(), rtol=1e-5, atol=1e-6)
+    q = QWeight.quantize(w)
+    with pytest.raises(ValueError, match="GPU"):
+        backend.linear(q, x.bfloat16())
+    assert set(backend.native_table()) == set(contract.Ops.NAMES)
+
+
+def test_kv_quant_torch_branch_matches_oracle(orc):
+    g = synth.generator()
+    x = synth.activations(5, 96, g)
+    out_q = torch.empty(5, 96, dtype=torch.int8)
+    out_s = torch.empty(5, dtype=torch.float32)
+    assert backend.kv_quant(x, out_q, out_s) is out_q
+    q, s = orc.quant_act_i8(x.view(torch.int16).numpy().view(np.uint16))
+    assert (out_q.numpy() == q).all() and (out_s.numpy() == s).all()
+    with pytest.raises(ValueError):
+        backend.kv_quant(x, out_q[:4], out_s)
+
+
+# --------------------------------------------------------------------- C ABI
+
+def _declared_symbols() -> list[str]:
+    text = (ROOT / "include" / "coffin_mi355.h").read_text()
+    return sorted(set(re.findall(r"\b(cmi_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _native.load()
+    names = _declared_symbols()
+    assert len(names) == 8
+    for name in names:
+        assert getattr(lib, name) is not None
+    assert set(_native.SIGNATURES) | {"cmi_abi_version", "cmi_last_error"} == set(names)
+    assert lib.cmi_abi_version() == _native.ABI_VERSION
+
+
+def test_entry_points_reject_bad_arguments_before_touching_the_device():
+    lib = _native.load()
+    null, one = ctypes.c_void_p(0), ctypes.c_void_p(256)
+    assert lib.cmi_quant_act_i8(null, one, one, 1, 8, null) == _native.E_ARG
+    assert "null pointer" in _native.last_error()
+    assert lib.cmi_gemv_w8a16(one, one, one, one, 17, 8, 16, null) == _native.E_UNSUPPORTED
+    assert "outside 1..16" in _native.last_error()
+    assert lib.cmi_gemv_w8a16(one, one, one, one, 1, 8, 24, null) == _native.E_UNSUPPORTED
+    assert lib.cmi_gemv_w8a16(ctypes.c_void_p(8), one, one, one, 1, 8, 16, null) == _native.E_ARG
+    assert lib.cmi_gemv_w4a8(one, one, one, one, one, null, 1, 8, 256, 64, null) == _native.E_UNSUPPORTED
+    assert lib.cmi_gemv_w4a8(one, one, one, one, one, null, 1, 8, 192, 128, null) == _native.E_UNSUPPORTED
+    assert lib.cmi_gemm_w8a8(one, one, one, one, one, null, 4, 8, 64, 4, null) == _native.E_ARG
+    assert "ldy" in _native.last_error()
+    assert lib.cmi_gemm_w4a8(one, one, one, one, one, null, 4, 8, 200, 128, null) == _native.E_UNSUPPORTED
+    assert lib.cmi_w4_repack(one, one, one, one, 8, 100, 128, null) == _native.E_UNSUPPORTED
+    with pytest.raises(ValueError, match="cmi_gemv_w8a16"):
+        _native.check(lib.cmi_gemv_w8a16(one, one, one, one, 0, 8, 16, null), "gemv")
