@@ -1,0 +1,331 @@
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+Headline workload (``config.workload``): every int8 weight-only decode GEMV of a
+Qwen3.5-4B-shaped model at M=1 -- 32 layers of {qkv 2560->6144, o 4096->2560,
+gate_up 2560->19456, down 9728->2560} (q/k/v and gate/up fused along N exactly
+as their callers fuse them) plus lm_head 2560->151936 -- 129 launches over
+3.6 GB of distinct weights per step, so neither the L2s nor the 256 MB
+Infinity Cache can serve a weight twice.  A step is replayed as one HIP graph
+(``--no-graph`` launches eagerly through the C ABI instead).
+
+``value`` is algorithmic bytes per step / step time, weights resident in HBM
+before the clock starts.  One JSON line is printed; ``extra`` carries the other
+configurations (M=4/8/16, W4A8 GEMV, W8A8/W4A8 prefill GEMM, the quantiser).
+"""
+
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, published
+INT8_PEAK_TOPS = 5033.0       # MI355X dense int8 MFMA, published (256 CU x 8192 op/clk x 2.4 GHz)
+LAYERS = 32
+
+METRIC = "decode GEMV HBM GB/s (% of peak) + W8A8 prefill int8 TOPS, Qwen3.5-4B shapes"
+
+
+def parse_args():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawTextHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--rows", type=int, default=1, help="activation rows M of the headline workload")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the CPU baseline leg (0 = skip)")
+    return ap.parse_args()
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; the path needs no collectives and "
+              "--gpus above 1 is not supported", file=sys.stderr)
+        return 2
+
+    import torch
+    from coffin_amd import _native, synth
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 3
+    lib = _native.load()
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    vp = ctypes.c_void_p
+
+    def ptr(t):
+        return vp(t.data_ptr())
+
+    def cur_stream():
+        return vp(torch.cuda.current_stream().cuda_stream)
+
+    def timed(fn, iters: int, warm: int = 2) -> float:
+        """Seconds per call of fn(), HIP events on the launch stream."""
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / iters
+
+    gen = synth.generator(1234, dev)
+
+    # ------------------------------------------------------------ headline: decode GEMVs
+    M = args.rows
+    shapes = list(synth.DECODE_LAYER_FUSED)
+    launches = []       # (wq, scale, x, y, M, N, K)
+    x_by_k = {}
+    for k in sorted({k for _, _, k in shapes} | {synth.LM_HEAD[2]}):
+        x_by_k[k] = synth.activations(16, k, gen)
+    for _layer in range(LAYERS):
+        for _, n, k in shapes:
+            q = synth.int8_weight(n, k, gen)
+            y = torch.empty((16, n), dtype=torch.bfloat16, device=dev)
+            launches.append((q.wq, q.scale, x_by_k[k], y, n, k))
+    _, n, k = synth.LM_HEAD
+    q = synth.int8_weight(n, k, gen)
+    launches.append((q.wq, q.scale, x_by_k[k], torch.empty((16, n), dtype=torch.bfloat16, device=dev), n, k))
+    weight_bytes = sum(w.numel() for w, *_ in launches)
+
+    def step_bytes(m):
+        return sum(synth.gemv_bytes(m, n_, k_) for *_, n_, k_ in launches)
+
+    def run_step(m):
+        st = cur_stream()
+        for wq, sc, x, y, n_, k_ in launches:
+            rc = lib.cmi_gemv_w8a16(ptr(wq), ptr(sc), ptr(x), ptr(y), m, n_, k_, st)
+            if rc:
+                _native.check(rc, "cmi_gemv_w8a16")
+
+    def make_runner(m):
+        """Eager launcher, or a HIP graph of one step checked against the eager result."""
+        if args.no_graph:
+            return (lambda: run_step(m)), "eager"
+        run_step(m)
+        torch.cuda.synchronize()
+        want = [y[:m].clone() for *_, y, _, _ in launches[:4]] + [launches[-1][3][:m].clone()]
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            run_step(m)
+        for _ in range(3):
+            for *_, y, _, _ in launches:
+                y[:m].zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            got = [y[:m] for *_, y, _, _ in launches[:4]] + [launches[-1][3][:m]]
+            if not all(bool((a.view(torch.int16) == b.view(torch.int16)).all()) for a, b in zip(want, got)):
+                raise RuntimeError("HIP graph replay differs from the eager step")
+        return graph.replay, "hipgraph"
+
+    runner, launch_mode = make_runner(M)
+    for _ in range(args.warmup):
+        runner()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    wall0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        runner()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - wall0
+    step_s = e0.elapsed_time(e1) * 1e-3 / args.steps
+    bytes_per_step = step_bytes(M)
+    value = bytes_per_step / step_s / 1e9
+    n_launch = len(launches)
+
+    result = {
+        "metric": METRIC,
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 weights x bf16 activations, fp32 accumulate",
+        "data": "synthetic",
+        "config": {
+            "workload": f"int8 weight-only decode GEMVs of a Qwen3.5-4B-shaped model, M={M}: "
+                        f"{LAYERS} layers x (qkv 2560->6144, o 4096->2560, gate_up 2560->19456, "
+                        f"down 9728->2560) + lm_head 2560->151936",
+            "rows": M,
+            "launches_per_step": n_launch,
+            "weight_bytes": weight_bytes,
+            "algorithmic_bytes_per_step": bytes_per_step,
+            "launch": launch_mode,
+            "wall_ms_per_step": round(wall / args.steps * 1e3, 4),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(value, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(value / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "kernel": "gemv_w8a16_kernel",
+            "avg_launch_us": round(step_s / n_launch * 1e6, 3),
+            "algorithmic_bytes_per_launch": round(bytes_per_step / n_launch),
+        },
+    }
+
+    # ------------------------------------------------------------------ secondary configs
+    if not args.no_extra:
+        extra = {}
+        for m in (1, 4, 8, 16):
+            if m == M:
+                extra[f"decode_gemv_int8_M{m}_GBps"] = round(value, 1)
+                continue
+            r, _ = make_runner(m)
+            t = timed(r, max(3, args.steps // 2), warm=2)
+            extra[f"decode_gemv_int8_M{m}_GBps"] = round(step_bytes(m) / t / 1e9, 1)
+        # per-shape kernel time, weights rotated through > 1 GB so HBM serves them
+        per_shape = {}
+        for name, n_, k_ in shapes + [synth.LM_HEAD]:
+            group = [l for l in launches if (l[4], l[5]) == (n_, k_)]
+            def one(group=group):
+                st = cur_stream()
+                for wq, sc, x, y, nn, kk in group:
+                    lib.cmi_gemv_w8a16(ptr(wq), ptr(sc), ptr(x), ptr(y), 1, nn, kk, st)
+            t = timed(one, 5) / len(group)
+            per_shape[name] = {"us": round(t * 1e6, 2),
+                               "GBps": round(synth.gemv_bytes(1, n_, k_) / t / 1e9, 1)}
+        extra["decode_gemv_int8_M1_per_shape_eager"] = per_shape
+        launches.clear()
+        torch.cuda.empty_cache()
+
+        # W4A8 decode GEMV (quantiser + GEMV, as the adapter issues them)
+        w4 = {}
+        for n_, k_ in ((9728, 2560), (2560, 9728)):
+            copies = 40
+            ws_ = []
+            for _ in range(copies):
+                w = synth.int4_weight(n_, k_, gen)
+                d4 = torch.empty((n_, k_ // 2), dtype=torch.uint8, device=dev)
+                ds = torch.empty((n_, k_ // 128), dtype=torch.float32, device=dev)
+                _native.check(lib.cmi_w4_repack(ptr(w.packed), ptr(w.scale), ptr(d4), ptr(ds), n_, k_, 128,
+                                                cur_stream()), "repack")
+                ws_.append((d4, ds))
+            torch.cuda.synchronize()
+            for m in (1, 16):
+                x = synth.activations(m, k_, gen)
+                xq = torch.empty((m, k_), dtype=torch.int8, device=dev)
+                xs = torch.empty(m, dtype=torch.float32, device=dev)
+                y = torch.empty((m, n_), dtype=torch.bfloat16, device=dev)
+                def one(m=m, x=x, xq=xq, xs=xs, y=y, ws_=ws_, n_=n_, k_=k_):
+                    st = cur_stream()
+                    for d4, ds in ws_:
+                        lib.cmi_quant_act_i8(ptr(x), ptr(xq), ptr(xs), m, k_, st)
+                        lib.cmi_gemv_w4a8(ptr(d4), ptr(ds), ptr(xq), ptr(xs), ptr(y), vp(0), m, n_, k_, 128, st)
+                t = timed(one, 5) / copies
+                w4[f"{k_}->{n_}_M{m}"] = {"us": round(t * 1e6, 2),
+                                          "GBps": round(synth.w4_gemv_bytes(m, n_, k_) / t / 1e9, 1)}
+            del ws_
+        extra["w4a8_gemv_quant_plus_gemv"] = w4
+        torch.cuda.empty_cache()
+
+        # W8A8 prefill GEMM (GEMM kernel alone, and quantiser + GEMM)
+        mm = {}
+        for m, n_ in ((2048, 9728), (2048, 4096), (512, 9728), (8192, 9728)):
+            k_ = 2560
+            q = synth.int8_weight(n_, k_, gen)
+            x = synth.activations(m, k_, gen, outliers=True)
+            xq = torch.empty((m, k_), dtype=torch.int8, device=dev)
+            xs = torch.empty(m, dtype=torch.float32, device=dev)
+            y = torch.empty((m, n_), dtype=torch.bfloat16, device=dev)
+            lib.cmi_quant_act_i8(ptr(x), ptr(xq), ptr(xs), m, k_, cur_stream())
+            def gemm():
+                lib.cmi_gemm_w8a8(ptr(xq), ptr(q.wq), ptr(xs), ptr(q.scale), ptr(y), vp(0), m, n_, k_, n_, cur_stream())
+            def both():
+                lib.cmi_quant_act_i8(ptr(x), ptr(xq), ptr(xs), m, k_, cur_stream())
+                gemm()
+            tg, tb = timed(gemm, 20), timed(both, 20)
+            tops = synth.gemm_ops(m, n_, k_) / tg / 1e12
+            mm[f"M{m}_N{n_}_K{k_}"] = {"gemm_us": round(tg * 1e6, 2), "tops": round(tops, 1),
+                                      "frac_of_int8_peak": round(tops / INT8_PEAK_TOPS, 4),
+                                      "quant_plus_gemm_us": round(tb * 1e6, 2)}
+        extra["w8a8_prefill_gemm"] = mm
+        extra["w8a8_prefill_int8_TOPS_M2048_N9728"] = mm["M2048_N9728_K2560"]["tops"]
+
+        # W4A8 prefill GEMM, larger dense shape
+        m, n_, k_ = 1024, 25600, 5120
+        w = synth.int4_weight(n_, k_, gen)
+        d4 = torch.empty((n_, k_ // 2), dtype=torch.uint8, device=dev)
+        ds = torch.empty((n_, k_ // 128), dtype=torch.float32, device=dev)
+        lib.cmi_w4_repack(ptr(w.packed), ptr(w.scale), ptr(d4), ptr(ds), n_, k_, 128, cur_stream())
+        x = synth.activations(m, k_, gen)
+        xq = torch.empty((m, k_), dtype=torch.int8, device=dev)
+        xs = torch.empty(m, dtype=torch.float32, device=dev)
+        y = torch.empty((m, n_), dtype=torch.bfloat16, device=dev)
+        lib.cmi_quant_act_i8(ptr(x), ptr(xq), ptr(xs), m, k_, cur_stream())
+        def w4gemm():
+            lib.cmi_gemm_w4a8(ptr(d4), ptr(ds), ptr(xq), ptr(xs), ptr(y), vp(0), m, n_, k_, 128, cur_stream())
+        t = timed(w4gemm, 10)
+        tops = synth.gemm_ops(m, n_, k_) / t / 1e12
+        extra["w4a8_prefill_gemm_M1024_N25600_K5120"] = {
+            "us": round(t * 1e6, 2), "tops": round(tops, 1), "frac_of_int8_peak": round(tops / INT8_PEAK_TOPS, 4)}
+
+        # quantiser alone at prefill size
+        m, k_ = 8192, 2560
+        x = synth.activations(m, k_, gen)
+        xq = torch.empty((m, k_), dtype=torch.int8, device=dev)
+        xs = torch.empty(m, dtype=torch.float32, device=dev)
+        t = timed(lambda: lib.cmi_quant_act_i8(ptr(x), ptr(xq), ptr(xs), m, k_, cur_stream()), 20)
+        extra["quant_act_i8_M8192_K2560"] = {"us": round(t * 1e6, 2),
+                                             "GBps": round(synth.quant_bytes(m, k_) / t / 1e9, 1)}
+        result["extra"] = extra
+
+    # ------------------------------------------------------------------ CPU baseline leg
+    if args.cpu_seconds > 0:
+        from oracle import oracle as orc
+        cpu_gen = synth.generator(1234)
+        ops = []
+        for _, n_, k_ in synth.DECODE_LAYER:
+            q = synth.int8_weight(n_, k_, cpu_gen)
+            x = synth.activations(1, k_, cpu_gen)
+            ops.append((q.wq.numpy(), q.scale.numpy(), orc.bits(x), synth.gemv_bytes(1, n_, k_)))
+        threads = min(orc.num_threads(), int(os.environ.get("OMP_NUM_THREADS", "0") or orc.num_threads()))
+        orc.set_num_threads(threads)
+        for wq, sc, xb, _ in ops[:1]:
+            orc.linear_qweight(wq, sc, xb)
+        done, t0 = 0, time.perf_counter()
+        passes = 0
+        while time.perf_counter() - t0 < args.cpu_seconds:
+            for wq, sc, xb, nb in ops:
+                orc.linear_qweight(wq, sc, xb)
+                done += nb
+            passes += 1
+        dt = time.perf_counter() - t0
+        result["cpu_baseline"] = {
+            "value": round(done / dt / 1e9, 3),
+            "unit": "GB/s",
+            "cores": threads,
+            "kind": "port",
+            "sample": f"{passes} passes over one decode layer (7 int8 GEMVs, M=1, 101.1 MB) through the C "
+                      f"oracle of the torch reference path (full weight dequant per call, as the reference does), "
+                      f"{dt:.1f} s on the host cores",
+        }
+
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -51,6 +51,11 @@ def load() -> ctypes.CDLL:
     if _load_error is not None:
         raise RuntimeError(_load_error)
     try:
+        # torch ships its own HIP runtime under the same soname as the system
+        # one; importing torch first makes the kernels bind to the runtime that
+        # owns torch's device memory and streams, whatever the import order of
+        # the caller.
+        import torch  # noqa: F401
         if not LIB_PATH.exists():
             raise OSError(f"{LIB_PATH} is missing; build it with `python -m coffin_amd.build`")
         lib = ctypes.CDLL(str(LIB_PATH))

@@ -1,0 +1,199 @@
+"""The table entries as coffin's callers use them, on the device.
+
+Mirrors the reference's own assertions for this path (tests/test_backends.py:451-469:
+``linear``, ``linear_m`` and ``linear_prefill`` agree with a matmul against the
+dequantised weight, and dispatch happens on the storage type) and the contract
+rules of backends/protocol.py:143-159,252-258.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from coffin_amd import backend, gemv, synth
+from coffin_amd.vendors import mi355x
+from coffin_amd.weights import QWeight, W4A8Weight
+from tests import gpu_util as G
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL = 2e-2      # tests/test_backends.py:54
+FP32_TOL = 1e-5      # tests/test_backends.py:57
+
+
+def _rel(got: torch.Tensor, ref: torch.Tensor) -> float:
+    """max |got-ref| / max |ref| -- the reference's metric (tests/test_backends.py:74-80)."""
+    return float((got.float() - ref.float()).abs().max() / ref.float().abs().max().clamp_min(1e-12))
+
+
+def _q8(n, k, g):
+    q = synth.int8_weight(n, k, g)
+    return QWeight(q.wq.to(G.DEV), q.scale.to(G.DEV))
+
+
+def _w4(n, k, g):
+    w = synth.int4_weight(n, k, g)
+    return W4A8Weight(w.packed.to(G.DEV), w.scale.to(G.DEV), k=k)
+
+
+def test_vendor_builds_the_native_table():
+    ops = mi355x.build_ops()
+    assert set(ops.implemented()) == {"linear", "linear_m", "linear_m_verify", "linear_prefill",
+                                      "kv_quant"}
+    from coffin_amd import contract
+    assert contract.detect(mi355x.SPEC.detection) == contract.CLAIM_NAME
+
+
+def test_reference_linear_assertions_on_device():
+    torch.manual_seed(1234)
+    w, x = torch.randn(8, 6, device=G.DEV), torch.randn(6, device=G.DEV)
+    assert _rel(backend.linear(w, x), x @ w.t()) < FP32_TOL
+    X = torch.randn(5, 6, device=G.DEV)
+    assert _rel(backend.linear_m(w, X), X @ w.t()) < FP32_TOL
+    assert _rel(backend.linear_prefill(w, X), X @ w.t()) < FP32_TOL
+    # int8 storage with fp32 activations: the torch statement, dispatch on storage type
+    q = QWeight.quantize(w)
+    dense = q.dequant(torch.float32)
+    assert _rel(backend.linear(q, x), x @ dense.t()) < FP32_TOL
+    assert _rel(backend.linear_m(q, X[:3]), X[:3] @ dense.t()) < FP32_TOL
+    assert _rel(backend.linear_prefill(q, X[:3]), X[:3] @ dense.t()) < FP32_TOL
+
+
+@pytest.mark.parametrize("rows", [None, 1, 2, 8, 16, 17, 40])
+def test_int8_entries_agree_with_dequant_matmul(rows):
+    g = synth.generator()
+    q = _q8(1536, 2560, g)
+    x = synth.activations(rows or 1, 2560, g).to(G.DEV)
+    x = x[0] if rows is None else x
+    dense = q.dequant(torch.float32)
+    ref = x.float() @ dense.t()
+    for fn in (backend.linear, backend.linear_m, backend.linear_m_verify, backend.linear_prefill):
+        y = fn(q, x)
+        assert y.dtype == x.dtype and y.shape == ref.shape and y.is_contiguous()
+        assert _rel(y, ref) < BF16_TOL
+    # weight-only entries are bit-identical to each other whatever the batch
+    a, b = backend.linear(q, x), backend.linear_m(q, x)
+    assert (a.view(torch.int16) == b.view(torch.int16)).all()
+    if rows is not None and rows > 1:
+        one = backend.linear(q, x[rows - 1])
+        assert (one.view(torch.int16) == a[rows - 1].view(torch.int16)).all()
+
+
+def test_prefill_switches_to_w8a8_and_matches_the_oracle(orc):
+    g = synth.generator()
+    q = _q8(1024, 2560, g)
+    x = synth.activations(200, 2560, g, outliers=True).to(G.DEV)
+    y = backend.linear_prefill(q, x)
+    xq, xs = orc.quant_act_i8(G.bits(x))
+    _, y_ref = orc.gemm_w8a8(xq, q.wq.cpu().numpy(), xs, q.scale.cpu().numpy(), want_acc=False)
+    assert (G.bits(y) == y_ref).all()
+    # below the threshold prefill keeps weight-only numerics
+    small = backend.linear_prefill(q, x[:63].contiguous())
+    assert (small.view(torch.int16) == backend.linear_m(q, x[:63].contiguous()).view(torch.int16)).all()
+    # and the W8A8 answer is the unquantised product up to int8 activation noise (rows
+    # with a x20 outlier have a 20x coarser step, hence the loose bound)
+    assert _rel(y, x.float() @ q.dequant(torch.float32).t()) < 1e-1
+
+
+@pytest.mark.parametrize("rows", [None, 1, 4, 16, 17, 64, 300])
+def test_w4_entries_match_the_oracle_bit_for_bit(orc, rows):
+    g = synth.generator()
+    w = _w4(768, 2560, g)
+    x = synth.activations(rows or 1, 2560, g).to(G.DEV)
+    xq, xs = orc.quant_act_i8(G.bits(x))
+    _, y_ref = orc.linear_w4a8(xq, xs, w.packed.cpu().numpy(), w.scale.cpu().numpy(), 2560, 128)
+    arg = x[0] if rows is None else x
+    for fn in (backend.linear, backend.linear_m, backend.linear_m_verify, backend.linear_prefill):
+        y = fn(w, arg)
+        assert y.dtype == torch.bfloat16
+        assert y.shape == ((768,) if rows is None else (x.shape[0], 768))
+        assert (G.bits(y).reshape(y_ref.shape) == y_ref).all()
+    # unquantised-activation reference (what the torch backend computes) is close
+    ref = x.float() @ w.to(torch.float32).t()
+    assert _rel(y.reshape(ref.shape), ref) < 5e-2
+
+
+def test_outputs_are_fresh_and_inputs_untouched():
+    g = synth.generator()
+    q, w = _q8(256, 512, g), _w4(256, 512, g)
+    x = synth.activations(3, 512, g).to(G.DEV)
+    keep = x.clone()
+    wq_keep, packed_keep = q.wq.clone(), w.packed.clone()
+    a, b = backend.linear(q, x), backend.linear(q, x)
+    c, d = backend.linear(w, x), backend.linear(w, x)
+    assert a.data_ptr() != b.data_ptr() and c.data_ptr() != d.data_ptr()
+    assert (x == keep).all() and (q.wq == wq_keep).all() and (w.packed == packed_keep).all()
+    # the re-laid-out int4 copy is made once per weight
+    from coffin_amd.backend import _w4_operands
+    assert _w4_operands(w)[0].data_ptr() == _w4_operands(w)[0].data_ptr()
+
+
+def test_shape_and_device_errors():
+    g = synth.generator()
+    q, w = _q8(64, 128, g), _w4(64, 128, g)
+    bad = torch.zeros(3, 64, dtype=torch.bfloat16, device=G.DEV)
+    for weight in (q, w):
+        with pytest.raises(ValueError):
+            backend.linear(weight, bad)
+        with pytest.raises(ValueError):
+            backend.linear(weight, torch.zeros(2, 3, 128, dtype=torch.bfloat16, device=G.DEV))
+        with pytest.raises(ValueError, match="GPU"):
+            backend.linear(weight, torch.zeros(128, dtype=torch.bfloat16))
+    odd = W4A8Weight(torch.full((128, 8), 0x88, dtype=torch.uint8, device=G.DEV),
+                     torch.ones((4, 8), device=G.DEV), k=256, group_size=64)
+    with pytest.raises(ValueError, match="group size"):
+        backend.linear(odd, torch.zeros(256, dtype=torch.bfloat16, device=G.DEV))
+    empty = backend.linear_m(q, torch.zeros(0, 128, dtype=torch.bfloat16, device=G.DEV))
+    assert empty.shape == (0, 64)
+
+
+def test_kv_quant_writes_through_caller_buffers(orc):
+    g = synth.generator()
+    x = synth.activations(9, 256, g).to(G.DEV)
+    out_q = torch.zeros(9, 256, dtype=torch.int8, device=G.DEV)
+    out_s = torch.zeros(9, dtype=torch.float32, device=G.DEV)
+    qp, sp = out_q.data_ptr(), out_s.data_ptr()
+    assert backend.kv_quant(x, out_q, out_s) is out_q
+    assert (out_q.data_ptr(), out_s.data_ptr()) == (qp, sp)
+    q, s = orc.quant_act_i8(G.bits(x))
+    assert (out_q.cpu().numpy() == q).all() and (out_s.cpu().numpy() == s).all()
+    # fp32 rows take the torch statement of the same formula
+    xf = x.float()
+    backend.kv_quant(xf, out_q, out_s)
+    assert (out_q.cpu().numpy() == q).all()
+
+
+def test_gemv_objects_on_device():
+    g = synth.generator()
+    qa, qb = _q8(512, 2560, g), _q8(256, 2560, g)
+    x = synth.activations(4, 2560, g).to(G.DEV)
+    single_a, single_b = gemv.GEMV(qa), gemv.GEMV(qb)
+    group = gemv.GEMVGroup([qa, qb])
+    fa, fb = group(x[0])
+    assert (fa.view(torch.int16) == single_a(x[0]).view(torch.int16)).all()
+    assert (fb.view(torch.int16) == single_b(x[0]).view(torch.int16)).all()
+    ma, mb = group.linear_m(x)
+    assert ma.shape == (4, 512) and mb.shape == (4, 256)
+    assert (ma.view(torch.int16) == single_a.linear_m(x).view(torch.int16)).all()
+    pa, _ = group.prefill(x[:1])
+    assert pa.shape == (1, 512)
+    wa, wb = _w4(256, 2560, g), _w4(128, 2560, g)
+    g4 = gemv.GEMVGroup([wa, wb])
+    ya, yb = g4(x[0])
+    assert (ya.view(torch.int16) == gemv.GEMV(wa)(x[0]).view(torch.int16)).all()
+    assert (yb.view(torch.int16) == gemv.GEMV(wb)(x[0]).view(torch.int16)).all()
+
+
+def test_launches_follow_the_current_stream():
+    g = synth.generator()
+    q = _q8(512, 2560, g)
+    x = synth.activations(1, 2560, g).to(G.DEV)
+    want = backend.linear(q, x)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        got = backend.linear(q, x)
+    side.synchronize()
+    assert (got.view(torch.int16) == want.view(torch.int16)).all()
