@@ -274,14 +274,16 @@ Plan make_plan(int M, int N, int K) {
     p.mt = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
     const int nseg = (K / 16 + 63) / 64;
     const int unit = unit_segments(nseg);
+    const int units = (nseg + unit - 1) / unit;
     const int chmax = p.mt <= 2 ? 4 : p.mt <= 4 ? 3 : 1;
     p.cht = unit < chmax ? unit : chmax;
     // balance the sub-trips of a unit (e.g. 4 segments at CHT<=3 -> 2 + 2)
     const int subtrips = (unit + p.cht - 1) / p.cht;
     p.cht = (unit + subtrips - 1) / subtrips;
     p.single = nseg <= p.cht;
+    // Two rows per wavefront; one when that would leave fewer than ~8 wavefronts per CU.
     p.r = p.mt >= 16 ? 1 : 2;
-    (void)N;
+    if ((long)((N + 1) / 2) * units < 2048) p.r = 1;
     return p;
 }
 
