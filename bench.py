@@ -43,6 +43,8 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one 256 MiB device-to-device copy (known traffic, for scaling HBM counters)")
     return ap.parse_args()
 
 
@@ -84,6 +86,13 @@ def main() -> int:
         return e0.elapsed_time(e1) * 1e-3 / iters
 
     gen = synth.generator(1234, dev)
+
+    if args.calibration_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)          # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
 
     # ------------------------------------------------------------ headline: decode GEMVs
     M = args.rows
