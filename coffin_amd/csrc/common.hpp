@@ -18,6 +18,10 @@ int check_launch(const char *what);
         if (!(cond)) return cmi::fail(code, __VA_ARGS__); \
     } while (0)
 
+// gemm_mfma.hip: register-staged W8A8 GEMM for K % 64 != 0 (see gemm_w8a8.hip for the fast path).
+int gemm_w8a8_generic(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws, void *y,
+                      int32_t *acc_out, int M, int N, int K, int ldy, void *stream);
+
 static inline bool aligned(const void *p, uintptr_t a) {
     return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
 }
@@ -25,6 +29,7 @@ static inline bool aligned(const void *p, uintptr_t a) {
 // ------------------------------------------------------------- device helpers
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef int v4i32 __attribute__((ext_vector_type(4)));
+typedef int v16i32 __attribute__((ext_vector_type(16)));
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t v) {
     return __uint_as_float(v << 16);

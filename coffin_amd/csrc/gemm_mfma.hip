@@ -302,16 +302,9 @@ int launch(GemmArgs &a, hipStream_t st, const char *what) {
 
 }  // namespace
 
-extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws,
-                             void *y, int32_t *acc_out, int M, int N, int K, int ldy,
-                             void *stream) {
-    CMI_REQUIRE(M >= 0 && N >= 1 && K >= 16, CMI_E_ARG, "cmi_gemm_w8a8: bad shape M=%d N=%d K=%d", M, N, K);
-    if (M == 0) return CMI_OK;  // an empty batch has no storage to point at
-    CMI_REQUIRE(xq && wq && xs && ws && y, CMI_E_ARG, "cmi_gemm_w8a8: null pointer");
-    CMI_REQUIRE(ldy >= N, CMI_E_ARG, "cmi_gemm_w8a8: ldy=%d is smaller than N=%d", ldy, N);
-    CMI_REQUIRE(K % 16 == 0, CMI_E_UNSUPPORTED, "cmi_gemm_w8a8: K=%d is not a multiple of 16", K);
-    CMI_REQUIRE(aligned(xq, 16) && aligned(wq, 16), CMI_E_ARG,
-                "cmi_gemm_w8a8: xq and wq must be 16-byte aligned");
+// Register-staged W8A8 kernel: any K that is a multiple of 16 (arguments already validated).
+int cmi::gemm_w8a8_generic(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws,
+                           void *y, int32_t *acc_out, int M, int N, int K, int ldy, void *stream) {
     GemmArgs a;
     a.xq = xq;
     a.w = wq;
