@@ -25,12 +25,19 @@
 // wavefronts (R = 2: 2 KiB x CHT in flight each, ~70 VGPRs), which is what keeps
 // HBM saturated from the first microsecond to the last: the hardware dispatcher
 // back-fills retiring wavefronts, so late memory service of one wavefront never
-// idles the rest.  A unit wider than the register budget of M rows is walked in
-// sub-trips with the next sub-trip's loads in flight.  When K spans several
-// units the wavefronts of a workgroup each take one unit of the same rows and
-// the unit totals meet in LDS (summed in unit order by one lane per output);
-// otherwise there is no LDS and no barrier: lane 63, which holds the tree
-// result, scales and stores.
+// idles the rest.  The activations are the same few cache lines for every
+// wavefront on the chip; fetched per wavefront they serialise on the L2
+// channels that own those lines, so a workgroup (4 wavefronts, 16 for 16 rows)
+// copies them into LDS once -- requested before the weights, because memory
+// returns data in issue order -- and every wavefront reads its fragments from
+// there, at most 8 activation rows in registers at a time (for 4 rows and more
+// in an order that makes the reads free of bank conflicts).  Batches whose
+// activations do not fit LDS are split into narrower calls.  A unit wider than
+// the register budget of M rows is walked in sub-trips with the next sub-trip's
+// weights in flight.  When K spans several units the wavefronts of a team each take units
+// of the same rows and the unit totals meet in LDS (summed in unit order by one
+// lane per output); otherwise lane 63, which holds the tree result, scales and
+// stores.
 #include "common.hpp"
 
 namespace {
@@ -50,8 +57,10 @@ struct GemvArgs {
     int unit;       // segments per unit (canonical, from K)
     int units;      // ceil(nseg / unit)
     int subtrips;   // ceil(unit / CHT)
+    uint32_t xvecs_rcp;  // ceil(2^32 / (K/8)): idx / (K/8) == umulhi(idx, xvecs_rcp) for idx < 2^16
     int nblocks;    // ceil(N / R)
-    int teams;      // row blocks per workgroup (units == 1: 4, else 1)
+    int uw;         // wavefronts of a team (they stride over the units)
+    int teams;      // row blocks per workgroup
 };
 
 // Segments per unit: the largest of 4,3,2,1 that pads K by at most a fifth.
@@ -77,6 +86,19 @@ __device__ __forceinline__ void widen4(uint32_t w, bf16x2_t &lo, bf16x2_t &hi) {
     hi = __builtin_bit_cast(bf16x2_t, p1);
 }
 
+// Wavefronts per workgroup (they share one LDS copy of the activations); wide
+// batches get smaller workgroups so that each wavefront may use more registers.
+constexpr int block_waves(int m) { return m >= 16 ? 16 : 4; }
+
+// Wavefronts per SIMD the register allocation must leave room for.
+constexpr int simd_waves(int m, int cht) { return m >= 16 || (m == 4 && cht == 1) ? 4 : 1; }
+
+// Activation rows held in registers at a time; wider batches loop over tiles of this many.
+constexpr int m_tile(int m) { return m < 8 ? m : 8; }
+
+// 16-byte vectors of activations each thread carries from global memory to LDS.
+constexpr int xstage_vectors(int m) { return m <= 1 ? 8 : m <= 2 ? 16 : m <= 4 ? 20 : 8; }
+
 template <int M, int CHT>
 struct XStage {
     uint4 x[M][CHT][2];
@@ -87,24 +109,26 @@ struct WStage {
     u32x4 w[R][CHT];
 };
 
-// MODE 0: K is one unit that fits one sub-trip (no loop, no LDS, no barrier).
+// MODE 0: K is one unit that fits one sub-trip (no loop, no unit exchange).
 // MODE 1: several units, each one sub-trip (all loads up front, totals via LDS).
 // MODE 2: general: units walked in pipelined sub-trips.
-template <int M, int R, int CHT, int MODE>
-__global__ void __launch_bounds__(256)
+// XLDS: the workgroup stages the activations in LDS; otherwise each wavefront
+//       reads them from global memory (only when they do not fit).
+template <int M, int R, int CHT, int MODE, bool XLDS>
+__global__ void __launch_bounds__(64 * block_waves(M), simd_waves(M, CHT))
 gemv_w8a16_kernel(const GemvArgs a) {
-    constexpr bool SINGLE = MODE == 0;
-    extern __shared__ float unit_total[];  // [units][R*M], only when units > 1
+    extern __shared__ uint4 smem[];  // [a.M][K] bf16 activations + 32 zero bytes (XLDS), then unit totals
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int nwaves = blockDim.x >> 6;
-    const int rb = SINGLE ? blockIdx.x * a.teams + wave : blockIdx.x;
-    const bool idle = rb >= a.nblocks;  // only in the last workgroup of a SINGLE launch
-    int u = SINGLE ? 0 : wave;          // unit in hand; wavefronts stride over the units
-    int seg_end = min((u + 1) * a.unit, a.nseg);
+    const int team = wave / a.uw;
+    const int rb = blockIdx.x * a.teams + team;
+    const bool idle = rb >= a.nblocks;  // only in the last workgroup
+    int u = wave - team * a.uw;         // unit in hand; the team's wavefronts stride over units
+    const int xvecs = a.K / 8;          // uint4 per activation row
+    float *unit_total = reinterpret_cast<float *>(smem + (XLDS ? a.M * xvecs + 2 : 0)) +
+                        team * a.units * (R * M);
 
     const u32x4 *wrow[R];
-    float scale[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         int n = rb * R + r;
@@ -115,29 +139,47 @@ gemv_w8a16_kernel(const GemvArgs a) {
     // Loads are unconditional: a dead chunk's address is clamped to the row's
     // last chunk and its activations are zeroed, so nothing branches between a
     // load and the arithmetic it overlaps.
-    auto load_w = [&](WStage<R, CHT> &s, int t) {
+    auto load_w = [&](WStage<R, CHT> &s, int unit_idx, int t) {
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
             for (int j = 0; j < CHT; ++j) {
-                const int chunk = (u * a.unit + t * CHT + j) * 64 + lane;
+                const int chunk = (unit_idx * a.unit + t * CHT + j) * 64 + lane;
                 s.w[r][j] = __builtin_nontemporal_load(wrow[r] + min(chunk, a.nchunks - 1));
             }
     };
-    auto load_x = [&](XStage<M, CHT> &s, int t) {
+    constexpr int MT = m_tile(M), MH = M / MT;
+    int xoff = 0;  // always 0; carries the ordering dependency described at its asm
+    auto load_x = [&](XStage<MT, CHT> &s, int unit_idx, int t, int mh) {
+        const int seg_end = min((unit_idx + 1) * a.unit, a.nseg);
 #pragma unroll
         for (int j = 0; j < CHT; ++j) {
-            const int seg = u * a.unit + t * CHT + j;
+            const int seg = unit_idx * a.unit + t * CHT + j;
             const int chunk = seg * 64 + lane;
             const bool live = seg < seg_end && chunk < a.nchunks;
             const int safe = min(chunk, a.nchunks - 1);
 #pragma unroll
-            for (int m = 0; m < M; ++m) {
-                const int mrow = m < a.M ? m : a.M - 1;
-                const uint4 *xp = reinterpret_cast<const uint4 *>(a.x + (size_t)mrow * a.K);
-                const uint4 lo = xp[2 * safe], hi = xp[2 * safe + 1];
-                s.x[m][j][0] = live ? lo : make_uint4(0, 0, 0, 0);
-                s.x[m][j][1] = live ? hi : make_uint4(0, 0, 0, 0);
+            for (int m = 0; m < MT; ++m) {
+                const int mrow = mh * MT + m < a.M ? mh * MT + m : a.M - 1;
+                if constexpr (XLDS) {
+                    // dead chunks read the zeroed slot behind the activations: a select
+                    // on the address, so the LDS reads stay unconditional
+                    if constexpr (M >= 4) {
+                        const int cseg = min(64, a.nchunks - seg * 64);  // chunks in this segment
+                        const int lo = mrow * xvecs + seg * 128 + lane + xoff;
+                        s.x[m][j][0] = smem[live ? lo : a.M * xvecs];
+                        s.x[m][j][1] = smem[live ? lo + cseg : a.M * xvecs];
+                    } else {
+                        const int at = live ? mrow * xvecs + 2 * chunk : a.M * xvecs;
+                        s.x[m][j][0] = smem[at];
+                        s.x[m][j][1] = smem[at + 1];
+                    }
+                } else {
+                    const uint4 *xp = reinterpret_cast<const uint4 *>(a.x + (size_t)mrow * a.K);
+                    const uint4 lo = xp[2 * safe], hi = xp[2 * safe + 1];
+                    s.x[m][j][0] = live ? lo : make_uint4(0, 0, 0, 0);
+                    s.x[m][j][1] = live ? hi : make_uint4(0, 0, 0, 0);
+                }
             }
         }
     };
@@ -148,7 +190,7 @@ gemv_w8a16_kernel(const GemvArgs a) {
 #pragma unroll
         for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
 
-    auto compute = [&](const WStage<R, CHT> &ws_, const XStage<M, CHT> &xs_) {
+    auto compute = [&](const WStage<R, CHT> &ws_, const XStage<MT, CHT> &xs_, int mh) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
 #pragma unroll
@@ -159,80 +201,130 @@ gemv_w8a16_kernel(const GemvArgs a) {
                 widen4(ws_.w[r][j].z, wb[4], wb[5]);
                 widen4(ws_.w[r][j].w, wb[6], wb[7]);
 #pragma unroll
-                for (int m = 0; m < M; ++m) {
+                for (int m = 0; m < MT; ++m) {
                     const uint32_t xv[8] = {xs_.x[m][j][0].x, xs_.x[m][j][0].y, xs_.x[m][j][0].z,
                                             xs_.x[m][j][0].w, xs_.x[m][j][1].x, xs_.x[m][j][1].y,
                                             xs_.x[m][j][1].z, xs_.x[m][j][1].w};
-                    float v = acc[r][m];
+                    float v = acc[r][mh * MT + m];
 #pragma unroll
                     for (int i = 0; i < 8; ++i)
                         v = __builtin_amdgcn_fdot2_f32_bf16(wb[i], __builtin_bit_cast(bf16x2_t, xv[i]),
                                                             v, false);
-                    acc[r][m] = v;
+                    acc[r][mh * MT + m] = v;
                 }
             }
         }
     };
 
-    for (; SINGLE || u < a.units; u += nwaves) {
-        if (idle) break;
-        seg_end = min((u + 1) * a.unit, a.nseg);
-        WStage<R, CHT> w0;
-        XStage<M, CHT> x0;
-        load_w(w0, 0);
-        load_x(x0, 0);
+    // Activation fetch first (memory returns data in issue order, so whatever a
+    // wavefront waits for must have been requested before the long weight
+    // stream), then all first-trip weights, then the LDS hand-over: the copy and
+    // its barrier run in the shadow of the weight latency.
+    constexpr int XV = xstage_vectors(M);
+    uint4 xstage[XV];
+    const int xtotal = a.M * xvecs;
+    if constexpr (XLDS) {
+        const uint4 *xg = reinterpret_cast<const uint4 *>(a.x);
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int n = rb * R + r;
-            scale[r] = a.ws[n < a.N ? n : a.N - 1];
+        for (int j = 0; j < XV; ++j) {
+            const int idx = threadIdx.x + j * blockDim.x;
+            xstage[j] = idx < xtotal ? xg[idx] : make_uint4(0, 0, 0, 0);
         }
+    }
+    WStage<R, CHT> w0;
+    load_w(w0, min(u, a.units - 1), 0);
+    float scale[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int n = rb * R + r;
+        scale[r] = a.ws[n < a.N ? n : a.N - 1];
+    }
+    if constexpr (XLDS) {
+#pragma unroll
+        for (int j = 0; j < XV; ++j) {
+            const int idx = threadIdx.x + j * blockDim.x;
+            // Within a segment (64 chunks of 16 weights) the first halves of all chunks
+            // come first, then the second halves: a wavefront's 16-byte reads are then
+            // contiguous across lanes (no bank conflicts).
+            if constexpr (M >= 4) {
+                const int row = __umulhi((uint32_t)idx, a.xvecs_rcp);
+                const int v = idx - row * xvecs;
+                const int seg = v >> 7, half = v & 1, c = (v & 127) >> 1;
+                const int cseg = min(64, a.nchunks - seg * 64);
+                if (idx < xtotal) smem[row * xvecs + seg * 128 + half * cseg + c] = xstage[j];
+            } else {
+                if (idx < xtotal) smem[idx] = xstage[j];  // little LDS traffic: plain order
+            }
+        }
+        if (threadIdx.x < 2) smem[xtotal + threadIdx.x] = make_uint4(0, 0, 0, 0);
+        __syncthreads();
+    }
+
+#pragma unroll 1
+    for (; u < a.units; u += a.uw) {
+        if (idle) break;
+        XStage<MT, CHT> x0;
+        auto consume = [&](const WStage<R, CHT> &w, int t) {
+#pragma unroll
+            for (int mh = 0; mh < MH; ++mh) {
+                // keep one activation tile in registers: no LDS reads of the next
+                // tile hoisted above this one's arithmetic (other wavefronts fill in)
+                load_x(x0, u, t, mh);
+                compute(w, x0, mh);
+                // Wide batches: the next tile's LDS address is made to depend on this
+                // tile's sums, so only one activation tile is ever live in registers
+                // (other wavefronts of the SIMD cover the LDS latency).
+                if constexpr (M >= 16) {
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        float *p = &acc[r][mh * MT];
+                        asm volatile("" : "+v"(p[0]), "+v"(p[1]), "+v"(p[2]), "+v"(p[3]), "+v"(p[4]),
+                                          "+v"(p[5]), "+v"(p[6]), "+v"(p[7]), "+v"(xoff));
+                    }
+                }
+            }
+        };
         if constexpr (MODE != 2) {
-            compute(w0, x0);
+            consume(w0, 0);
         } else {
+            // sub-trips of the unit, next weights in flight while these are consumed
             WStage<R, CHT> w1;
-            XStage<M, CHT> x1;
-            // sub-trips of the unit, next one in flight while this one is consumed
             int t = 0;
+#pragma unroll 1
             for (; t + 2 < a.subtrips; t += 2) {
-                load_w(w1, t + 1);
-                load_x(x1, t + 1);
-                compute(w0, x0);
-                load_w(w0, t + 2);
-                load_x(x0, t + 2);
-                compute(w1, x1);
+                load_w(w1, u, t + 1);
+                consume(w0, t);
+                load_w(w0, u, t + 2);
+                consume(w1, t + 1);
             }
             if (t + 1 < a.subtrips) {
-                load_w(w1, t + 1);
-                load_x(x1, t + 1);
-                compute(w0, x0);
-                compute(w1, x1);
+                load_w(w1, u, t + 1);
+                consume(w0, t);
+                consume(w1, t + 1);
             } else {
-                compute(w0, x0);
+                consume(w0, t);
             }
         }
+        if (MODE != 0 && u + a.uw < a.units) load_w(w0, u + a.uw, 0);  // next unit of this wavefront
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
             for (int m = 0; m < M; ++m) acc[r][m] = wave_sum_to_lane63(acc[r][m]);
-        if constexpr (SINGLE) break;
-        if (a.units > 1) {
-            // unit totals meet in LDS; one lane per output adds them in unit order below
-            if (lane == 63) {
-#pragma unroll
-                for (int r = 0; r < R; ++r)
-#pragma unroll
-                    for (int m = 0; m < M; ++m) unit_total[u * (R * M) + r * M + m] = acc[r][m];
-            }
+        if constexpr (MODE == 0) break;
+        // unit totals meet in LDS; one lane per output adds them in unit order below
+        if (lane == 63) {
 #pragma unroll
             for (int r = 0; r < R; ++r)
 #pragma unroll
-                for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
-        } else {
-            break;
+                for (int m = 0; m < M; ++m) unit_total[u * (R * M) + r * M + m] = acc[r][m];
         }
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
     }
 
-    if (SINGLE || a.units == 1) {
+    if constexpr (MODE == 0) {
         if (!idle && lane == 63) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
@@ -245,28 +337,28 @@ gemv_w8a16_kernel(const GemvArgs a) {
                 }
             }
         }
-        return;
-    }
-
-    __syncthreads();
-    if (wave == 0 && lane < R * M) {
-        const int r = lane / M, m = lane - r * M;
-        const int n = rb * R + r;
-        if (n < a.N && m < a.M) {
-            float total = unit_total[lane];
-            for (int v = 1; v < a.units; ++v) total += unit_total[v * (R * M) + lane];
-            a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(a.ws[n] * total);
+    } else {
+        __syncthreads();
+        if (!idle && wave == team * a.uw && lane < R * M) {
+            const int r = lane / M, m = lane - r * M;
+            const int n = rb * R + r;
+            if (n < a.N && m < a.M) {
+                float total = unit_total[lane];
+                for (int v = 1; v < a.units; ++v) total += unit_total[v * (R * M) + lane];
+                a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(a.ws[n] * total);
+            }
         }
     }
 }
 
 struct Plan {
-    int mt, r, cht;
-    bool single;
+    int mt, r, cht, mode;
 };
 
 //: Most K-units one launch handles (LDS holds one total per unit and output).
-constexpr int MAX_UNITS = 256;
+constexpr int MAX_UNITS = 64;
+//: Activations up to this many bytes are staged in LDS.
+constexpr size_t XLDS_MAX_BYTES = 96 * 1024;
 
 // Blocking is a pure function of (M, N, K); it never changes results.
 Plan make_plan(int M, int N, int K) {
@@ -275,36 +367,65 @@ Plan make_plan(int M, int N, int K) {
     const int nseg = (K / 16 + 63) / 64;
     const int unit = unit_segments(nseg);
     const int units = (nseg + unit - 1) / unit;
-    const int chmax = p.mt <= 2 ? 4 : p.mt <= 4 ? 3 : 1;
+    // Registers allow 4 chunks per trip for 1-2 rows, 3 for 4 rows (and that only pays
+    // when the whole K fits one trip), 1 beyond.
+    const int chmax = p.mt <= 2 ? 4 : (p.mt <= 4 && units == 1 && unit <= 3) ? 3 : 1;
     p.cht = unit < chmax ? unit : chmax;
     // balance the sub-trips of a unit (e.g. 4 segments at CHT<=3 -> 2 + 2)
     const int subtrips = (unit + p.cht - 1) / p.cht;
     p.cht = (unit + subtrips - 1) / subtrips;
-    p.single = nseg <= p.cht;
-    // Two rows per wavefront; one when that would leave fewer than ~8 wavefronts per CU.
-    p.r = p.mt >= 16 ? 1 : 2;
-    if ((long)((N + 1) / 2) * units < 2048) p.r = 1;
+    p.mode = subtrips > 1 ? 2 : units > 1 ? 1 : 0;
+    p.r = 2;
+    (void)N;
     return p;
 }
 
-template <int M, int R, int CHT, int MODE>
+template <int M, int R, int CHT, int MODE, bool XLDS>
 int launch(GemvArgs &a, hipStream_t st) {
-    constexpr bool SINGLE = MODE == 0;
     a.nblocks = (a.N + R - 1) / R;
     a.subtrips = (a.unit + CHT - 1) / CHT;
-    a.teams = SINGLE ? 4 : 1;
-    const dim3 grid(SINGLE ? (a.nblocks + 3) / 4 : a.nblocks);
-    const dim3 block(SINGLE ? 256 : 64 * (a.units < 4 ? a.units : 4));
-    const size_t lds = (SINGLE || a.units == 1) ? 0 : sizeof(float) * a.units * R * M;
-    gemv_w8a16_kernel<M, R, CHT, MODE><<<grid, block, lds, st>>>(a);
+    a.xvecs_rcp = (uint32_t)(((1ull << 32) + (a.K / 8) - 1) / (a.K / 8));
+    a.uw = a.units < 4 ? a.units : 4;
+    a.teams = block_waves(M) / a.uw;
+    const dim3 grid((a.nblocks + a.teams - 1) / a.teams);
+    const dim3 block(64 * a.uw * a.teams);
+    const size_t lds = (XLDS ? (size_t)a.M * a.K * 2 + 32 : 0) +
+                       (MODE == 0 ? 0 : sizeof(float) * a.teams * a.units * R * M);
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_w8a16_kernel<M, R, CHT, MODE, XLDS>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024) != hipSuccess)
+            return fail(CMI_E_HIP, "cmi_gemv_w8a16: cannot reserve LDS");
+        configured = true;
+    }
+    gemv_w8a16_kernel<M, R, CHT, MODE, XLDS><<<grid, block, lds, st>>>(a);
     return check_launch("cmi_gemv_w8a16");
+}
+
+// Whether a workgroup of the M-tile's kernel can carry [rows, K] activations into LDS.
+bool x_fits_lds(int mt, int rows, int K, int units) {
+    const size_t xbytes = (size_t)rows * K * 2;
+    const int uw = units < 4 ? units : 4;
+    const int bw = mt >= 16 ? block_waves(16) : block_waves(1);
+    const int xv = mt <= 1 ? xstage_vectors(1) : mt <= 2 ? xstage_vectors(2) : mt <= 4 ? xstage_vectors(4)
+                                                                             : xstage_vectors(8);
+    const size_t threads = 64 * (size_t)uw * (bw / uw);  // as launch() sizes the workgroup
+    return xbytes <= XLDS_MAX_BYTES && xbytes <= 16 * (size_t)xv * threads;
+}
+
+template <int M, int R, int CHT, int MODE>
+int dispatch_lds(GemvArgs &a, hipStream_t st) {
+    if (x_fits_lds(M, a.M, a.K, a.units)) return launch<M, R, CHT, MODE, true>(a, st);
+    return launch<M, R, CHT, MODE, false>(a, st);
 }
 
 template <int M, int R, int CHT>
 int dispatch_x(GemvArgs &a, const Plan &p, hipStream_t st) {
-    if (p.single) return launch<M, R, CHT, 0>(a, st);
-    if ((a.unit + CHT - 1) / CHT == 1) return launch<M, R, CHT, 1>(a, st);
-    return launch<M, R, CHT, 2>(a, st);
+    if (p.mode == 0) return dispatch_lds<M, R, CHT, 0>(a, st);
+    if (p.mode == 1) return dispatch_lds<M, R, CHT, 1>(a, st);
+    // sub-trips only arise where a unit exceeds the register budget of the M tile
+    if constexpr (M >= 4 && CHT == 1) return dispatch_lds<M, R, CHT, 2>(a, st);
+    return fail(CMI_E_UNSUPPORTED, "cmi_gemv_w8a16: no sub-trip kernel for M-tile %d, %d chunks", M, CHT);
 }
 
 template <int M, int R>
@@ -351,6 +472,14 @@ extern "C" int cmi_gemv_w8a16(const int8_t *wq, const float *ws, const void *x, 
     a.units = (a.nseg + a.unit - 1) / a.unit;
     CMI_REQUIRE(a.units <= MAX_UNITS, CMI_E_UNSUPPORTED, "cmi_gemv_w8a16: K=%d above %d", K,
                 MAX_UNITS * 4096);
+    // Activations too large for LDS: narrower batches fit more often, and rows are
+    // independent (same bits whatever the batch), so halve the batch instead.
+    if (M > 1 && !x_fits_lds(p.mt, M, K, a.units)) {
+        const int half = p.mt / 2;
+        const int rc = cmi_gemv_w8a16(wq, ws, x, y, half, N, K, stream);
+        if (rc != CMI_OK) return rc;
+        return cmi_gemv_w8a16(wq, ws, a.x + (size_t)half * K, a.y + (size_t)half * N, M - half, N, K, stream);
+    }
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (p.mt) {
         case 1: return dispatch_r<1>(a, p, st);
