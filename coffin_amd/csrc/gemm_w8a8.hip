@@ -1,43 +1,46 @@
-// W8A8 prefill GEMM, software-pipelined for CDNA4 int8 MFMA (K a multiple of 128).
+// W8A8 prefill GEMM for CDNA4 int8 MFMA (K a multiple of 128).
 //
 //   acc[m,n] = sum_k xq[m,k] * wq[n,k]           int32, exact
 //   y[m,n]   = bf16((float)acc * xs[m] * ws[n])   left to right, one narrowing
 //
-// v_mfma_i32_32x32x32_i8 (one wavefront per SIMD already sustains ~90 % of the
-// int8 peak with it; the 16x16x64 form needs two) with the weight on the MFMA
-// rows and the activation on the MFMA columns, both K-contiguous in memory
-// (16 consecutive k per lane), so a lane ends with groups of four consecutive n
-// of one m.
+// v_mfma_i32_32x32x32_i8 with the weight on the MFMA rows and the activation on
+// the MFMA columns, both K-contiguous in memory (16 consecutive k per lane), so
+// a lane ends with groups of four consecutive n of one m.
 //
-// Workgroup = 4 wavefronts (2 x 2), block tile 128(m) x 128(n), wavefront tile
-// 64 x 64 = 2 x 2 MFMA tiles held in registers for the whole K loop.  K is walked
-// in steps of 128 (one whole cache line per row: with 64-byte steps every line
-// was fetched from L2 twice, the L1 being too small to keep it for a step)
-// through two LDS stages filled by direct global -> LDS loads
-// (global_load_lds_dwordx4: no staging registers); the register copy of the
-// current fragments acts as the third stage.  Two workgroups share a CU.  A direct load lays the 64 lanes' 16-byte chunks out
+// Common to both kernels below: K is walked in steps of 128 (one whole cache
+// line per row and request: with 64-byte steps every line is fetched from L2
+// twice); operand tiles go global -> LDS directly (global_load_lds_dwordx4, no
+// staging registers).  A direct load lays the 64 lanes' 16-byte chunks out
 // contiguously, so the bank-conflict-free arrangement is made on the global
 // side: lane i of a load fetches the chunk that belongs at LDS slot i, with the
-// chunk index XOR-swizzled by (row / 2) % 8.  Sixteen consecutive lanes of a
-// fragment read (16 rows, one k chunk) then touch 16 distinct 16-byte slots of
-// the 256-byte bank row.  Fragments for step s+1 are read from LDS while the 8
-// MFMAs of step s issue.  The epilogue goes through LDS once more so that every
-// lane stores 16 contiguous bytes of y.
-// One s_barrier per step, with explicit vmcnt/lgkmcnt waits (a __syncthreads
-// would drain the whole prefetch ring).  Workgroup ids are remapped so each of
-// the 8 XCDs (private L2) owns a contiguous band of n tiles.
+// chunk index XOR-swizzled by (row / 2) % 8.  Waits are explicit vmcnt/lgkmcnt
+// counts with one s_barrier per step (a __syncthreads would drain the prefetch),
+// and the interleaving of MFMAs, LDS reads and global loads inside a step is
+// spelled out with scheduling group barriers: left alone, the compiler puts the
+// wait for the *next* fragments in front of the current MFMAs.  The epilogue goes
+// through LDS once more so that every lane stores 16 contiguous bytes of y.
+// Workgroup ids are remapped so each of the 8 XCDs (private L2) owns a
+// contiguous band of n tiles.
+//
+//   gemm_w8a8_pipe_kernel: 128 x 128 block tile, 4 wavefronts of 64 x 64, two
+//     LDS stages, whole-step fragment double buffering in registers, two
+//     workgroups per CU (one's prologue/epilogue hides under the other's MFMAs).
+//   gemm_w8a8_big_kernel: 256 x 256 block tile, 8 wavefronts of 128 x 64, a ring
+//     of five single-operand LDS slots.  Half the L2 -> LDS bytes per MFMA.
+//
+// The launcher picks by how well the tile count fills the 256 CUs.
 #include "common.hpp"
+
+#include <cmath>
+#include <cstdlib>
+#include <type_traits>
 
 namespace {
 
 using namespace cmi;
 
-constexpr int BM = 128, BN = 128, BK = 128;   // BK = one 128-byte cache line per row and step
-constexpr int STAGES = 2;
-constexpr int THREADS = 256;
-constexpr int TILE_BYTES = 128 * BK;            // one operand, one stage: 16 KiB
-constexpr int STAGE_BYTES = 2 * TILE_BYTES;     // W tile then X tile
-constexpr int LDS_BYTES = STAGES * STAGE_BYTES; // 64 KiB: two workgroups per CU
+constexpr int BK = 128;        // one 128-byte cache line per row and step
+constexpr int THREADS = 256;   // 2 x 2 wavefronts
 
 struct Args {
     const int8_t *xq;
@@ -52,127 +55,63 @@ struct Args {
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
 
-__global__ void __launch_bounds__(THREADS)
-gemm_w8a8_pipe_kernel(const Args a) {
-    extern __shared__ __align__(16) int8_t lds[];
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int wn = wave & 1, wm = wave >> 1;
+// TN, TM: 32 x 32 MFMA tiles per wavefront along n (weight rows) and m
+// (activation rows); block tile = (64*TM) x (64*TN).  NST: LDS stages.
+template <int TN, int TM, int NST>
+struct Cfg {
+    static constexpr int BN = 64 * TN, BM = 64 * TM;
+    static constexpr int W_BYTES = BN * BK, X_BYTES = BM * BK;
+    static constexpr int STAGE_BYTES = W_BYTES + X_BYTES;
+    static constexpr int LDS_BYTES = NST * STAGE_BYTES;
+    static constexpr int WL = BN / 32, XL = BM / 32;  // loads per wavefront and stage (8 rows each)
+    static constexpr int LPW = WL + XL;
+    static constexpr int PITCH = 64 * TN + 16;        // epilogue: one m row of the wavefront tile + 16 B
+    static_assert(4 * 32 * TM * PITCH <= LDS_BYTES, "epilogue does not fit the operand stages");
+    static_assert((NST - 2) * LPW <= 63, "vmcnt range");
+};
 
-    // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs; XCD x
-    // gets logical tiles [x*per, (x+1)*per), m fastest inside a band of n tiles.
-    const int total = a.tiles_m * a.tiles_n;
-    int tile = blockIdx.x;
-    if (total % 8 == 0) tile = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
-    const int tn = tile / a.tiles_m, tm = tile - tn * a.tiles_m;
-    const int m0 = tm * BM, n0 = tn * BN;
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    if constexpr (N == 0) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    else if constexpr (N == 4) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+    else if constexpr (N == 6) asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
+    else if constexpr (N == 8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+    else if constexpr (N == 12) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");
+    else if constexpr (N == 16) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
+    else if constexpr (N == 18) asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)" ::: "memory");
+    else if constexpr (N == 24) asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)" ::: "memory");
+    else if constexpr (N == 32) asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)" ::: "memory");
+    else if constexpr (N == 36) asm volatile("s_waitcnt vmcnt(36) lgkmcnt(0)" ::: "memory");
+    else static_assert(N < 0, "add the vmcnt literal");
+}
 
-    // Global side of the direct loads.  One load instruction moves 8 rows x 128 B
-    // (whole cache lines) into 1 KiB of LDS; a wavefront fills row groups
-    // 4*wave .. 4*wave+3 of both tiles.  Lane i lands in slot i of the group:
-    // row = i/8, stored chunk = i%8, which holds k chunk (i%8) ^ ((row/2) % 8).
-    const int lrow = lane >> 3;
-    const int8_t *wsrc[4], *xsrc[4];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-        const int row = (4 * wave + g) * 8 + lrow;
-        const int kc = (lane & 7) ^ ((row >> 1) & 7);
-        const int nrow = min(n0 + row, a.N - 1), mrow = min(m0 + row, a.M - 1);
-        wsrc[g] = a.wq + (size_t)nrow * a.K + kc * 16;
-        xsrc[g] = a.xq + (size_t)mrow * a.K + kc * 16;
-    }
-    auto issue = [&](int stage, int ks) {
-        int8_t *base = lds + stage * STAGE_BYTES + (4 * wave) * 1024;
-        const int k = ks * BK;
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            __builtin_amdgcn_global_load_lds((const void *)(wsrc[g] + k),
-                                             (lds_ptr_t)(base + g * 1024), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((const void *)(xsrc[g] + k),
-                                             (lds_ptr_t)(base + TILE_BYTES + g * 1024), 16, 0, 0);
-        }
-    };
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
 
-    // LDS side: lane reads row (lane%32) of a 32-row MFMA tile; for k quarter q
-    // (32 k each) its 16 bytes are k chunk 2q + lane/32.
-    const int frow = lane & 31;
-    const int fsw = (frow >> 1) & 7;
-    int foff[4];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) foff[q] = frow * BK + ((2 * q + (lane >> 5)) ^ fsw) * 16;
-    // frag[t][q]: MFMA tile t (0..1), k quarter q (0..3)
-    auto read_frags = [&](int stage, v4i32 (&wf)[2][4], v4i32 (&xf)[2][4]) {
-        const int8_t *wt = lds + stage * STAGE_BYTES + wn * 64 * BK;
-        const int8_t *xt = lds + stage * STAGE_BYTES + TILE_BYTES + wm * 64 * BK;
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                wf[t][q] = *reinterpret_cast<const v4i32 *>(wt + t * 32 * BK + foff[q]);
-                xf[t][q] = *reinterpret_cast<const v4i32 *>(xt + t * 32 * BK + foff[q]);
-            }
-    };
+// Two fp32 -> packed bf16, round to nearest even (v_cvt_pk_bf16_f32).
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2v));
+}
 
-    v16i32 acc[2][2];  // [n tile][m tile]
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
-    auto mma = [&](const v4i32 (&wf)[2][4], const v4i32 (&xf)[2][4]) {
-#pragma unroll
-        for (int h = 0; h < 4; ++h)
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[i][h], xf[j][h], acc[i][j], 0, 0, 0);
-    };
-
-    const int ksteps = a.K / BK;
-    // One pipeline step.  Stage ks%2 was emptied into registers during step ks-1,
-    // so once every wavefront is past the barrier it takes the loads of step ks+2;
-    // stage (ks+1)%2 has landed (it was requested a whole step ago) and its
-    // fragments are read while the 16 MFMAs of step ks issue.
-    auto step = [&](int ks, const v4i32 (&cw)[2][4], const v4i32 (&cx)[2][4], v4i32 (&nw)[2][4],
-                    v4i32 (&nx)[2][4]) {
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        if (ks + 2 < ksteps) issue(ks % STAGES, ks + 2);
-        if (ks + 1 < ksteps) read_frags((ks + 1) % STAGES, nw, nx);
-        mma(cw, cx);
-    };
-
-    issue(0, 0);
-    if (ksteps > 1) issue(1, 1);
-    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");   // stage 0 (8 loads per stage and wavefront)
-    if (ksteps == 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    v4i32 w0[2][4], x0[2][4], w1[2][4], x1[2][4];
-    read_frags(0, w0, x0);
-    int ks = 0;
-    for (; ks + 1 < ksteps; ks += 2) {
-        step(ks, w0, x0, w1, x1);
-        step(ks + 1, w1, x1, w0, x0);
-    }
-    if (ks < ksteps) step(ks, w0, x0, w1, x1);
-
-    // Epilogue.  Accumulator element v of tile (i, j) in lane l is
-    //   n = nb + 32*i + 8*(v/4) + 4*(l/32) + v%4,   m = mb + 32*j + l%32.
-    // Scale, narrow, park the wavefront's 64 x 64 bf16 tile in LDS (row = m,
-    // 144-byte pitch), then write rows back 16 bytes per lane.
+// Epilogue of one wavefront tile of TN x TM MFMA tiles whose corner is (nb, mb).
+// Accumulator element v of tile (i, j) in lane l is
+//   n = nb + 32*i + 8*(v/4) + 4*(l/32) + v%4,   m = mb + 32*j + l%32.
+// Scale, narrow, park the wavefront's bf16 tile in LDS (row = m), then write
+// rows back 16 bytes per lane.  Every wavefront of the workgroup must call it
+// (one barrier inside: the operand stages are reused as parking space).
+template <int TN, int TM>
+__device__ __forceinline__ void epilogue(const Args &a, v16i32 (&acc)[TN][TM], int8_t *lds, int wave,
+                                         int lane, int nb, int mb) {
     if (a.acc_out) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < TN; ++i)
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const int m = m0 + wm * 64 + j * 32 + (lane & 31);
+            for (int j = 0; j < TM; ++j) {
+                const int m = mb + j * 32 + (lane & 31);
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const int n = n0 + wn * 64 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                    const int n = nb + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
                     if (m < a.M && n < a.N) a.acc_out[(size_t)m * a.N + n] = acc[i][j][v];
                 }
             }
@@ -180,42 +119,51 @@ gemm_w8a8_pipe_kernel(const Args a) {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();  // every wavefront is done reading operand stages
     asm volatile("" ::: "memory");
-    constexpr int PITCH = 144;     // 64 bf16 + 16 B: 8 rows -> 8 distinct 16-byte bank groups
-    int8_t *park = lds + wave * (64 * PITCH);
+    constexpr int PITCH = 64 * TN + 16;  // one m row of the wavefront tile + 16 B
+    int8_t *park = lds + wave * (32 * TM * PITCH);
+    // per-column scales of this lane's columns: 4 consecutive n per (i, q)
+    float wsv[TN][4][4];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int n = nb + i * 32 + 8 * q + 4 * (lane >> 5);
+            if (n + 3 < a.N) {
+                const float4 sc = *reinterpret_cast<const float4 *>(a.ws + n);
+                wsv[i][q][0] = sc.x, wsv[i][q][1] = sc.y, wsv[i][q][2] = sc.z, wsv[i][q][3] = sc.w;
+            } else {
+                // ragged edge: clamped reads; those columns are never stored
+#pragma unroll
+                for (int r = 0; r < 4; ++r) wsv[i][q][r] = a.ws[min(n + r, a.N - 1)];
+            }
+        }
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
         const int ml = j * 32 + (lane & 31);
-        const int m = m0 + wm * 64 + ml;
-        const float xm = a.xs[min(m, a.M - 1)];
+        const float xm = a.xs[min(mb + ml, a.M - 1)];
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < TN; ++i)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int nl = i * 32 + 8 * q + 4 * (lane >> 5);
-                const int n = n0 + wn * 64 + nl;
-                const float4 sc = *reinterpret_cast<const float4 *>(a.ws + min(n, a.N - 4));
-                const float scv[4] = {sc.x, sc.y, sc.z, sc.w};
-                uint32_t o[4];
+                float t[4];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    // ws index is clamped for the ragged edge; those columns are never stored
-                    const float wsn = n + 3 < a.N ? scv[r] : a.ws[min(n + r, a.N - 1)];
-                    const float t = (float)acc[i][j][4 * q + r] * xm;
-                    o[r] = f32_to_bf16_bits(t * wsn);
-                }
+                for (int r = 0; r < 4; ++r) t[r] = ((float)acc[i][j][4 * q + r] * xm) * wsv[i][q][r];
                 uint2 pk;
-                pk.x = o[0] | (o[1] << 16);
-                pk.y = o[2] | (o[3] << 16);
+                pk.x = pack_bf16(t[0], t[1]);
+                pk.y = pack_bf16(t[2], t[3]);
                 *reinterpret_cast<uint2 *>(park + ml * PITCH + nl * 2) = pk;
             }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own tile only: no barrier needed
     const bool vec_ok = (a.ldy % 8 == 0) && ((reinterpret_cast<uintptr_t>(a.y) & 15) == 0);
+    constexpr int CPR = 4 * TN;        // 16-byte chunks per row of the wavefront tile
+    constexpr int RPP = 64 / CPR;      // rows per pass
 #pragma unroll
-    for (int p = 0; p < 8; ++p) {
-        const int ml = p * 8 + (lane >> 3), c = lane & 7;  // 8 lanes x 16 B = one 64-wide row
-        const int m = m0 + wm * 64 + ml;
-        const int n = n0 + wn * 64 + c * 8;
+    for (int p = 0; p < 32 * TM / RPP; ++p) {
+        const int ml = p * RPP + lane / CPR, c = lane % CPR;
+        const int m = mb + ml;
+        const int n = nb + c * 8;
         if (m >= a.M || n >= a.N) continue;
         const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * PITCH + c * 16);
         uint16_t *dst = a.y + (size_t)m * a.ldy + n;
@@ -228,6 +176,354 @@ gemm_w8a8_pipe_kernel(const Args a) {
                 if (n + r < a.N) dst[r] = (uint16_t)(w[r >> 1] >> ((r & 1) * 16));
         }
     }
+}
+
+template <int TN, int TM, int NST>
+__global__ void __launch_bounds__(THREADS)
+gemm_w8a8_pipe_kernel(const Args a) {
+    using C = Cfg<TN, TM, NST>;
+    extern __shared__ __align__(16) int8_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: keeps LDS bases scalar
+    const int wn = wave & 1, wm = wave >> 1;
+
+    // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs; XCD x
+    // gets logical tiles [x*per, (x+1)*per), m fastest inside a band of n tiles.
+    const int total = a.tiles_m * a.tiles_n;
+    int tile = blockIdx.x;
+    if (total % 8 == 0) tile = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
+    const int tn = tile / a.tiles_m, tm = tile - tn * a.tiles_m;
+    const int m0 = tm * C::BM, n0 = tn * C::BN;
+
+    // Global side of the direct loads.  One load instruction moves 8 rows x 128 B
+    // (whole cache lines) into 1 KiB of LDS; each wavefront fills a contiguous run
+    // of rows (consecutive loads on consecutive rows measured 30 % faster than
+    // wavefronts interleaved row group by row group).  Lane i lands in slot i of the group: row = i/8, stored chunk
+    // = i%8, which holds k chunk (i%8) ^ ((row/2) % 8).
+    const int lrow = lane >> 3;
+    const int8_t *wsrc[C::WL], *xsrc[C::XL];
+#pragma unroll
+    for (int g = 0; g < C::WL; ++g) {
+        const int row = (C::WL * wave + g) * 8 + lrow;
+        const int kc = (lane & 7) ^ ((row >> 1) & 7);
+        wsrc[g] = a.wq + (size_t)min(n0 + row, a.N - 1) * a.K + kc * 16;
+    }
+#pragma unroll
+    for (int g = 0; g < C::XL; ++g) {
+        const int row = (C::XL * wave + g) * 8 + lrow;
+        const int kc = (lane & 7) ^ ((row >> 1) & 7);
+        xsrc[g] = a.xq + (size_t)min(m0 + row, a.M - 1) * a.K + kc * 16;
+    }
+    auto issue = [&](int stage, int ks) {
+        int8_t *base = lds + stage * C::STAGE_BYTES;
+        const int k = ks * BK;
+#pragma unroll
+        for (int g = 0; g < C::WL; ++g)
+            __builtin_amdgcn_global_load_lds((const void *)(wsrc[g] + k), (lds_ptr_t)(base + (C::WL * wave + g) * 1024), 16, 0, 0);
+#pragma unroll
+        for (int g = 0; g < C::XL; ++g)
+            __builtin_amdgcn_global_load_lds((const void *)(xsrc[g] + k),
+                                             (lds_ptr_t)(base + C::W_BYTES + (C::XL * wave + g) * 1024), 16, 0, 0);
+    };
+
+    // LDS side: lane reads row (lane%32) of a 32-row MFMA tile; for k quarter q
+    // (32 k each) its 16 bytes are k chunk 2q + lane/32.
+    const int frow = lane & 31;
+    const int fsw = (frow >> 1) & 7;
+    int foff[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) foff[q] = frow * BK + ((2 * q + (lane >> 5)) ^ fsw) * 16;
+    auto read_frags = [&](int stage, v4i32 (&wf)[TN][4], v4i32 (&xf)[TM][4]) {
+        const int8_t *wt = lds + stage * C::STAGE_BYTES + wn * 32 * TN * BK;
+        const int8_t *xt = lds + stage * C::STAGE_BYTES + C::W_BYTES + wm * 32 * TM * BK;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+#pragma unroll
+            for (int t = 0; t < TN; ++t) wf[t][q] = *reinterpret_cast<const v4i32 *>(wt + t * 32 * BK + foff[q]);
+#pragma unroll
+            for (int t = 0; t < TM; ++t) xf[t][q] = *reinterpret_cast<const v4i32 *>(xt + t * 32 * BK + foff[q]);
+        }
+    };
+
+    v16i32 acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+    auto mma = [&](const v4i32 (&wf)[TN][4], const v4i32 (&xf)[TM][4]) {
+#pragma unroll
+        for (int h = 0; h < 4; ++h)
+#pragma unroll
+            for (int i = 0; i < TN; ++i)
+#pragma unroll
+                for (int j = 0; j < TM; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[i][h], xf[j][h], acc[i][j], 0, 0, 0);
+    };
+
+    const int ksteps = a.K / BK;
+    // One pipeline step.  The fragments of step ks are in registers.  Stage
+    // (ks+1)%NST must have landed: of the loads this wavefront issued after it,
+    // NST-2 stages' worth may still be in flight while new loads are being issued
+    // (ISSUE), none after that.  After the barrier every wavefront has emptied
+    // stage ks%NST into registers, so it takes the loads of step ks+NST.  The
+    // fragments of step ks+1 are read while the MFMAs of step ks run: the step is
+    // one basic block and the group barriers below spell out the interleaving
+    // (MFMA first: the compiler's own wait for the current fragments must not
+    // cover the new LDS reads).  Past the last step the read fetches a stale stage
+    // that nobody uses.
+    auto step = [&](auto issue_tag, int ks, const v4i32 (&cw)[TN][4], const v4i32 (&cx)[TM][4],
+                    v4i32 (&nw)[TN][4], v4i32 (&nx)[TM][4]) {
+        constexpr bool ISSUE = decltype(issue_tag)::value;
+        if constexpr (ISSUE) wait_vmcnt<(NST - 2) * C::LPW>();
+        else wait_vmcnt<0>();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if constexpr (ISSUE) issue(ks % NST, ks + NST);
+        read_frags((ks + 1) % NST, nw, nx);
+        mma(cw, cx);
+        // The global -> LDS loads come first in program order (the compiler keeps LDS
+        // writes and LDS reads in order), two per MFMA; the fragment reads follow,
+        // spread over the remaining MFMAs but the last.
+        constexpr int N_MMA = 4 * TN * TM, N_DS = 4 * (TN + TM), N_VM = ISSUE ? C::LPW : 0;
+        constexpr int VM_SLOTS = (N_VM + 1) / 2;
+        constexpr int DS_PER = (N_DS + (N_MMA - VM_SLOTS - 1) - 1) / (N_MMA - VM_SLOTS - 1);
+#pragma unroll
+        for (int i = 0; i < N_MMA; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                         // one MFMA
+            if (i < VM_SLOTS) __builtin_amdgcn_sched_group_barrier(0x010, 2, 0);       // global -> LDS loads
+            else if ((i - VM_SLOTS) * DS_PER < N_DS)
+                __builtin_amdgcn_sched_group_barrier(0x100, DS_PER, 0);                // LDS reads
+        }
+    };
+    using issue_t = std::integral_constant<bool, true>;
+    using drain_t = std::integral_constant<bool, false>;
+
+    for (int s = 0; s < NST; ++s)
+        if (s < ksteps) issue(s, s);
+    if (ksteps >= NST) wait_vmcnt<(NST - 1) * C::LPW>();
+    else wait_vmcnt<0>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    v4i32 w0[TN][4], x0[TM][4], w1[TN][4], x1[TM][4];
+    read_frags(0, w0, x0);
+    const int n_issue = ksteps > NST ? ksteps - NST : 0;  // steps that still request a stage
+    int ks = 0;
+    for (; ks + 1 < n_issue; ks += 2) {
+        step(issue_t{}, ks, w0, x0, w1, x1);
+        step(issue_t{}, ks + 1, w1, x1, w0, x0);
+    }
+    if (ks < n_issue) {
+        step(issue_t{}, ks, w0, x0, w1, x1);
+        step(drain_t{}, ks + 1, w1, x1, w0, x0);
+        ks += 2;
+    }
+    for (; ks + 1 < ksteps; ks += 2) {
+        step(drain_t{}, ks, w0, x0, w1, x1);
+        step(drain_t{}, ks + 1, w1, x1, w0, x0);
+    }
+    if (ks < ksteps) step(drain_t{}, ks, w0, x0, w1, x1);
+
+    epilogue<TN, TM>(a, acc, lds, wave, lane, n0 + wn * 32 * TN, m0 + wm * 32 * TM);
+}
+
+template <int TN, int TM, int NST>
+int launch(Args &a, hipStream_t st) {
+    using C = Cfg<TN, TM, NST>;
+    a.tiles_m = (a.M + C::BM - 1) / C::BM;
+    a.tiles_n = (a.N + C::BN - 1) / C::BN;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w8a8_pipe_kernel<TN, TM, NST>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES) != hipSuccess)
+            return fail(CMI_E_HIP, "cmi_gemm_w8a8: cannot reserve %d bytes of LDS", C::LDS_BYTES);
+        configured = true;
+    }
+    gemm_w8a8_pipe_kernel<TN, TM, NST><<<dim3(a.tiles_m * a.tiles_n), dim3(THREADS), C::LDS_BYTES, st>>>(a);
+    return check_launch("cmi_gemm_w8a8");
+}
+
+// ---------------------------------------------------------------------------
+// 256 x 256 block tile, 8 wavefronts (2 along n x 4 along m, two per SIMD), each
+// 128(n) x 64(m) = 4 x 2 MFMA tiles.  The operand bytes a CU must pull from L2
+// per MFMA cycle halve against the 128 x 128 tile, which is what bounds that
+// kernel.  LDS is a ring of five 32 KiB slots; the ring units alternate W tile,
+// X tile of successive k steps (unit 2s = W of step s, unit 2s+1 = X of step s),
+// so that beside the two units being computed from, up to three are in flight or
+// landed -- with whole two-operand stages only two would fit and the memory
+// pipe would drain at every step.  Fragments are double-buffered per k quarter
+// (32 k), not per step, to stay within 256 registers.  One barrier per step:
+// when the last quarter's fragments have been read the step's two slots are
+// free and take units 2s+5, 2s+6, while units 2s+2, 2s+3 must have landed (only
+// unit 2s+4 may still be in flight); those loads and the first fragments of
+// step s+1 are issued under the last quarter's MFMAs.
+namespace big {
+constexpr int BM = 256, BN = 256, TN = 4, TM = 2;
+constexpr int SLOT_BYTES = 256 * BK, SLOTS = 5;
+constexpr int PARK_BYTES = 8 * 32 * TM * (64 * TN + 16);
+constexpr int LDS_BYTES = SLOTS * SLOT_BYTES > PARK_BYTES ? SLOTS * SLOT_BYTES : PARK_BYTES;
+constexpr int LPU = 4;  // loads per wavefront and unit
+}  // namespace big
+
+__global__ void __launch_bounds__(512, 2)
+gemm_w8a8_big_kernel(const Args a) {
+    using namespace big;
+    extern __shared__ __align__(16) int8_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wn = wave & 1, wm = wave >> 1;
+
+    const int total = a.tiles_m * a.tiles_n;
+    int tile = blockIdx.x;
+    if (total % 8 == 0) tile = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
+    const int tn = tile / a.tiles_m, tm = tile - tn * a.tiles_m;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    // Wavefront w fills rows 32w .. 32w+31 of an operand tile: 4 loads of
+    // 8 rows x 128 B each; slot and swizzle as in the 4-wavefront kernel.
+    const int lrow = lane >> 3;
+    const int8_t *wsrc[4], *xsrc[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const int row = (4 * wave + g) * 8 + lrow;
+        const int kc = (lane & 7) ^ ((row >> 1) & 7);
+        wsrc[g] = a.wq + (size_t)min(n0 + row, a.N - 1) * a.K + kc * 16;
+        xsrc[g] = a.xq + (size_t)min(m0 + row, a.M - 1) * a.K + kc * 16;
+    }
+    // ring slot of a unit, as a byte offset
+    auto slot_of = [](int unit) { return (unit % SLOTS) * SLOT_BYTES; };
+    auto issue_w = [&](int ks) {
+        int8_t *base = lds + slot_of(2 * ks) + (4 * wave) * 1024;
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+            __builtin_amdgcn_global_load_lds((const void *)(wsrc[g] + ks * BK), (lds_ptr_t)(base + g * 1024), 16, 0, 0);
+    };
+    auto issue_x = [&](int ks) {
+        int8_t *base = lds + slot_of(2 * ks + 1) + (4 * wave) * 1024;
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+            __builtin_amdgcn_global_load_lds((const void *)(xsrc[g] + ks * BK), (lds_ptr_t)(base + g * 1024), 16, 0, 0);
+    };
+
+    const int frow = lane & 31;
+    const int fsw = (frow >> 1) & 7;
+    int foff[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) foff[q] = frow * BK + ((2 * q + (lane >> 5)) ^ fsw) * 16;
+    struct Frag {
+        v4i32 w[TN], x[TM];
+    };
+    auto read_q = [&](int ks, int q, Frag &f) {
+        const int8_t *wt = lds + slot_of(2 * ks) + wn * 32 * TN * BK + foff[q];
+        const int8_t *xt = lds + slot_of(2 * ks + 1) + wm * 32 * TM * BK + foff[q];
+#pragma unroll
+        for (int t = 0; t < TN; ++t) f.w[t] = *reinterpret_cast<const v4i32 *>(wt + t * 32 * BK);
+#pragma unroll
+        for (int t = 0; t < TM; ++t) f.x[t] = *reinterpret_cast<const v4i32 *>(xt + t * 32 * BK);
+    };
+
+    v16i32 acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+    auto mma_q = [&](const Frag &f) {
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w[i], f.x[j], acc[i][j], 0, 0, 0);
+    };
+    // 8 MFMAs with the 6 fragment reads of the next quarter spread between them
+    auto pace_quarter = [&]() {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (i < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+    };
+
+    const int ksteps = a.K / BK;
+    Frag f0, f1;
+    // Step ks computes from units 2ks, 2ks+1 (first-quarter fragments in f0).
+    // PHASE 2: steady state, two more units are requested (W of step ks+3 goes to
+    // the slot of this step's X... no slot arithmetic is needed: unit u always
+    // lives in slot u % 5, and units 2ks+5, 2ks+6 map onto the slots of 2ks, 2ks+1).
+    // PHASE 1: only unit 2ks+5 exists (X of step ks+2).  PHASE 0: nothing left.
+    auto step = [&](auto phase_tag, int ks) {
+        constexpr int PHASE = decltype(phase_tag)::value;
+        read_q(ks, 1, f1);
+        mma_q(f0);
+        pace_quarter();
+        read_q(ks, 2, f0);
+        mma_q(f1);
+        pace_quarter();
+        read_q(ks, 3, f1);
+        mma_q(f0);
+        pace_quarter();
+        // this wavefront's reads of the step's slots are done; units 2ks+2, 2ks+3 landed
+        if constexpr (PHASE == 2) wait_vmcnt<LPU>();
+        else wait_vmcnt<0>();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if constexpr (PHASE >= 1) issue_x(ks + 2);
+        if constexpr (PHASE == 2) issue_w(ks + 3);
+        read_q(ks + 1, 0, f0);  // past the last step: a stale slot nobody uses
+        mma_q(f1);
+        constexpr int VM_SLOTS = PHASE * 2;  // two loads per MFMA
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (i < VM_SLOTS) __builtin_amdgcn_sched_group_barrier(0x010, 2, 0);
+            else if (i - VM_SLOTS < 3) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+    };
+    using steady_t = std::integral_constant<int, 2>;
+    using last_x_t = std::integral_constant<int, 1>;
+    using drain_t = std::integral_constant<int, 0>;
+
+    // Prologue: units 0..4 = W0 X0 W1 X1 W2.
+    issue_w(0);
+    issue_x(0);
+    if (ksteps > 1) {
+        issue_w(1);
+        issue_x(1);
+    }
+    if (ksteps > 2) {
+        issue_w(2);
+        wait_vmcnt<3 * LPU>();
+    } else if (ksteps > 1) {
+        wait_vmcnt<2 * LPU>();
+    } else {
+        wait_vmcnt<0>();
+    }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    read_q(0, 0, f0);
+    // Step ks requests X of step ks+2 and W of step ks+3.
+    int ks = 0;
+    for (; ks + 3 < ksteps; ++ks) step(steady_t{}, ks);
+    if (ks + 2 < ksteps) step(last_x_t{}, ks++);
+    for (; ks < ksteps; ++ks) step(drain_t{}, ks);
+
+    epilogue<TN, TM>(a, acc, lds, wave, lane, n0 + wn * 32 * TN, m0 + wm * 32 * TM);
+}
+
+int launch_big(Args &a, hipStream_t st) {
+    a.tiles_m = (a.M + big::BM - 1) / big::BM;
+    a.tiles_n = (a.N + big::BN - 1) / big::BN;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w8a8_big_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, big::LDS_BYTES) != hipSuccess)
+            return fail(CMI_E_HIP, "cmi_gemm_w8a8: cannot reserve %d bytes of LDS", big::LDS_BYTES);
+        configured = true;
+    }
+    gemm_w8a8_big_kernel<<<dim3(a.tiles_m * a.tiles_n), dim3(512), big::LDS_BYTES, st>>>(a);
+    return check_launch("cmi_gemm_w8a8");
 }
 
 }  // namespace
@@ -254,16 +550,20 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
     a.N = N;
     a.K = K;
     a.ldy = ldy;
-    a.tiles_m = (M + BM - 1) / BM;
-    a.tiles_n = (N + BN - 1) / BN;
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w8a8_pipe_kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
-            return fail(CMI_E_HIP, "cmi_gemm_w8a8: cannot reserve %d bytes of LDS", LDS_BYTES);
-        configured = true;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // Tile choice: how full the last round of workgroups is (256 CUs; one 256 x 256
+    // workgroup or two 128 x 128 workgroups per CU), times the measured steady-state
+    // advantage of the large tile.  CMI_GEMM_TILE=128|256 overrides (tests, tuning).
+    const char *force = getenv("CMI_GEMM_TILE");
+    bool use_big;
+    if (force && force[0]) {
+        use_big = atoi(force) == 256;
+    } else {
+        const double tb = (double)((M + 255) / 256) * ((N + 255) / 256);
+        const double tsm = (double)((M + 127) / 128) * ((N + 127) / 128);
+        const double eff_big = tb / (ceil(tb / 256.0) * 256.0) * 1.23;
+        const double eff_small = tsm / (ceil(tsm / 512.0) * 512.0);
+        use_big = eff_big > eff_small;
     }
-    gemm_w8a8_pipe_kernel<<<dim3(a.tiles_m * a.tiles_n), dim3(THREADS), LDS_BYTES,
-                            static_cast<hipStream_t>(stream)>>>(a);
-    return check_launch("cmi_gemm_w8a8");
+    return use_big ? launch_big(a, st) : launch<2, 2, 2>(a, st);
 }

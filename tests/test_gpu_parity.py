@@ -153,10 +153,21 @@ def test_gemv_w8a16_lm_head_sampled_rows(orc):
 
 # ------------------------------------------------------------------ W8A8 GEMM
 
+@pytest.fixture(params=["auto", "128", "256"])
+def gemm_tile(request, monkeypatch):
+    """Force the 128 x 128 or the 256 x 256 block-tile kernel (the library reads
+    CMI_GEMM_TILE on every call), or leave the choice to the library."""
+    if request.param != "auto":
+        monkeypatch.setenv("CMI_GEMM_TILE", request.param)
+    else:
+        monkeypatch.delenv("CMI_GEMM_TILE", raising=False)
+    return request.param
+
+
 @pytest.mark.parametrize("m,n,k", [(128, 128, 128), (256, 256, 256), (512, 4096, 2560),
                                    (100, 200, 320), (130, 132, 2560), (64, 128, 64),
                                    (3, 5, 16), (300, 1030, 1040)])
-def test_gemm_w8a8_bit_exact(orc, m, n, k):
+def test_gemm_w8a8_bit_exact(orc, gemm_tile, m, n, k):
     g = seeded()
     q = synth.int8_weight(n, k, g)
     x = synth.activations(m, k, g, outliers=True)
@@ -169,7 +180,7 @@ def test_gemm_w8a8_bit_exact(orc, m, n, k):
     assert (y2.view(torch.int16) == y.view(torch.int16)).all()
 
 
-def test_gemm_w8a8_golden_and_row_stride(orc, golden):
+def test_gemm_w8a8_golden_and_row_stride(orc, golden, gemm_tile):
     g = golden("gemm_w8a8")
     acc, y = G.gemm_w8a8(G.dev(g["xq"]), G.dev(g["wq"]), G.dev(g["xs"]), G.dev(g["ws"]))
     assert (acc.cpu().numpy() == g["acc"]).all() and (G.bits(y) == g["y"]).all()
@@ -179,7 +190,7 @@ def test_gemm_w8a8_golden_and_row_stride(orc, golden):
 
 
 @pytest.mark.parametrize("m,n", [(2048, 9728), (8192, 4096)])
-def test_gemm_w8a8_full_size_sampled_and_blockwise(orc, m, n):
+def test_gemm_w8a8_full_size_sampled_and_blockwise(orc, gemm_tile, m, n):
     k = 2560
     g = synth.generator(1234, G.DEV)
     q = synth.int8_weight(n, k, g)
