@@ -43,6 +43,9 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="time only the W8A8 prefill GEMM (M=2048 and 8192, N=9728, K=2560): the profiling "
+                         "target for that kernel; prints its own JSON line")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (known traffic, for scaling HBM counters)")
     return ap.parse_args()
@@ -93,6 +96,23 @@ def main() -> int:
         dst.copy_(src)          # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
+
+    if args.prefill_only:
+        out = {}
+        for m, n_, k_ in ((2048, 9728, 2560), (8192, 9728, 2560)):
+            q = synth.int8_weight(n_, k_, gen)
+            x = synth.activations(m, k_, gen, outliers=True)
+            xq = torch.empty((m, k_), dtype=torch.int8, device=dev)
+            xs = torch.empty(m, dtype=torch.float32, device=dev)
+            y = torch.empty((m, n_), dtype=torch.bfloat16, device=dev)
+            lib.cmi_quant_act_i8(ptr(x), ptr(xq), ptr(xs), m, k_, cur_stream())
+            t = timed(lambda: lib.cmi_gemm_w8a8(ptr(xq), ptr(q.wq), ptr(xs), ptr(q.scale), ptr(y), vp(0),
+                                                m, n_, k_, n_, cur_stream()), args.steps, args.warmup)
+            tops = synth.gemm_ops(m, n_, k_) / t / 1e12
+            out[f"M{m}_N{n_}_K{k_}"] = {"gemm_us": round(t * 1e6, 2), "tops": round(tops, 1),
+                                        "frac_of_int8_peak": round(tops / INT8_PEAK_TOPS, 4)}
+        print(json.dumps({"metric": "W8A8 prefill GEMM int8 TOPS", "unit": "TOP/s", "w8a8_prefill_gemm": out}))
+        return 0
 
     # ------------------------------------------------------------ headline: decode GEMVs
     M = args.rows

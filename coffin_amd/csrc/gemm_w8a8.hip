@@ -85,6 +85,25 @@ __device__ __forceinline__ void wait_vmcnt() {
     else static_assert(N < 0, "add the vmcnt literal");
 }
 
+// Tile of this workgroup.  Workgroups are dealt round-robin to the 8 XCDs (each
+// with a private L2), so XCD x is given the contiguous run of logical tiles
+// [x*per, (x+1)*per); logical tiles walk bands of 8 m tiles, m fastest inside a
+// band, so the ~32-64 workgroups an XCD runs at a time form an 8 x (4..8) patch
+// that shares its X rows and W rows through that L2 instead of streaming the
+// whole of X once per n tile.
+__device__ __forceinline__ void tile_coords(const Args &a, int &tm, int &tn) {
+    constexpr int GM = 8;
+    const int total = a.tiles_m * a.tiles_n;
+    int t = blockIdx.x;
+    if (total % 8 == 0) t = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
+    const int width = GM * a.tiles_n;
+    const int band = t / width, in_band = t - band * width;
+    const int first_m = band * GM;
+    const int rows = min(a.tiles_m - first_m, GM);
+    tn = in_band / rows;
+    tm = first_m + (in_band - tn * rows);
+}
+
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
 
@@ -187,12 +206,8 @@ gemm_w8a8_pipe_kernel(const Args a) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: keeps LDS bases scalar
     const int wn = wave & 1, wm = wave >> 1;
 
-    // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs; XCD x
-    // gets logical tiles [x*per, (x+1)*per), m fastest inside a band of n tiles.
-    const int total = a.tiles_m * a.tiles_n;
-    int tile = blockIdx.x;
-    if (total % 8 == 0) tile = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
-    const int tn = tile / a.tiles_m, tm = tile - tn * a.tiles_m;
+    int tm, tn;
+    tile_coords(a, tm, tn);
     const int m0 = tm * C::BM, n0 = tn * C::BN;
 
     // Global side of the direct loads.  One load instruction moves 8 rows x 128 B
@@ -374,10 +389,8 @@ gemm_w8a8_big_kernel(const Args a) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wn = wave & 1, wm = wave >> 1;
 
-    const int total = a.tiles_m * a.tiles_n;
-    int tile = blockIdx.x;
-    if (total % 8 == 0) tile = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
-    const int tn = tile / a.tiles_m, tm = tile - tn * a.tiles_m;
+    int tm, tn;
+    tile_coords(a, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
 
     // Wavefront w fills rows 32w .. 32w+31 of an operand tile: 4 loads of
