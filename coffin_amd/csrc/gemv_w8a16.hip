@@ -30,7 +30,7 @@
 // channels that own those lines, so a workgroup (4 wavefronts, 16 for 16 rows)
 // copies them into LDS once -- requested before the weights, because memory
 // returns data in issue order -- and every wavefront reads its fragments from
-// there, at most 8 activation rows in registers at a time (for 4 rows and more
+// there, at most 4 activation rows in registers at a time (for 4 rows and more
 // in an order that makes the reads free of bank conflicts).  Batches whose
 // activations do not fit LDS are split into narrower calls.  A unit wider than
 // the register budget of M rows is walked in sub-trips with the next sub-trip's
@@ -88,13 +88,24 @@ __device__ __forceinline__ void widen4(uint32_t w, bf16x2_t &lo, bf16x2_t &hi) {
 
 // Wavefronts per workgroup (they share one LDS copy of the activations); wide
 // batches get smaller workgroups so that each wavefront may use more registers.
-constexpr int block_waves(int m) { return m >= 16 ? 16 : 4; }
+constexpr int block_waves(int m) { return m >= 16 ? 16 : m >= 8 ? 8 : 4; }
 
 // Wavefronts per SIMD the register allocation must leave room for.
-constexpr int simd_waves(int m, int cht) { return m >= 16 || (m == 4 && cht == 1) ? 4 : 1; }
+constexpr int simd_waves(int m, int cht) { return m >= 8 || (m == 4 && cht == 1) ? 4 : 1; }
 
-// Activation rows held in registers at a time; wider batches loop over tiles of this many.
-constexpr int m_tile(int m) { return m < 8 ? m : 8; }
+// uint4 vectors of the LDS copy of the activations.  Up to 2 rows: [row][K] as in memory plus
+// one zeroed 32-byte slot.  From 4 rows: [segment][row of the M tile][half][lane], 2 KiB per
+// (segment, row) with the tail of the last segment and any dead segments zeroed, so a
+// wavefront's reads are contiguous across lanes, rows differ by a compile-time offset and
+// dead chunks read zeros without a select.
+__host__ __device__ constexpr int xlds_vectors(int mt, int rows, int K, int segs) {
+    return mt >= 4 ? segs * mt * 128 : rows * (K / 8) + 2;
+}
+
+// Activation rows held in registers at a time; wider batches loop over tiles of this many
+// (4 rows = 32 registers: with accumulators and weights the kernel stays under 128, which
+// 4 wavefronts per SIMD need; a spill inside the K loop costs a memory round trip each).
+constexpr int m_tile(int m) { return m < 4 ? m : 4; }
 
 // 16-byte vectors of activations each thread carries from global memory to LDS.
 constexpr int xstage_vectors(int m) { return m <= 1 ? 8 : m <= 2 ? 16 : m <= 4 ? 20 : 8; }
@@ -117,7 +128,7 @@ struct WStage {
 template <int M, int R, int CHT, int MODE, bool XLDS>
 __global__ void __launch_bounds__(64 * block_waves(M), simd_waves(M, CHT))
 gemv_w8a16_kernel(const GemvArgs a) {
-    extern __shared__ uint4 smem[];  // [a.M][K] bf16 activations + 32 zero bytes (XLDS), then unit totals
+    extern __shared__ uint4 smem[];  // staged activations (XLDS, see xlds_vectors), then unit totals
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int team = wave / a.uw;
@@ -125,7 +136,8 @@ gemv_w8a16_kernel(const GemvArgs a) {
     const bool idle = rb >= a.nblocks;  // only in the last workgroup
     int u = wave - team * a.uw;         // unit in hand; the team's wavefronts stride over units
     const int xvecs = a.K / 8;          // uint4 per activation row
-    float *unit_total = reinterpret_cast<float *>(smem + (XLDS ? a.M * xvecs + 2 : 0)) +
+    const int segs = a.units * a.unit;  // segments the unit loop walks (>= nseg)
+    float *unit_total = reinterpret_cast<float *>(smem + (XLDS ? xlds_vectors(M, a.M, a.K, segs) : 0)) +
                         team * a.units * (R * M);
 
     const u32x4 *wrow[R];
@@ -165,10 +177,9 @@ gemv_w8a16_kernel(const GemvArgs a) {
                     // dead chunks read the zeroed slot behind the activations: a select
                     // on the address, so the LDS reads stay unconditional
                     if constexpr (M >= 4) {
-                        const int cseg = min(64, a.nchunks - seg * 64);  // chunks in this segment
-                        const int lo = mrow * xvecs + seg * 128 + lane + xoff;
-                        s.x[m][j][0] = smem[live ? lo : a.M * xvecs];
-                        s.x[m][j][1] = smem[live ? lo + cseg : a.M * xvecs];
+                        const int at = (seg * M + mh * MT + m) * 128 + lane + xoff;
+                        s.x[m][j][0] = smem[at];
+                        s.x[m][j][1] = smem[at + 64];
                     } else {
                         const int at = live ? mrow * xvecs + 2 * chunk : a.M * xvecs;
                         s.x[m][j][0] = smem[at];
@@ -250,13 +261,27 @@ gemv_w8a16_kernel(const GemvArgs a) {
                 const int row = __umulhi((uint32_t)idx, a.xvecs_rcp);
                 const int v = idx - row * xvecs;
                 const int seg = v >> 7, half = v & 1, c = (v & 127) >> 1;
-                const int cseg = min(64, a.nchunks - seg * 64);
-                if (idx < xtotal) smem[row * xvecs + seg * 128 + half * cseg + c] = xstage[j];
+                if (idx < xtotal) smem[(seg * M + row) * 128 + half * 64 + c] = xstage[j];
             } else {
                 if (idx < xtotal) smem[idx] = xstage[j];  // little LDS traffic: plain order
             }
         }
-        if (threadIdx.x < 2) smem[xtotal + threadIdx.x] = make_uint4(0, 0, 0, 0);
+        if constexpr (M >= 4) {
+            // zero what no activation covers: lanes past K in the last segment, dead segments
+            const int last = a.nseg - 1, cl = a.nchunks - last * 64;  // chunks in the last segment
+            const int tail = 64 - cl;                                  // zero vectors per (row, half) there
+            const int n_tail = a.M * 2 * tail;
+            for (int i = threadIdx.x; i < n_tail; i += blockDim.x) {
+                const int row = i / (2 * tail), rem = i - row * 2 * tail;
+                const int half = rem / tail, c = cl + rem - half * tail;
+                smem[(last * M + row) * 128 + half * 64 + c] = make_uint4(0, 0, 0, 0);
+            }
+            const int n_dead = (segs - a.nseg) * M * 128;
+            for (int i = threadIdx.x; i < n_dead; i += blockDim.x)
+                smem[a.nseg * M * 128 + i] = make_uint4(0, 0, 0, 0);
+        } else {
+            if (threadIdx.x < 2) smem[xtotal + threadIdx.x] = make_uint4(0, 0, 0, 0);
+        }
         __syncthreads();
     }
 
@@ -274,12 +299,11 @@ gemv_w8a16_kernel(const GemvArgs a) {
                 // Wide batches: the next tile's LDS address is made to depend on this
                 // tile's sums, so only one activation tile is ever live in registers
                 // (other wavefronts of the SIMD cover the LDS latency).
-                if constexpr (M >= 16) {
+                if constexpr (M >= 8) {
 #pragma unroll
                     for (int r = 0; r < R; ++r) {
                         float *p = &acc[r][mh * MT];
-                        asm volatile("" : "+v"(p[0]), "+v"(p[1]), "+v"(p[2]), "+v"(p[3]), "+v"(p[4]),
-                                          "+v"(p[5]), "+v"(p[6]), "+v"(p[7]), "+v"(xoff));
+                        asm volatile("" : "+v"(p[0]), "+v"(p[1]), "+v"(p[2]), "+v"(p[3]), "+v"(xoff));
                     }
                 }
             }
@@ -358,7 +382,7 @@ struct Plan {
 //: Most K-units one launch handles (LDS holds one total per unit and output).
 constexpr int MAX_UNITS = 64;
 //: Activations up to this many bytes are staged in LDS.
-constexpr size_t XLDS_MAX_BYTES = 96 * 1024;
+constexpr size_t XLDS_MAX_BYTES = 128 * 1024;
 
 // Blocking is a pure function of (M, N, K); it never changes results.
 Plan make_plan(int M, int N, int K) {
@@ -389,7 +413,7 @@ int launch(GemvArgs &a, hipStream_t st) {
     a.teams = block_waves(M) / a.uw;
     const dim3 grid((a.nblocks + a.teams - 1) / a.teams);
     const dim3 block(64 * a.uw * a.teams);
-    const size_t lds = (XLDS ? (size_t)a.M * a.K * 2 + 32 : 0) +
+    const size_t lds = (XLDS ? 16 * (size_t)xlds_vectors(M, a.M, a.K, a.units * a.unit) : 0) +
                        (MODE == 0 ? 0 : sizeof(float) * a.teams * a.units * R * M);
     static bool configured = false;
     if (!configured) {
@@ -403,19 +427,20 @@ int launch(GemvArgs &a, hipStream_t st) {
 }
 
 // Whether a workgroup of the M-tile's kernel can carry [rows, K] activations into LDS.
-bool x_fits_lds(int mt, int rows, int K, int units) {
-    const size_t xbytes = (size_t)rows * K * 2;
+bool x_fits_lds(int mt, int rows, int K, int units, int segs) {
+    const size_t xbytes = (size_t)rows * K * 2;                              // carried by the threads
+    const size_t ldsbytes = 16 * (size_t)xlds_vectors(mt, rows, K, segs);   // held in LDS
     const int uw = units < 4 ? units : 4;
-    const int bw = mt >= 16 ? block_waves(16) : block_waves(1);
+    const int bw = mt >= 16 ? block_waves(16) : mt >= 8 ? block_waves(8) : block_waves(1);
     const int xv = mt <= 1 ? xstage_vectors(1) : mt <= 2 ? xstage_vectors(2) : mt <= 4 ? xstage_vectors(4)
                                                                              : xstage_vectors(8);
     const size_t threads = 64 * (size_t)uw * (bw / uw);  // as launch() sizes the workgroup
-    return xbytes <= XLDS_MAX_BYTES && xbytes <= 16 * (size_t)xv * threads;
+    return ldsbytes <= XLDS_MAX_BYTES && xbytes <= 16 * (size_t)xv * threads;
 }
 
 template <int M, int R, int CHT, int MODE>
 int dispatch_lds(GemvArgs &a, hipStream_t st) {
-    if (x_fits_lds(M, a.M, a.K, a.units)) return launch<M, R, CHT, MODE, true>(a, st);
+    if (x_fits_lds(M, a.M, a.K, a.units, a.units * a.unit)) return launch<M, R, CHT, MODE, true>(a, st);
     return launch<M, R, CHT, MODE, false>(a, st);
 }
 
@@ -474,7 +499,7 @@ extern "C" int cmi_gemv_w8a16(const int8_t *wq, const float *ws, const void *x, 
                 MAX_UNITS * 4096);
     // Activations too large for LDS: narrower batches fit more often, and rows are
     // independent (same bits whatever the batch), so halve the batch instead.
-    if (M > 1 && !x_fits_lds(p.mt, M, K, a.units)) {
+    if (M > 1 && !x_fits_lds(p.mt, M, K, a.units, a.units * a.unit)) {
         const int half = p.mt / 2;
         const int rc = cmi_gemv_w8a16(wq, ws, x, y, half, N, K, stream);
         if (rc != CMI_OK) return rc;
