@@ -266,6 +266,15 @@ def main() -> int:
                 t = timed(one, 5) / copies
                 w4[f"{k_}->{n_}_M{m}"] = {"us": round(t * 1e6, 2),
                                           "GBps": round(synth.w4_gemv_bytes(m, n_, k_) / t / 1e9, 1)}
+                if m <= 4:
+                    def fused(m=m, x=x, y=y, ws_=ws_, n_=n_, k_=k_):
+                        st = cur_stream()
+                        for d4, ds in ws_:
+                            lib.cmi_gemv_w4a8_bf16(ptr(d4), ptr(ds), ptr(x), ptr(y), vp(0), vp(0), vp(0),
+                                                   m, n_, k_, 128, st)
+                    t = timed(fused, 5) / copies
+                    w4[f"{k_}->{n_}_M{m}_fused"] = {"us": round(t * 1e6, 2),
+                                                    "GBps": round(synth.w4_gemv_bytes(m, n_, k_) / t / 1e9, 1)}
             del ws_
         extra["w4a8_gemv_quant_plus_gemv"] = w4
         torch.cuda.empty_cache()

@@ -47,6 +47,8 @@ GEMV_MAX_ROWS = 16
 PREFILL_MIN_ROWS = 64
 #: W4A8 switches from the GEMV to the MFMA GEMM above this many rows.
 W4_GEMM_MIN_ROWS = 17
+#: Up to this many rows the W4A8 GEMV quantises its activations itself (one launch).
+W4_FUSED_MAX_ROWS = 4
 
 _vp = ctypes.c_void_p
 
@@ -175,12 +177,20 @@ def _rows_w4(w, act: torch.Tensor) -> torch.Tensor:
     n, k, gs = int(w.n), int(w.k), int(w.group_size)
     rows = act.shape[0]
     w4, ws = _w4_operands(w)
-    xq, xs = _scratch(rows, k, act.device)
     out = torch.empty((rows, n), dtype=torch.bfloat16, device=act.device)
     if rows == 0:
         return out
-    _quantize_rows(act, xq, xs)
     lib = _native.load()
+    if rows <= W4_FUSED_MAX_ROWS:
+        # decode: one launch, activations quantised inside the GEMV (same bits)
+        rc = lib.cmi_gemv_w4a8_bf16(_ptr(w4), _ptr(ws), _ptr(act), _ptr(out), _vp(0), _vp(0), _vp(0),
+                                    rows, n, k, gs, _stream())
+        if rc == 0:
+            return out
+        if rc != _native.E_UNSUPPORTED:
+            _native.check(rc, "gemv_w4a8_bf16")
+    xq, xs = _scratch(rows, k, act.device)
+    _quantize_rows(act, xq, xs)
     fn, what = ((lib.cmi_gemm_w4a8, "gemm_w4a8") if rows >= W4_GEMM_MIN_ROWS
                 else (lib.cmi_gemv_w4a8, "gemv_w4a8"))
     _native.check(fn(_ptr(w4), _ptr(ws), _ptr(xq), _ptr(xs), _ptr(out), _vp(0), rows, n, k, gs,

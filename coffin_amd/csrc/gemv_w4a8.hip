@@ -14,7 +14,7 @@
 // the arithmetic is a strict chain over the groups and is order sensitive, so
 // group sums go through LDS and one lane per (row, m) walks them in order:
 // the result does not depend on how K was split over wavefronts or trips.
-#include "common.hpp"
+#include "quant_math.hpp"
 
 namespace {
 
@@ -23,12 +23,16 @@ using namespace cmi;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int GS = 128;  // group size the kernels are built for
+constexpr int FUSED_MAX_ROWS = 4;  // activation rows the fused-quantiser variant takes
 
 struct W4Args {
     const uint8_t *w4;
     const float *ws;
     const int8_t *xq;
     const float *xs;
+    const uint16_t *xb;   // bf16 activations (fused quantiser) or null
+    int8_t *xq_out;       // optional copies of the fused quantiser's results
+    float *xs_out;
     uint16_t *y;
     int32_t *group_acc;
     int M, N, K;
@@ -37,11 +41,62 @@ struct W4Args {
     int KW, teams, iters;
 };
 
-template <int M, int R2, int CH>
+// XV == 0: activations arrive quantised (a.xq, a.xs).  XV > 0: they arrive as bf16
+// (a.xb) and every workgroup (256 threads) quantises them into LDS first -- XV
+// 16-byte vectors per thread and row -- with the arithmetic of the stand-alone
+// quantiser; the bf16 loads are issued before anything else and the weight
+// stream hides the work.  Saves a launch and the int8 round trip through memory.
+template <int M, int R2, int CH, int XV>
 __global__ void __launch_bounds__(256)
 gemv_w4a8_kernel(const W4Args a) {
     constexpr int ROWS = 2 * R2;
-    extern __shared__ int32_t sums[];  // [teams][iters*KW*CH*8 groups][ROWS*M]
+    extern __shared__ int32_t sums_base[];  // [fused: M*K int8, M scales, M*4 partial maxima] [teams][groups][ROWS*M]
+    int8_t *xq_lds = reinterpret_cast<int8_t *>(sums_base);
+    float *xs_lds = reinterpret_cast<float *>(xq_lds + (XV ? (size_t)M * a.K : 0));
+    int32_t *sums = reinterpret_cast<int32_t *>(xs_lds + (XV ? M * 5 : 0));
+    if constexpr (XV > 0) {
+        const int xvecs = a.K / 8;
+        uint4 v[M][XV];
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            const uint4 *xg = reinterpret_cast<const uint4 *>(a.xb + (size_t)(m < a.M ? m : a.M - 1) * a.K);
+#pragma unroll
+            for (int j = 0; j < XV; ++j) {
+                const int idx = threadIdx.x + j * 256;
+                v[m][j] = idx < xvecs ? xg[idx] : make_uint4(0, 0, 0, 0);
+            }
+        }
+        float *part = xs_lds + M;
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            float amax = 0.f;
+#pragma unroll
+            for (int j = 0; j < XV; ++j) amax = absmax8(v[m][j], amax);
+            amax = wave_max_to_lane63(amax);
+            if ((threadIdx.x & 63) == 63) part[m * 4 + (threadIdx.x >> 6)] = amax;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            const float amax = fmaxf(fmaxf(part[m * 4], part[m * 4 + 1]), fmaxf(part[m * 4 + 2], part[m * 4 + 3]));
+            const float sc = quant_scale(amax);
+            if (threadIdx.x == 0) {
+                xs_lds[m] = sc;
+                if (a.xs_out && blockIdx.x == 0 && m < a.M) a.xs_out[m] = sc;
+            }
+#pragma unroll
+            for (int j = 0; j < XV; ++j) {
+                const int idx = threadIdx.x + j * 256;
+                if (idx < xvecs) {
+                    const uint2 q = quant8(v[m][j], sc);
+                    reinterpret_cast<uint2 *>(xq_lds + (size_t)m * a.K)[idx] = q;
+                    if (a.xq_out && blockIdx.x == 0 && m < a.M)
+                        reinterpret_cast<uint2 *>(a.xq_out + (size_t)m * a.K)[idx] = q;
+                }
+            }
+        }
+        __syncthreads();
+    }
     const int lane = threadIdx.x & 63;
     const int half = lane >> 5, hl = lane & 31;
     const int wave = threadIdx.x >> 6;
@@ -83,7 +138,8 @@ gemv_w4a8_kernel(const W4Args a) {
 #pragma unroll
         for (int m = 0; m < M; ++m) {
             const int mrow = m < a.M ? m : a.M - 1;
-            const uint4 *xp = reinterpret_cast<const uint4 *>(a.xq + (size_t)mrow * a.K);
+            const uint4 *xp = XV ? reinterpret_cast<const uint4 *>(xq_lds + (size_t)m * a.K)
+                                 : reinterpret_cast<const uint4 *>(a.xq + (size_t)mrow * a.K);
 #pragma unroll
             for (int j = 0; j < CH; ++j) {
                 if (live[j]) {
@@ -144,7 +200,7 @@ gemv_w4a8_kernel(const W4Args a) {
                 if (a.group_acc) a.group_acc[((size_t)m * a.G + g) * a.N + n] = s;
                 total = fmaf((float)s, wsn[g], total);
             }
-            a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * a.xs[m]);
+            a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * (XV ? xs_lds[m] : a.xs[m]));
         }
     }
 }
@@ -191,15 +247,32 @@ Plan make_plan(int M, int N, int K) {
     return p;
 }
 
-template <int M, int R2, int CH>
-int launch(const W4Args &a, hipStream_t st) {
+template <int M, int R2, int CH, int XV>
+int launch_xv(const W4Args &a, hipStream_t st) {
     const int rows_per_block = 2 * R2 * a.teams;
     const dim3 grid((a.N + rows_per_block - 1) / rows_per_block);
-    const size_t lds = sizeof(int32_t) * a.teams * (a.iters * a.KW * CH * 8) * (2 * R2 * M);
+    const size_t lds = sizeof(int32_t) * a.teams * (a.iters * a.KW * CH * 8) * (2 * R2 * M) +
+                       (XV ? (size_t)M * a.K + sizeof(float) * M * 5 : 0);
     if (lds > 64 * 1024)
         return fail(CMI_E_UNSUPPORTED, "cmi_gemv_w4a8: K=%d needs %zu bytes of LDS", a.K, lds);
-    gemv_w4a8_kernel<M, R2, CH><<<grid, dim3(64 * a.KW * a.teams), lds, st>>>(a);
+    gemv_w4a8_kernel<M, R2, CH, XV><<<grid, dim3(64 * a.KW * a.teams), lds, st>>>(a);
     return check_launch("cmi_gemv_w4a8");
+}
+
+template <int M, int R2, int CH>
+int launch(const W4Args &a, hipStream_t st) {
+    if (!a.xb) return launch_xv<M, R2, CH, 0>(a, st);
+    if constexpr (M <= FUSED_MAX_ROWS) {
+        // the fused prologue is written for 256 threads
+        if (a.KW * a.teams != 4)
+            return fail(CMI_E_UNSUPPORTED, "cmi_gemv_w4a8_bf16: K=%d leaves a workgroup of %d wavefronts", a.K,
+                        a.KW * a.teams);
+        const int xv = (a.K / 8 + 255) / 256;
+        if (xv <= 2) return launch_xv<M, R2, CH, 2>(a, st);
+        if (xv <= 5) return launch_xv<M, R2, CH, 5>(a, st);
+        if (xv <= 8) return launch_xv<M, R2, CH, 8>(a, st);
+    }
+    return fail(CMI_E_UNSUPPORTED, "cmi_gemv_w4a8_bf16: M=%d K=%d outside the fused kernel's range", a.M, a.K);
 }
 
 template <int M, int R2>
@@ -223,22 +296,24 @@ int dispatch_r(const W4Args &a, const Plan &p, hipStream_t st) {
 
 }  // namespace
 
-extern "C" int cmi_gemv_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs,
-                             void *y, int32_t *group_acc, int M, int N, int K, int gs,
-                             void *stream) {
-    CMI_REQUIRE(w4 && ws && xq && xs && y, CMI_E_ARG, "cmi_gemv_w4a8: null pointer");
-    CMI_REQUIRE(M >= 1 && M <= 16, CMI_E_UNSUPPORTED, "cmi_gemv_w4a8: M=%d outside 1..16", M);
-    CMI_REQUIRE(N >= 1 && K >= GS, CMI_E_ARG, "cmi_gemv_w4a8: bad shape N=%d K=%d", N, K);
-    CMI_REQUIRE(gs == GS, CMI_E_UNSUPPORTED, "cmi_gemv_w4a8: group size %d, kernels are built for %d", gs, GS);
-    CMI_REQUIRE(K % GS == 0, CMI_E_UNSUPPORTED, "cmi_gemv_w4a8: K=%d is not a multiple of %d", K, GS);
-    CMI_REQUIRE(aligned(w4, 16) && aligned(xq, 16), CMI_E_ARG,
-                "cmi_gemv_w4a8: w4 and xq must be 16-byte aligned");
+namespace {
+
+int run_gemv_w4a8(const char *who, const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs,
+                  const void *xb, int8_t *xq_out, float *xs_out, void *y, int32_t *group_acc, int M, int N,
+                  int K, int gs, void *stream) {
+    CMI_REQUIRE(M >= 1 && M <= 16, CMI_E_UNSUPPORTED, "%s: M=%d outside 1..16", who, M);
+    CMI_REQUIRE(N >= 1 && K >= GS, CMI_E_ARG, "%s: bad shape N=%d K=%d", who, N, K);
+    CMI_REQUIRE(gs == GS, CMI_E_UNSUPPORTED, "%s: group size %d, kernels are built for %d", who, gs, GS);
+    CMI_REQUIRE(K % GS == 0, CMI_E_UNSUPPORTED, "%s: K=%d is not a multiple of %d", who, K, GS);
     const Plan p = make_plan(M, N, K);
     W4Args a;
     a.w4 = w4;
     a.ws = ws;
     a.xq = xq;
     a.xs = xs;
+    a.xb = static_cast<const uint16_t *>(xb);
+    a.xq_out = xq_out;
+    a.xs_out = xs_out;
     a.y = static_cast<uint16_t *>(y);
     a.group_acc = group_acc;
     a.M = M;
@@ -257,4 +332,29 @@ extern "C" int cmi_gemv_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
         case 8: return dispatch_r<8>(a, p, st);
         default: return dispatch_r<16>(a, p, st);
     }
+}
+
+}  // namespace
+
+extern "C" int cmi_gemv_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs,
+                             void *y, int32_t *group_acc, int M, int N, int K, int gs,
+                             void *stream) {
+    CMI_REQUIRE(w4 && ws && xq && xs && y, CMI_E_ARG, "cmi_gemv_w4a8: null pointer");
+    CMI_REQUIRE(aligned(w4, 16) && aligned(xq, 16), CMI_E_ARG,
+                "cmi_gemv_w4a8: w4 and xq must be 16-byte aligned");
+    return run_gemv_w4a8("cmi_gemv_w4a8", w4, ws, xq, xs, nullptr, nullptr, nullptr, y, group_acc, M, N, K, gs,
+                         stream);
+}
+
+extern "C" int cmi_gemv_w4a8_bf16(const uint8_t *w4, const float *ws, const void *x, void *y,
+                                  int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
+                                  int gs, void *stream) {
+    CMI_REQUIRE(w4 && ws && x && y, CMI_E_ARG, "cmi_gemv_w4a8_bf16: null pointer");
+    CMI_REQUIRE(aligned(w4, 16) && aligned(x, 16) && (!xq_out || aligned(xq_out, 8)), CMI_E_ARG,
+                "cmi_gemv_w4a8_bf16: w4 and x must be 16-byte aligned, xq_out 8-byte aligned");
+    CMI_REQUIRE(M >= 1 && M <= FUSED_MAX_ROWS, CMI_E_UNSUPPORTED,
+                "cmi_gemv_w4a8_bf16: M=%d outside 1..%d (quantise with cmi_quant_act_i8 and call cmi_gemv_w4a8)",
+                M, FUSED_MAX_ROWS);
+    return run_gemv_w4a8("cmi_gemv_w4a8_bf16", w4, ws, nullptr, nullptr, x, xq_out, xs_out, y, group_acc, M, N, K,
+                         gs, stream);
 }

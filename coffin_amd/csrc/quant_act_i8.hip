@@ -5,43 +5,13 @@
 // thread), so HBM traffic is the algorithmic 2 B in + 1 B out per element.
 // The scale and the rounding follow the torch spec bit for bit: IEEE fp32
 // division by the scale (not a reciprocal multiply), round-half-even, clamp.
-#include "common.hpp"
+#include "quant_math.hpp"
 
 namespace {
 
 using namespace cmi;
 
 constexpr int QUANT_THREADS = 256;
-
-__device__ __forceinline__ float absmax8(const uint4 &v, float amax) {
-    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        amax = fmaxf(amax, fabsf(bf16_bits_to_f32(w[i] & 0xffffu)));
-        amax = fmaxf(amax, fabsf(__uint_as_float(w[i] & 0xffff0000u)));
-    }
-    return amax;
-}
-
-__device__ __forceinline__ uint32_t quant1(float x, float sc) {
-    float q = rintf(__fdiv_rn(x, sc));
-    q = fminf(fmaxf(q, -127.f), 127.f);
-    return (uint32_t)((int)q) & 0xffu;
-}
-
-__device__ __forceinline__ uint2 quant8(const uint4 &v, float sc) {
-    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-    uint32_t b[8];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        b[2 * i] = quant1(bf16_bits_to_f32(w[i] & 0xffffu), sc);
-        b[2 * i + 1] = quant1(__uint_as_float(w[i] & 0xffff0000u), sc);
-    }
-    uint2 o;
-    o.x = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
-    o.y = b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24);
-    return o;
-}
 
 // Block-wide max of non-negative values; every thread returns the result.
 __device__ __forceinline__ float block_max(float v, float *smem) {
@@ -76,7 +46,7 @@ quant_act_i8_vec(const uint4 *__restrict__ x, uint2 *__restrict__ q, float *__re
 #pragma unroll
         for (int i = 0; i < VPT; ++i) amax = absmax8(v[i], amax);
         amax = block_max(amax, smem);
-        const float sc = fmaxf(amax, 1e-5f) / 127.0f;
+        const float sc = quant_scale(amax);
         if (threadIdx.x == 0) s[row] = sc;
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
@@ -86,7 +56,7 @@ quant_act_i8_vec(const uint4 *__restrict__ x, uint2 *__restrict__ q, float *__re
     } else {
         for (int idx = threadIdx.x; idx < nvec; idx += QUANT_THREADS) amax = absmax8(xr[idx], amax);
         amax = block_max(amax, smem);
-        const float sc = fmaxf(amax, 1e-5f) / 127.0f;
+        const float sc = quant_scale(amax);
         if (threadIdx.x == 0) s[row] = sc;
         for (int idx = threadIdx.x; idx < nvec; idx += QUANT_THREADS) qr[idx] = quant8(xr[idx], sc);
     }
@@ -104,7 +74,7 @@ quant_act_i8_scalar(const uint16_t *__restrict__ x, int8_t *__restrict__ q,
     for (int k = threadIdx.x; k < K; k += QUANT_THREADS)
         amax = fmaxf(amax, fabsf(bf16_bits_to_f32(xr[k])));
     amax = block_max(amax, smem);
-    const float sc = fmaxf(amax, 1e-5f) / 127.0f;
+    const float sc = quant_scale(amax);
     if (threadIdx.x == 0) s[row] = sc;
     for (int k = threadIdx.x; k < K; k += QUANT_THREADS)
         qr[k] = (int8_t)quant1(bf16_bits_to_f32(xr[k]), sc);

@@ -79,6 +79,17 @@ int cmi_w4_repack(const uint8_t *packed, const float *scale, uint8_t *w4, float 
 int cmi_gemv_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs,
                   void *y, int32_t *group_acc, int M, int N, int K, int gs, void *stream);
 
+/* cmi_gemv_w4a8 with the activation quantiser folded in, 1 <= M <= 4: x is bf16
+ * [M,K]; every workgroup quantises it on the fly with the arithmetic of
+ * cmi_quant_act_i8 (same bits), so one launch replaces quant_act_i8 + w4a8_gemv
+ * on the decode path (backends/corex/__init__.py:640-649 issues the two).
+ * xq_out / xs_out (nullable; xq_out 8-byte aligned) receive the int8 rows and
+ * scales the kernel used, for parity checks.  Shapes the fused kernel does not
+ * take return CMI_E_UNSUPPORTED: quantise and call cmi_gemv_w4a8 then. */
+int cmi_gemv_w4a8_bf16(const uint8_t *w4, const float *ws, const void *x, void *y,
+                       int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
+                       int gs, void *stream);
+
 /* W8A8 GEMM with fused epilogue:
  *   acc[m,n] = sum_k xq[m,k]*wq[n,k]  (int32) ; y[m,n] = bf16((float)acc*xs[m]*ws[n])
  * xq int8 [M,K], wq int8 [N,K], y bf16 with row stride ldy >= N.  K % 64 == 0.

@@ -79,3 +79,16 @@ def w4a8(w4, ws, xq, xs, k, gemm: bool, want_acc=True, gs=128):
     _native.check(fn(ptr(w4), ptr(ws), ptr(xq), ptr(xs), ptr(y), ptr(gacc), m, n, k, gs, stream()),
                   "gemm_w4a8" if gemm else "gemv_w4a8")
     return gacc, y
+
+
+def gemv_w4a8_bf16(w4, ws, x, k, gs=128):
+    """Fused quantiser + W4A8 GEMV; returns (group sums, y, xq used, xs used)."""
+    m = x.shape[0]
+    n = w4.shape[0]
+    y = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+    gacc = torch.empty((m, k // gs, n), dtype=torch.int32, device=DEV)
+    xq = torch.empty((m, k), dtype=torch.int8, device=DEV)
+    xs = torch.empty(m, dtype=torch.float32, device=DEV)
+    _native.check(_native.load().cmi_gemv_w4a8_bf16(ptr(w4), ptr(ws), ptr(x), ptr(y), ptr(gacc), ptr(xq),
+                                                    ptr(xs), m, n, k, gs, stream()), "gemv_w4a8_bf16")
+    return gacc, y, xq, xs

@@ -236,6 +236,34 @@ def test_gemv_w4a8_bit_exact(orc, m, n, k):
     assert (y2.view(torch.int16) == y.view(torch.int16)).all()
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 9728, 2560), (1, 2560, 9728), (4, 512, 256), (2, 333, 1280),
+                                   (3, 7, 128), (4, 6144, 2560), (1, 2560, 4096), (4, 2560, 9728),
+                                   (2, 640, 16384)])
+def test_gemv_w4a8_bf16_fused_quantiser_bit_exact(orc, m, n, k):
+    """One launch from bf16 activations: the quantised rows, the scales, the group
+    sums and the output all carry the bits of quantiser + GEMV run separately."""
+    g = seeded()
+    w = synth.int4_weight(n, k, g)
+    x = synth.activations(m, k, g, outliers=True)
+    xq_ref, xs_ref = orc.quant_act_i8(G.bits(x))
+    gacc_ref, y_ref = orc.linear_w4a8(xq_ref, xs_ref, w.packed.numpy(), w.scale.numpy(), k, 128,
+                                      want_group_acc=True)
+    w4, ws = G.w4_repack(w.packed.to(G.DEV), w.scale.to(G.DEV), k)
+    gacc, y, xq, xs = G.gemv_w4a8_bf16(w4, ws, x.to(G.DEV), k)
+    assert (xq.cpu().numpy() == xq_ref).all()
+    assert (xs.cpu().numpy().view(np.uint32) == xs_ref.view(np.uint32)).all()
+    assert (gacc.cpu().numpy() == gacc_ref).all()
+    assert (G.bits(y) == y_ref).all()
+
+
+def test_gemv_w4a8_bf16_refuses_wide_batches():
+    g = seeded()
+    w = synth.int4_weight(256, 256, g)
+    w4, ws = G.w4_repack(w.packed.to(G.DEV), w.scale.to(G.DEV), 256)
+    with pytest.raises(ValueError):
+        G.gemv_w4a8_bf16(w4, ws, synth.activations(5, 256, g).to(G.DEV), 256)
+
+
 @pytest.mark.parametrize("m,n,k", [(128, 128, 128), (64, 256, 256), (512, 2560, 2560),
                                    (256, 1280, 5120), (100, 200, 384), (1, 1024, 2560),
                                    (16, 300, 2560)])

@@ -212,7 +212,7 @@ def _declared_symbols() -> list[str]:
 def test_library_exports_every_declared_symbol():
     lib = _native.load()
     names = _declared_symbols()
-    assert len(names) == 8
+    assert len(names) == 9
     for name in names:
         assert getattr(lib, name) is not None
     assert set(_native.SIGNATURES) | {"cmi_abi_version", "cmi_last_error"} == set(names)
