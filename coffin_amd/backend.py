@@ -47,8 +47,10 @@ GEMV_MAX_ROWS = 16
 PREFILL_MIN_ROWS = 64
 #: W4A8 switches from the GEMV to the MFMA GEMM above this many rows.
 W4_GEMM_MIN_ROWS = 17
-#: Up to this many rows the W4A8 GEMV quantises its activations itself (one launch).
-W4_FUSED_MAX_ROWS = 4
+#: Up to this many rows the W4A8 GEMV quantises its activations itself (one launch); the
+#: kernel takes up to 4, but from 2 rows on every workgroup redoing the divisions costs more
+#: than the separate quantiser launch.
+W4_FUSED_MAX_ROWS = 1
 
 _vp = ctypes.c_void_p
 

@@ -22,6 +22,12 @@ int check_launch(const char *what);
 int gemm_w8a8_generic(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws, void *y,
                       int32_t *acc_out, int M, int N, int K, int ldy, void *stream);
 
+// gemv_w4a8_decode.hip: W4A8 GEMV for 1..4 rows, K <= 10240, from bf16 activations (x) or
+// quantised ones (xq, xs); returns CMI_E_UNSUPPORTED (no error text) for other shapes.
+int gemv_w4a8_decode(const uint8_t *w4, const float *ws, const void *x, const int8_t *xq, const float *xs,
+                     void *y, int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
+                     void *stream);
+
 static inline bool aligned(const void *p, uintptr_t a) {
     return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
 }

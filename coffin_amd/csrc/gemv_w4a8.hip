@@ -342,6 +342,10 @@ extern "C" int cmi_gemv_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     CMI_REQUIRE(w4 && ws && xq && xs && y, CMI_E_ARG, "cmi_gemv_w4a8: null pointer");
     CMI_REQUIRE(aligned(w4, 16) && aligned(xq, 16), CMI_E_ARG,
                 "cmi_gemv_w4a8: w4 and xq must be 16-byte aligned");
+    if (gs == GS && N >= 1 && M >= 1) {
+        const int rc = gemv_w4a8_decode(w4, ws, nullptr, xq, xs, y, group_acc, nullptr, nullptr, M, N, K, stream);
+        if (rc != CMI_E_UNSUPPORTED) return rc;
+    }
     return run_gemv_w4a8("cmi_gemv_w4a8", w4, ws, xq, xs, nullptr, nullptr, nullptr, y, group_acc, M, N, K, gs,
                          stream);
 }
@@ -355,6 +359,12 @@ extern "C" int cmi_gemv_w4a8_bf16(const uint8_t *w4, const float *ws, const void
     CMI_REQUIRE(M >= 1 && M <= FUSED_MAX_ROWS, CMI_E_UNSUPPORTED,
                 "cmi_gemv_w4a8_bf16: M=%d outside 1..%d (quantise with cmi_quant_act_i8 and call cmi_gemv_w4a8)",
                 M, FUSED_MAX_ROWS);
+    CMI_REQUIRE(N >= 1 && K >= GS, CMI_E_ARG, "cmi_gemv_w4a8_bf16: bad shape N=%d K=%d", N, K);
+    CMI_REQUIRE(gs == GS, CMI_E_UNSUPPORTED, "cmi_gemv_w4a8_bf16: group size %d, kernels are built for %d", gs, GS);
+    CMI_REQUIRE(K % GS == 0, CMI_E_UNSUPPORTED, "cmi_gemv_w4a8_bf16: K=%d is not a multiple of %d", K, GS);
+    // the decode kernel (whole rows requested up front) where it applies, else the general one
+    const int rc = gemv_w4a8_decode(w4, ws, x, nullptr, nullptr, y, group_acc, xq_out, xs_out, M, N, K, stream);
+    if (rc != CMI_E_UNSUPPORTED) return rc;
     return run_gemv_w4a8("cmi_gemv_w4a8_bf16", w4, ws, nullptr, nullptr, x, xq_out, xs_out, y, group_acc, M, N, K,
                          gs, stream);
 }

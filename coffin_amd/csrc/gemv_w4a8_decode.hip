@@ -1,0 +1,327 @@
+// W4A8 decode GEMV: bf16 activations in, 1..4 rows, K <= 10240, one launch.
+//
+//   xq, xs  = per-token int8 quantisation of x (arithmetic of cmi_quant_act_i8)
+//   sum_g   = sum_{k in group g} xq[m,k] * (code(n,k) - 8)     int32, exact
+//   total   = fma((float)sum_g, ws[n,g], total)                 g = 0,1,.. from 0.f
+//   y[m,n]  = bf16(total * xs[m])
+//
+// HBM-bound on the packed weight (half a byte per element).  One wavefront owns
+// four weight rows, a quarter-wavefront (16 lanes x 16 B = 256 B per load) each,
+// and requests the whole of its rows before it does anything else, so memory
+// sees every byte of the launch in flight from the first microsecond; a
+// workgroup is four such wavefronts.  While the weights travel the workgroup
+// quantises the activations into LDS (every workgroup redoes this small job:
+// it saves a launch and the int8 round trip), together with -8 * sum(xq) per
+// 32-element chunk -- the start value of the v_dot4_i32_i8 accumulators, which
+// lets the unsigned codes be used without re-biasing -- and the per-group
+// scales of its 16 rows.  Four adjacent lanes own one group of 128 k; their
+// int32 partials are added with two DPP quad permutes and parked in LDS, where
+// one lane per (row, m) walks the groups in order: the fp32 chain is order
+// sensitive and must not depend on how K was spread over lanes.
+#include "quant_math.hpp"
+
+namespace {
+
+using namespace cmi;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int GS = 128;
+constexpr int ROWS_PER_WAVE = 4, WAVES = 4, ROWS_PER_BLOCK = ROWS_PER_WAVE * WAVES;
+constexpr int XV = 5;           // 16-byte bf16 vectors per thread and activation row: K <= 5*256*8
+constexpr int MAX_K = XV * 256 * 8;
+
+struct Args {
+    const uint8_t *w4;
+    const float *ws;
+    const uint16_t *x;   // bf16 activations (PREQ == false)
+    const int8_t *xq;    // quantised activations and their scales (PREQ == true)
+    const float *xs;
+    uint16_t *y;
+    int32_t *group_acc;
+    int8_t *xq_out;
+    float *xs_out;
+    int M, N, K, G;
+};
+
+// LDS carve-up (bytes); every part 16-byte aligned.
+struct Lds {
+    int xq, xsum, wsc, sums, xs, part, total;
+};
+__host__ __device__ inline Lds lds_layout(int mt, int K, bool ksplit) {
+    const int G = K / GS;
+    const int rows = ksplit ? ROWS_PER_WAVE : ROWS_PER_BLOCK;
+    Lds l;
+    l.xq = 0;
+    l.xsum = l.xq + mt * K;                           // int8 [mt][K]
+    l.wsc = l.xsum + mt * (K / 32) * 4;               // int32 [mt][K/32]
+    l.sums = l.wsc + ((rows * G * 4 + 15) & ~15);     // float [rows][G]
+    l.xs = l.sums + ((rows * G * mt * 4 + 15) & ~15); // int32 [rows/4][G][4][mt]
+    l.part = l.xs + 16 * 4;                           // float [mt] (padded to 16)
+    l.total = l.part + 16 * 4 * 4;                    // float [mt][4]
+    return l;
+}
+
+// M: activation-row tile (1, 2, 4).  NL: 256-byte loads per weight row and wavefront.
+// KSPLIT: the four wavefronts of a workgroup share four weight rows and take every fourth
+//         256-byte piece each (few, long rows: more workgroups, same bytes in flight);
+//         otherwise each wavefront owns four rows of its own.
+// PREQ:   activations arrive already quantised (a.xq, a.xs) instead of as bf16.
+template <int M, int NL, bool KSPLIT, bool PREQ>
+__global__ void __launch_bounds__(256)
+gemv_w4a8_decode_kernel(const Args a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    const Lds L = lds_layout(M, a.K, KSPLIT);
+    int8_t *xq_lds = reinterpret_cast<int8_t *>(lds + L.xq);
+    int32_t *xsum_lds = reinterpret_cast<int32_t *>(lds + L.xsum);
+    float *ws_lds = reinterpret_cast<float *>(lds + L.wsc);
+    int32_t *sums = reinterpret_cast<int32_t *>(lds + L.sums);
+    float *xs_lds = reinterpret_cast<float *>(lds + L.xs);
+    float *part = reinterpret_cast<float *>(lds + L.part);
+
+    constexpr int RPB = KSPLIT ? ROWS_PER_WAVE : ROWS_PER_BLOCK;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int q16 = lane & 15, r = lane >> 4;
+    const int n0 = blockIdx.x * RPB;
+    const int nrow = min(n0 + (KSPLIT ? 0 : wave * ROWS_PER_WAVE) + r, a.N - 1);
+    const int row_bytes = a.K / 2;
+    const int nchunks = a.K / 32;
+
+    // 1. activations first (memory answers in request order and they are needed first)
+    constexpr int XVN = PREQ ? 3 : XV;  // 16-byte vectors per thread and row
+    const int xvecs = PREQ ? a.K / 16 : a.K / 8;
+    uint4 v[M][XVN];
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+        const int mrow = m < a.M ? m : a.M - 1;
+        const uint4 *xg = PREQ ? reinterpret_cast<const uint4 *>(a.xq + (size_t)mrow * a.K)
+                               : reinterpret_cast<const uint4 *>(a.x + (size_t)mrow * a.K);
+#pragma unroll
+        for (int j = 0; j < XVN; ++j) {
+            const int idx = threadIdx.x + j * 256;
+            v[m][j] = idx < xvecs ? xg[idx] : make_uint4(0, 0, 0, 0);
+        }
+    }
+    // 2. the per-group scales of the workgroup's rows (contiguous in memory), into registers
+    // for now: they must not be waited for after the weights, which return in request order
+    constexpr int WSV = 5;  // floats per thread: 16 rows x G <= 16 x 80
+    const int ws_total = min(RPB, a.N - n0) * a.G;
+    float wsreg[WSV];
+    {
+        const float *src = a.ws + (size_t)n0 * a.G;
+#pragma unroll
+        for (int i = 0; i < WSV; ++i) {
+            const int idx = threadIdx.x + i * 256;
+            wsreg[i] = idx < ws_total ? src[idx] : 0.f;
+        }
+    }
+    // 3. every weight byte this wavefront is responsible for
+    const u32x4 *wrow = reinterpret_cast<const u32x4 *>(a.w4 + (size_t)nrow * row_bytes);
+    auto chunk_of = [&](int j) { return (KSPLIT ? j * 4 + wave : j) * 16 + q16; };  // 16-byte chunk = 32 k
+    u32x4 w[NL];
+#pragma unroll
+    for (int j = 0; j < NL; ++j) w[j] = __builtin_nontemporal_load(wrow + min(chunk_of(j), nchunks - 1));
+#pragma unroll
+    for (int i = 0; i < WSV; ++i) {
+        const int idx = threadIdx.x + i * 256;
+        if (idx < ws_total) ws_lds[idx] = wsreg[i];
+    }
+
+    // 4. int8 rows, their scales and -8 * (sum of each 32-element chunk) into LDS
+    if constexpr (PREQ) {
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            if (threadIdx.x == 0) xs_lds[m] = a.xs[m < a.M ? m : a.M - 1];
+#pragma unroll
+            for (int j = 0; j < XVN; ++j) {
+                if (j * 256 >= xvecs) break;  // uniform
+                const int idx = threadIdx.x + j * 256;
+                const uint4 q = v[m][j];
+                int s8 = __builtin_amdgcn_sdot4((int)q.x, 0x01010101, 0, false);
+                s8 = __builtin_amdgcn_sdot4((int)q.y, 0x01010101, s8, false);
+                s8 = __builtin_amdgcn_sdot4((int)q.z, 0x01010101, s8, false);
+                s8 = __builtin_amdgcn_sdot4((int)q.w, 0x01010101, s8, false);
+                s8 += dpp_i32<0xB1, 0xf>(s8);  // two consecutive vectors = one chunk
+                if (idx < xvecs) {
+                    reinterpret_cast<uint4 *>(xq_lds + (size_t)m * a.K)[idx] = q;
+                    if ((idx & 1) == 0) xsum_lds[m * nchunks + (idx >> 1)] = -8 * s8;
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            float amax = 0.f;
+#pragma unroll
+            for (int j = 0; j < XVN; ++j)
+                if (j * 256 < xvecs) amax = absmax8(v[m][j], amax);  // uniform: skip vectors past K
+            amax = wave_max_to_lane63(amax);
+            if (lane == 63) part[m * 4 + wave] = amax;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            const float amax =
+                fmaxf(fmaxf(part[m * 4], part[m * 4 + 1]), fmaxf(part[m * 4 + 2], part[m * 4 + 3]));
+            const float sc = quant_scale(amax);
+            if (threadIdx.x == 0) {
+                xs_lds[m] = sc;
+                if (a.xs_out && blockIdx.x == 0 && m < a.M) a.xs_out[m] = sc;
+            }
+#pragma unroll
+            for (int j = 0; j < XVN; ++j) {
+                if (j * 256 >= xvecs) break;  // uniform
+                const int idx = threadIdx.x + j * 256;
+                const uint2 q = quant8(v[m][j], sc);
+                // four consecutive vectors (adjacent lanes) = one chunk
+                int s8 = __builtin_amdgcn_sdot4((int)q.x, 0x01010101, 0, false);
+                s8 = __builtin_amdgcn_sdot4((int)q.y, 0x01010101, s8, false);
+                s8 += dpp_i32<0xB1, 0xf>(s8);  // quad_perm [1,0,3,2]
+                s8 += dpp_i32<0x4E, 0xf>(s8);  // quad_perm [2,3,0,1]
+                if (idx < xvecs) {
+                    reinterpret_cast<uint2 *>(xq_lds + (size_t)m * a.K)[idx] = q;
+                    if ((idx & 3) == 0) xsum_lds[m * nchunks + (idx >> 2)] = -8 * s8;
+                    if (a.xq_out && blockIdx.x == 0 && m < a.M)
+                        reinterpret_cast<uint2 *>(a.xq_out + (size_t)m * a.K)[idx] = q;
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    // 5. integer group sums
+    int32_t *wsums = sums + (KSPLIT ? 0 : wave * (a.G * ROWS_PER_WAVE * M));
+#pragma unroll
+    for (int j = 0; j < NL; ++j) {
+        if ((KSPLIT ? j * 4 + wave : j) * 16 >= nchunks) break;  // uniform per wavefront
+        const int c = chunk_of(j);
+        const bool live = c < nchunks;
+        const int cs = live ? c : nchunks - 1;
+        const uint32_t ww[4] = {w[j].x, w[j].y, w[j].z, w[j].w};
+        uint32_t op[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            op[2 * i] = ww[i] & 0x0F0F0F0Fu;
+            op[2 * i + 1] = (ww[i] >> 4) & 0x0F0F0F0Fu;
+        }
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            const uint4 *xp = reinterpret_cast<const uint4 *>(xq_lds + (size_t)m * a.K) + 2 * cs;
+            const uint4 x0 = xp[0], x1 = xp[1];
+            const uint32_t xv[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+            int acc = xsum_lds[m * nchunks + cs];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc = __builtin_amdgcn_sdot4((int)op[i], (int)xv[i], acc, false);
+            acc += dpp_i32<0xB1, 0xf>(acc);
+            acc += dpp_i32<0x4E, 0xf>(acc);
+            if ((lane & 3) == 0 && live) wsums[((c >> 2) * ROWS_PER_WAVE + r) * M + m] = acc;
+        }
+    }
+    if constexpr (KSPLIT) {
+        __syncthreads();
+        if (wave != 0) return;
+    } else {
+        // the group sums below were written by this wavefront itself
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+    }
+
+    // 6. fp32 chain over the groups, one lane per (row, m)
+    if (lane < ROWS_PER_WAVE * M) {
+        const int rr = lane / M, m = lane - rr * M;
+        const int brow = (KSPLIT ? 0 : wave * ROWS_PER_WAVE) + rr;  // row within the workgroup
+        const int n = n0 + brow;
+        if (n < a.N && m < a.M) {
+            const float *wsn = ws_lds + brow * a.G;
+            float total = 0.f;
+            // four groups at a time: the eight LDS reads go out together, the fmas stay in order
+            int g = 0;
+            for (; g + 4 <= a.G; g += 4) {
+                int sv[4];
+                float wv[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    sv[i] = wsums[((g + i) * ROWS_PER_WAVE + rr) * M + m];
+                    wv[i] = wsn[g + i];
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if (a.group_acc) a.group_acc[((size_t)m * a.G + g + i) * a.N + n] = sv[i];
+                    total = fmaf((float)sv[i], wv[i], total);
+                }
+            }
+            for (; g < a.G; ++g) {
+                const int sg = wsums[(g * ROWS_PER_WAVE + rr) * M + m];
+                if (a.group_acc) a.group_acc[((size_t)m * a.G + g) * a.N + n] = sg;
+                total = fmaf((float)sg, wsn[g], total);
+            }
+            a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * xs_lds[m]);
+        }
+    }
+}
+
+template <int M, int NL, bool KSPLIT, bool PREQ>
+int launch(const Args &a, hipStream_t st) {
+    const Lds L = lds_layout(M, a.K, KSPLIT);
+    if (L.total > 64 * 1024) return CMI_E_UNSUPPORTED;
+    constexpr int RPB = KSPLIT ? ROWS_PER_WAVE : ROWS_PER_BLOCK;
+    const dim3 grid((a.N + RPB - 1) / RPB);
+    gemv_w4a8_decode_kernel<M, NL, KSPLIT, PREQ><<<grid, dim3(256), L.total, st>>>(a);
+    return check_launch("cmi_gemv_w4a8");
+}
+
+template <int M, bool PREQ>
+int dispatch(const Args &a, hipStream_t st) {
+    const int pieces = (a.K + 511) / 512;  // 256-byte pieces per weight row
+    // few rows: share each row among the four wavefronts so that the grid still covers the chip
+    const bool ksplit = (a.N + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK < 512 && pieces >= 4;
+    if (ksplit) {
+        const int nl = (pieces + 3) / 4;
+        if (nl <= 2) return launch<M, 2, true, PREQ>(a, st);
+        if (nl <= 5) return launch<M, 5, true, PREQ>(a, st);
+        return CMI_E_UNSUPPORTED;
+    }
+    if (pieces <= 5) return launch<M, 5, false, PREQ>(a, st);
+    if (pieces <= 8) return launch<M, 8, false, PREQ>(a, st);
+    if (pieces <= 10) return launch<M, 10, false, PREQ>(a, st);
+    if (pieces <= 20) return launch<M, 20, false, PREQ>(a, st);
+    return CMI_E_UNSUPPORTED;
+}
+
+}  // namespace
+
+namespace cmi {
+
+// Exactly one of x (bf16) and xq/xs (already quantised) is given.  Returns
+// CMI_E_UNSUPPORTED without setting the error text when the shape is outside
+// this kernel's range (the caller then uses the general kernel).
+int gemv_w4a8_decode(const uint8_t *w4, const float *ws, const void *x, const int8_t *xq, const float *xs,
+                     void *y, int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
+                     void *stream) {
+    if (M < 1 || M > 4 || K < GS || K > MAX_K || K % GS != 0 || N < 1) return CMI_E_UNSUPPORTED;
+    Args a;
+    a.w4 = w4;
+    a.ws = ws;
+    a.x = static_cast<const uint16_t *>(x);
+    a.xq = xq;
+    a.xs = xs;
+    a.y = static_cast<uint16_t *>(y);
+    a.group_acc = group_acc;
+    a.xq_out = xq_out;
+    a.xs_out = xs_out;
+    a.M = M;
+    a.N = N;
+    a.K = K;
+    a.G = K / GS;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (x) {
+        if (M <= 1) return dispatch<1, false>(a, st);
+        if (M <= 2) return dispatch<2, false>(a, st);
+        return dispatch<4, false>(a, st);
+    }
+    if (M <= 1) return dispatch<1, true>(a, st);
+    if (M <= 2) return dispatch<2, true>(a, st);
+    return dispatch<4, true>(a, st);
+}
+
+}  // namespace cmi
