@@ -319,28 +319,3 @@ int cmi::gemm_w8a8_generic(const int8_t *xq, const int8_t *wq, const float *xs, 
     a.G = 1;
     return launch<false>(a, static_cast<hipStream_t>(stream), "cmi_gemm_w8a8");
 }
-
-extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs,
-                             void *y, int32_t *group_acc, int M, int N, int K, int gs,
-                             void *stream) {
-    CMI_REQUIRE(M >= 0 && N >= 1 && K >= BK, CMI_E_ARG, "cmi_gemm_w4a8: bad shape M=%d N=%d K=%d", M, N, K);
-    if (M == 0) return CMI_OK;  // an empty batch has no storage to point at
-    CMI_REQUIRE(w4 && ws && xq && xs && y, CMI_E_ARG, "cmi_gemm_w4a8: null pointer");
-    CMI_REQUIRE(gs == BK, CMI_E_UNSUPPORTED, "cmi_gemm_w4a8: group size %d, kernels are built for %d", gs, BK);
-    CMI_REQUIRE(K % BK == 0, CMI_E_UNSUPPORTED, "cmi_gemm_w4a8: K=%d is not a multiple of %d", K, BK);
-    CMI_REQUIRE(aligned(xq, 16) && aligned(w4, 16), CMI_E_ARG,
-                "cmi_gemm_w4a8: xq and w4 must be 16-byte aligned");
-    GemmArgs a;
-    a.xq = xq;
-    a.w = w4;
-    a.xs = xs;
-    a.ws = ws;
-    a.y = static_cast<uint16_t *>(y);
-    a.acc_out = group_acc;
-    a.M = M;
-    a.N = N;
-    a.K = K;
-    a.ldy = N;
-    a.G = K / BK;
-    return launch<true>(a, static_cast<hipStream_t>(stream), "cmi_gemm_w4a8");
-}

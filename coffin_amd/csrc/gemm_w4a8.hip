@@ -1,0 +1,329 @@
+// W4A8 prefill GEMM for CDNA4 int8 MFMA on the re-laid-out int4 weight (group size 128).
+//
+//   sum_g  = sum_{k in group g} xq[m,k] * (code(n,k) - 8)     int32, exact
+//   total  = fma((float)sum_g, ws[n,g], total)                 g = 0,1,.. from 0.f
+//   y[m,n] = bf16(total * xs[m])
+//
+// Same bits as the W4A8 GEMV for every m: the integer part is exact and the
+// fp32 part is the one chain over the groups in ascending order.
+//
+// Block tile 128(m) x 128(n), 4 wavefronts (2 x 2) of 64 x 64, v_mfma_i32_32x32x32_i8,
+// K walked one scale group (128) per step, two LDS stages, two workgroups per CU.
+//   - activations go global -> LDS directly (global_load_lds_dwordx4, chunk
+//     index XOR-swizzled on the global side, as in the W8A8 kernel);
+//   - the packed weight (64 B per row and step) is fetched into registers one
+//     step ahead, widened there to int8 code-8 (no cross-byte borrow), and
+//     written to LDS once per workgroup, so the inner loop is the int8 one;
+//   - the activation is the MFMA row operand and the weight the column operand:
+//     a lane then owns ONE n per MFMA tile (and 16 m), so the per-group flush
+//     total = fma((float)sum, ws[n,g], total) needs one scale per tile and lane,
+//     fetched from memory a step ahead;
+//   - the integer accumulators restart every step (first MFMA of a group takes
+//     C = 0); the flush is 64 converts + 64 fmas per lane and step, which is why
+//     two workgroups share a CU: one flushes while the other multiplies.
+#include "common.hpp"
+
+#include <type_traits>
+
+namespace {
+
+using namespace cmi;
+
+constexpr int BM = 128, BN = 128, BK = 128;  // BK = the scale group
+constexpr int THREADS = 256;
+constexpr int X_BYTES = BM * BK, W_BYTES = BN * BK;  // int8 in LDS
+constexpr int STAGE_BYTES = X_BYTES + W_BYTES;
+constexpr int LDS_BYTES = 2 * STAGE_BYTES;           // 64 KiB
+
+struct Args {
+    const int8_t *xq;
+    const uint8_t *w4;
+    const float *xs;
+    const float *ws;  // [N, G]
+    uint16_t *y;
+    int32_t *group_acc;  // [M, G, N], nullable
+    int M, N, K, G;
+    int tiles_m, tiles_n;
+};
+
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+
+// Four codes (0..15, one per byte) -> four int8 (code - 8), no cross-byte borrow.
+__device__ __forceinline__ uint32_t rebias4(uint32_t c) {
+    return ((c | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
+}
+
+// DUMP: also write the int32 group sums (parity checks); a separate instantiation, the
+// 64 extra store addresses per lane would otherwise be carried through the hot loop.
+template <bool DUMP>
+__global__ void __launch_bounds__(THREADS, 2)
+gemm_w4a8_kernel(const Args a) {
+    extern __shared__ __align__(16) int8_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wn = wave & 1, wm = wave >> 1;
+
+    // banded tile order per XCD (see the W8A8 kernel)
+    int tm, tn;
+    {
+        constexpr int GM = 8;
+        const int total = a.tiles_m * a.tiles_n;
+        int t = blockIdx.x;
+        if (total % 8 == 0) t = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
+        const int width = GM * a.tiles_n;
+        const int band = t / width, in_band = t - band * width;
+        const int first_m = band * GM;
+        const int rows = min(a.tiles_m - first_m, GM);
+        tn = in_band / rows;
+        tm = first_m + (in_band - tn * rows);
+    }
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    // activations: direct loads, wavefront w fills rows 32w..32w+31 (4 loads of 8 rows x 128 B)
+    const int lrow = lane >> 3;
+    const int8_t *xsrc[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const int row = (4 * wave + g) * 8 + lrow;
+        const int kc = (lane & 7) ^ ((row >> 1) & 7);
+        xsrc[g] = a.xq + (size_t)min(m0 + row, a.M - 1) * a.K + kc * 16;
+    }
+    auto issue_x = [&](int stage, int ks) {
+        int8_t *base = lds + stage * STAGE_BYTES + (4 * wave) * 1024;
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+            __builtin_amdgcn_global_load_lds((const void *)(xsrc[g] + ks * BK), (lds_ptr_t)(base + g * 1024), 16, 0, 0);
+    };
+
+    // packed weight: 128 rows x 64 B per step = 512 x 16 B, two per thread; thread t takes
+    // 16-byte piece (t%4) of rows t/4 and t/4 + 64.  A piece holds 32 k: LDS chunks 2p, 2p+1.
+    const int wr = threadIdx.x >> 2, wp = threadIdx.x & 3;
+    const uint8_t *wsrc[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+        wsrc[h] = a.w4 + (size_t)min(n0 + wr + 64 * h, a.N - 1) * (a.K / 2) + wp * 16;
+    auto fetch_w = [&](uint4 (&reg)[2], int ks) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) reg[h] = *reinterpret_cast<const uint4 *>(wsrc[h] + ks * (BK / 2));
+    };
+    auto stash_w = [&](int stage, const uint4 (&reg)[2]) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int row = wr + 64 * h;
+            const uint32_t w[4] = {reg[h].x, reg[h].y, reg[h].z, reg[h].w};
+            uint4 lo, hi;  // k 0..15 and 16..31 of the piece
+            lo.x = rebias4(w[0] & 0x0F0F0F0Fu);
+            lo.y = rebias4((w[0] >> 4) & 0x0F0F0F0Fu);
+            lo.z = rebias4(w[1] & 0x0F0F0F0Fu);
+            lo.w = rebias4((w[1] >> 4) & 0x0F0F0F0Fu);
+            hi.x = rebias4(w[2] & 0x0F0F0F0Fu);
+            hi.y = rebias4((w[2] >> 4) & 0x0F0F0F0Fu);
+            hi.z = rebias4(w[3] & 0x0F0F0F0Fu);
+            hi.w = rebias4((w[3] >> 4) & 0x0F0F0F0Fu);
+            int8_t *dst = lds + stage * STAGE_BYTES + X_BYTES + row * BK;
+            const int sw = (row >> 1) & 7;
+            *reinterpret_cast<uint4 *>(dst + ((2 * wp) ^ sw) * 16) = lo;
+            *reinterpret_cast<uint4 *>(dst + ((2 * wp + 1) ^ sw) * 16) = hi;
+        }
+    };
+
+    // group scales of this lane's two n (one per MFMA column tile)
+    const float *wsp[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+        wsp[j] = a.ws + (size_t)min(n0 + wn * 64 + j * 32 + (lane & 31), a.N - 1) * a.G;
+
+    // fragments: lane reads row (lane%32) of a 32-row tile; k quarter q -> chunk 2q + lane/32
+    const int frow = lane & 31;
+    const int fsw = (frow >> 1) & 7;
+    int foff[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) foff[q] = frow * BK + ((2 * q + (lane >> 5)) ^ fsw) * 16;
+    struct Frag {
+        v4i32 x[2], w[2];
+    };
+    auto read_q = [&](int stage, int q, Frag &f) {
+        const int8_t *xt = lds + stage * STAGE_BYTES + wm * 64 * BK + foff[q];
+        const int8_t *wt = lds + stage * STAGE_BYTES + X_BYTES + wn * 64 * BK + foff[q];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            f.x[t] = *reinterpret_cast<const v4i32 *>(xt + t * 32 * BK);
+            f.w[t] = *reinterpret_cast<const v4i32 *>(wt + t * 32 * BK);
+        }
+    };
+
+    float total[2][2][16];  // [m tile][n tile][element]
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) total[i][j][v] = 0.f;
+
+    const int ksteps = a.K / BK;
+    const int mb = m0 + wm * 64, nb = n0 + wn * 64;
+    v16i32 acc[2][2];
+    auto mma_q = [&](const Frag &f, bool first) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                if (first) {
+                    const v16i32 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.x[i], f.w[j], zero, 0, 0, 0);
+                } else {
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.x[i], f.w[j], acc[i][j], 0, 0, 0);
+                }
+            }
+    };
+
+    // One group.  Its first-quarter fragments are in f0; stage ks%2 holds its operands.  After
+    // the third quarter's reads the stage is free: the activations of step ks+1 have landed in
+    // the other stage (requested a step ago), this wavefront's share of the weights of step
+    // ks+1 (in registers since a step ago) is widened into it, and behind the barrier the
+    // requests for step ks+2 go out while the last quarter multiplies.
+    Frag f0, f1;
+    uint4 wreg[2];
+    float sc[2];
+    auto step = [&](auto more_tag, int ks) {
+        constexpr bool MORE = decltype(more_tag)::value;  // a step ks+2 exists
+        const int cur = ks & 1;
+        // four MFMAs with the four fragment reads of the next quarter spread between them
+        auto pace_quarter = [&]() {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+        };
+        read_q(cur, 1, f1);
+        mma_q(f0, true);
+        pace_quarter();
+        read_q(cur, 2, f0);
+        mma_q(f1, false);
+        pace_quarter();
+        read_q(cur, 3, f1);
+        mma_q(f0, false);
+        pace_quarter();
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        if (ks + 1 < ksteps) stash_w(cur ^ 1, wreg);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        float sc_next[2] = {0.f, 0.f};
+        if constexpr (MORE) {
+            issue_x(cur, ks + 2);
+            fetch_w(wreg, ks + 2);
+        }
+        if (ks + 1 < ksteps) {
+            sc_next[0] = wsp[0][ks + 1];
+            sc_next[1] = wsp[1][ks + 1];
+        }
+        read_q(cur ^ 1, 0, f0);  // past the last step: a stale stage nobody uses
+        mma_q(f1, false);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (MORE) __builtin_amdgcn_sched_group_barrier(0x010, 2, 0);  // requests for step ks+2
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        if constexpr (DUMP) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int n = nb + j * 32 + (lane & 31);
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int m = mb + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                        if (m < a.M && n < a.N) a.group_acc[((size_t)m * a.G + ks) * a.N + n] = acc[i][j][v];
+                    }
+                }
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) total[i][j][v] = fmaf((float)acc[i][j][v], sc[j], total[i][j][v]);
+        sc[0] = sc_next[0];
+        sc[1] = sc_next[1];
+    };
+    using more_t = std::integral_constant<bool, true>;
+    using last_t = std::integral_constant<bool, false>;
+
+    // prologue: stage 0 complete (activations direct, weights through registers), step 1 on its way
+    issue_x(0, 0);
+    fetch_w(wreg, 0);
+    sc[0] = wsp[0][0];
+    sc[1] = wsp[1][0];
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    stash_w(0, wreg);
+    if (ksteps > 1) {
+        issue_x(1, 1);
+        fetch_w(wreg, 1);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    read_q(0, 0, f0);
+    int ks = 0;
+    for (; ks + 2 < ksteps; ++ks) step(more_t{}, ks);
+    for (; ks < ksteps; ++ks) step(last_t{}, ks);
+
+    // y[m,n] = bf16(total * xs[m]); a lane holds one n per tile: 32 lanes write 64 contiguous bytes
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int m = mb + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+            if (m >= a.M) continue;
+            const float xm = a.xs[m];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int n = nb + j * 32 + (lane & 31);
+                if (n < a.N) a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total[i][j][v] * xm);
+            }
+        }
+}
+
+}  // namespace
+
+extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs,
+                             void *y, int32_t *group_acc, int M, int N, int K, int gs,
+                             void *stream) {
+    CMI_REQUIRE(M >= 0 && N >= 1 && K >= BK, CMI_E_ARG, "cmi_gemm_w4a8: bad shape M=%d N=%d K=%d", M, N, K);
+    if (M == 0) return CMI_OK;  // an empty batch has no storage to point at
+    CMI_REQUIRE(w4 && ws && xq && xs && y, CMI_E_ARG, "cmi_gemm_w4a8: null pointer");
+    CMI_REQUIRE(gs == BK, CMI_E_UNSUPPORTED, "cmi_gemm_w4a8: group size %d, kernels are built for %d", gs, BK);
+    CMI_REQUIRE(K % BK == 0, CMI_E_UNSUPPORTED, "cmi_gemm_w4a8: K=%d is not a multiple of %d", K, BK);
+    CMI_REQUIRE(aligned(xq, 16) && aligned(w4, 16), CMI_E_ARG,
+                "cmi_gemm_w4a8: xq and w4 must be 16-byte aligned");
+    Args a;
+    a.xq = xq;
+    a.w4 = w4;
+    a.xs = xs;
+    a.ws = ws;
+    a.y = static_cast<uint16_t *>(y);
+    a.group_acc = group_acc;
+    a.M = M;
+    a.N = N;
+    a.K = K;
+    a.G = K / BK;
+    a.tiles_m = (M + BM - 1) / BM;
+    a.tiles_n = (N + BN - 1) / BN;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w4a8_kernel<false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess ||
+            hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w4a8_kernel<true>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
+            return fail(CMI_E_HIP, "cmi_gemm_w4a8: cannot reserve %d bytes of LDS", LDS_BYTES);
+        configured = true;
+    }
+    const dim3 grid(a.tiles_m * a.tiles_n), block(THREADS);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (group_acc) gemm_w4a8_kernel<true><<<grid, block, LDS_BYTES, st>>>(a);
+    else gemm_w4a8_kernel<false><<<grid, block, LDS_BYTES, st>>>(a);
+    return check_launch("cmi_gemm_w4a8");
+}
