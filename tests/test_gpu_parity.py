@@ -81,7 +81,8 @@ def _w8a16_case(orc, m, n, k, g):
 @pytest.mark.parametrize("m,n,k", [(1, 9728, 2560), (1, 2560, 9728), (4, 4096, 2560),
                                    (8, 1024, 2560), (16, 2560, 4096), (3, 1000, 4112),
                                    (1, 128, 16), (2, 6144, 2560), (16, 1024, 2560),
-                                   (5, 333, 2560), (11, 77, 1040), (1, 640, 25600)])
+                                   (5, 333, 2560), (11, 77, 1040), (1, 640, 25600), (8, 512, 5120),
+                                   (16, 300, 7168), (4, 96, 9728), (12, 640, 3088)])
 def test_gemv_w8a16_within_tolerance(orc, m, n, k):
     wq, ws, x, y = _w8a16_case(orc, m, n, k, seeded())
     got = y.float().cpu().numpy()
@@ -104,7 +105,7 @@ def test_gemv_w8a16_golden(golden):
     assert (np.abs(got - g["y_ref"]) <= WEIGHT_ONLY_TOL_RMS * rms + np.abs(g["y_ref"]) * 2.0 ** -7).all()
 
 
-@pytest.mark.parametrize("n,k", [(4096, 2560), (2560, 9728), (1000, 4112)])
+@pytest.mark.parametrize("n,k", [(4096, 2560), (2560, 9728), (1000, 4112), (512, 5120), (300, 7168)])
 def test_gemv_w8a16_batched_row_equals_single_row(n, k):
     g = seeded()
     q = synth.int8_weight(n, k, g)
@@ -226,7 +227,8 @@ def _w4_case(orc, m, n, k, g):
 
 @pytest.mark.parametrize("m,n,k", [(1, 9728, 2560), (1, 2560, 9728), (4, 512, 256),
                                    (16, 2560, 9728), (16, 1024, 2560), (2, 333, 1280),
-                                   (8, 4096, 2560), (1, 640, 25600), (3, 7, 128)])
+                                   (8, 4096, 2560), (1, 640, 25600), (3, 7, 128), (4, 2560, 4096),
+                                   (2, 9728, 2560), (1, 300, 10240)])
 def test_gemv_w4a8_bit_exact(orc, m, n, k):
     w4, ws, xq, xs, gacc_ref, y_ref = _w4_case(orc, m, n, k, seeded())
     gacc, y = G.w4a8(w4, ws, xq, xs, k, gemm=False)
@@ -238,7 +240,7 @@ def test_gemv_w4a8_bit_exact(orc, m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(1, 9728, 2560), (1, 2560, 9728), (4, 512, 256), (2, 333, 1280),
                                    (3, 7, 128), (4, 6144, 2560), (1, 2560, 4096), (4, 2560, 9728),
-                                   (2, 640, 16384)])
+                                   (2, 640, 16384), (1, 256, 10240), (3, 100, 7680), (4, 8200, 128)])
 def test_gemv_w4a8_bf16_fused_quantiser_bit_exact(orc, m, n, k):
     """One launch from bf16 activations: the quantised rows, the scales, the group
     sums and the output all carry the bits of quantiser + GEMV run separately."""
