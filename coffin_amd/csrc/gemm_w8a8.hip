@@ -76,6 +76,7 @@ __device__ __forceinline__ void wait_vmcnt() {
     else if constexpr (N == 4) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 6) asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+    else if constexpr (N == 9) asm volatile("s_waitcnt vmcnt(9) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 12) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 16) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 18) asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)" ::: "memory");
@@ -119,7 +120,8 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 // Scale, narrow, park the wavefront's bf16 tile in LDS (row = m), then write
 // rows back 16 bytes per lane.  Every wavefront of the workgroup must call it
 // (one barrier inside: the operand stages are reused as parking space).
-template <int TN, int TM>
+// JP: m tiles parked per pass (the parking space of a wavefront is 32*JP rows); TM % JP == 0.
+template <int TN, int TM, int JP = TM>
 __device__ __forceinline__ void epilogue(const Args &a, v16i32 (&acc)[TN][TM], int8_t *lds, int wave,
                                          int lane, int nb, int mb) {
     if (a.acc_out) {
@@ -139,7 +141,7 @@ __device__ __forceinline__ void epilogue(const Args &a, v16i32 (&acc)[TN][TM], i
     __builtin_amdgcn_s_barrier();  // every wavefront is done reading operand stages
     asm volatile("" ::: "memory");
     constexpr int PITCH = 64 * TN + 16;  // one m row of the wavefront tile + 16 B
-    int8_t *park = lds + wave * (32 * TM * PITCH);
+    int8_t *park = lds + wave * (32 * JP * PITCH);
     // per-column scales of this lane's columns: 4 consecutive n per (i, q)
     float wsv[TN][4][4];
 #pragma unroll
@@ -156,44 +158,49 @@ __device__ __forceinline__ void epilogue(const Args &a, v16i32 (&acc)[TN][TM], i
                 for (int r = 0; r < 4; ++r) wsv[i][q][r] = a.ws[min(n + r, a.N - 1)];
             }
         }
-#pragma unroll
-    for (int j = 0; j < TM; ++j) {
-        const int ml = j * 32 + (lane & 31);
-        const float xm = a.xs[min(mb + ml, a.M - 1)];
-#pragma unroll
-        for (int i = 0; i < TN; ++i)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int nl = i * 32 + 8 * q + 4 * (lane >> 5);
-                float t[4];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) t[r] = ((float)acc[i][j][4 * q + r] * xm) * wsv[i][q][r];
-                uint2 pk;
-                pk.x = pack_bf16(t[0], t[1]);
-                pk.y = pack_bf16(t[2], t[3]);
-                *reinterpret_cast<uint2 *>(park + ml * PITCH + nl * 2) = pk;
-            }
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own tile only: no barrier needed
     const bool vec_ok = (a.ldy % 8 == 0) && ((reinterpret_cast<uintptr_t>(a.y) & 15) == 0);
-    constexpr int CPR = 4 * TN;        // 16-byte chunks per row of the wavefront tile
-    constexpr int RPP = 64 / CPR;      // rows per pass
+    constexpr int CPR = 4 * TN;  // 16-byte chunks per row of the wavefront tile
 #pragma unroll
-    for (int p = 0; p < 32 * TM / RPP; ++p) {
-        const int ml = p * RPP + lane / CPR, c = lane % CPR;
-        const int m = mb + ml;
-        const int n = nb + c * 8;
-        if (m >= a.M || n >= a.N) continue;
-        const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * PITCH + c * 16);
-        uint16_t *dst = a.y + (size_t)m * a.ldy + n;
-        if (vec_ok && n + 7 < a.N) {
-            *reinterpret_cast<uint4 *>(dst) = v;
-        } else {
-            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    for (int j0 = 0; j0 < TM; j0 += JP) {
 #pragma unroll
-            for (int r = 0; r < 8; ++r)
-                if (n + r < a.N) dst[r] = (uint16_t)(w[r >> 1] >> ((r & 1) * 16));
+        for (int jj = 0; jj < JP; ++jj) {
+            const int j = j0 + jj;
+            const int ml = jj * 32 + (lane & 31);
+            const float xm = a.xs[min(mb + j * 32 + (lane & 31), a.M - 1)];
+#pragma unroll
+            for (int i = 0; i < TN; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int nl = i * 32 + 8 * q + 4 * (lane >> 5);
+                    float t[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) t[r] = ((float)acc[i][j][4 * q + r] * xm) * wsv[i][q][r];
+                    uint2 pk;
+                    pk.x = pack_bf16(t[0], t[1]);
+                    pk.y = pack_bf16(t[2], t[3]);
+                    *reinterpret_cast<uint2 *>(park + ml * PITCH + nl * 2) = pk;
+                }
         }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own tile only: no barrier needed
+#pragma unroll
+        for (int p = 0; p < (32 * JP * CPR + 63) / 64; ++p) {
+            const int idx = p * 64 + lane;
+            const int ml = idx / CPR, c = idx - ml * CPR;
+            const int m = mb + j0 * 32 + ml;
+            const int n = nb + c * 8;
+            if (ml >= 32 * JP || m >= a.M || n >= a.N) continue;
+            const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * PITCH + c * 16);
+            uint16_t *dst = a.y + (size_t)m * a.ldy + n;
+            if (vec_ok && n + 7 < a.N) {
+                *reinterpret_cast<uint4 *>(dst) = v;
+            } else {
+                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int r = 0; r < 8; ++r)
+                    if (n + r < a.N) dst[r] = (uint16_t)(w[r >> 1] >> ((r & 1) * 16));
+            }
+        }
+        if (j0 + JP < TM) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // reads done before the next pass parks
     }
 }
 
@@ -539,6 +546,171 @@ int launch_big(Args &a, hipStream_t st) {
     return check_launch("cmi_gemm_w8a8");
 }
 
+// ---------------------------------------------------------------------------
+// 256(m) x 320(n) block tile, 8 wavefronts (2 along n x 4 along m, two per SIMD) of
+// 64(m) x 160(n) = 2 x 5 MFMA tiles, 160 accumulator registers per lane.  Exists
+// for the tile count: N = 9728 (Qwen3.5-4B's MLP width) is 38 x 256 but 30.4 x 320, so
+// 2048 x 9728 is 248 of these tiles -- one round of the 256 CUs -- instead of 304 tiles of
+// 256 x 256 (1.19 rounds).  It also needs the fewest L2 -> LDS bytes per MFMA of the three
+// kernels.  Two LDS stages of 72 KiB, fragments double-buffered per k quarter, one barrier
+// per step (structure of the 256 x 256 kernel without the slot ring).
+namespace wide {
+constexpr int BM = 256, BN = 320, TN = 5, TM = 2;
+constexpr int W_BYTES = BN * BK, X_BYTES = BM * BK, STAGE_BYTES = W_BYTES + X_BYTES;
+constexpr int PARK_BYTES = 8 * 32 * (64 * TN + 16);  // one m tile per epilogue pass
+constexpr int LDS_BYTES = 2 * STAGE_BYTES > PARK_BYTES ? 2 * STAGE_BYTES : PARK_BYTES;
+constexpr int WL = 5, XL = 4;  // loads per wavefront and stage
+}  // namespace wide
+
+__global__ void __launch_bounds__(512, 2)
+gemm_w8a8_wide_kernel(const Args a) {
+    using namespace wide;
+    extern __shared__ __align__(16) int8_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wn = wave & 1, wm = wave >> 1;
+
+    int tm, tn;
+    tile_coords(a, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    // Wavefront w fills W rows 40w .. 40w+39 and X rows 32w .. 32w+31 (8 rows x 128 B per load).
+    // Addresses are a uniform base (tile corner, advanced by the k step) plus a 32-bit lane
+    // offset: 9 registers instead of 18 for 64-bit pointers, which this kernel cannot spare.
+    const int lrow = lane >> 3;
+    uint32_t woff[WL], xoff[XL];
+#pragma unroll
+    for (int g = 0; g < WL; ++g) {
+        const int row = (WL * wave + g) * 8 + lrow;
+        const int kc = (lane & 7) ^ ((row >> 1) & 7);
+        woff[g] = (uint32_t)min(row, a.N - 1 - n0) * (uint32_t)a.K + kc * 16;
+    }
+#pragma unroll
+    for (int g = 0; g < XL; ++g) {
+        const int row = (XL * wave + g) * 8 + lrow;
+        const int kc = (lane & 7) ^ ((row >> 1) & 7);
+        xoff[g] = (uint32_t)min(row, a.M - 1 - m0) * (uint32_t)a.K + kc * 16;
+    }
+    const int8_t *wtile = a.wq + (size_t)n0 * a.K, *xtile = a.xq + (size_t)m0 * a.K;
+    auto issue = [&](int stage, int ks) {
+        int8_t *base = lds + stage * STAGE_BYTES;
+        const int8_t *wk = wtile + ks * BK, *xk = xtile + ks * BK;
+#pragma unroll
+        for (int g = 0; g < WL; ++g)
+            __builtin_amdgcn_global_load_lds((const void *)(wk + woff[g]),
+                                             (lds_ptr_t)(base + (WL * wave + g) * 1024), 16, 0, 0);
+#pragma unroll
+        for (int g = 0; g < XL; ++g)
+            __builtin_amdgcn_global_load_lds((const void *)(xk + xoff[g]),
+                                             (lds_ptr_t)(base + W_BYTES + (XL * wave + g) * 1024), 16, 0, 0);
+    };
+
+    const int frow = lane & 31;
+    const int fsw = (frow >> 1) & 7;
+    int foff[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) foff[q] = frow * BK + ((2 * q + (lane >> 5)) ^ fsw) * 16;
+    struct Frag {
+        v4i32 w[TN], x[TM];
+    };
+    auto read_q = [&](int stage, int q, Frag &f) {
+        const int8_t *wt = lds + stage * STAGE_BYTES + wn * 32 * TN * BK + foff[q];
+        const int8_t *xt = lds + stage * STAGE_BYTES + W_BYTES + wm * 32 * TM * BK + foff[q];
+#pragma unroll
+        for (int t = 0; t < TN; ++t) f.w[t] = *reinterpret_cast<const v4i32 *>(wt + t * 32 * BK);
+#pragma unroll
+        for (int t = 0; t < TM; ++t) f.x[t] = *reinterpret_cast<const v4i32 *>(xt + t * 32 * BK);
+    };
+
+    v16i32 acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+    auto mma_q = [&](const Frag &f) {
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w[i], f.x[j], acc[i][j], 0, 0, 0);
+    };
+    constexpr int N_MMA = TN * TM, N_DS = TN + TM;
+    // a quarter's MFMAs with the fragment reads of the next quarter spread between them
+    auto pace_quarter = [&]() {
+#pragma unroll
+        for (int i = 0; i < N_MMA; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (i < N_DS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+    };
+
+    const int ksteps = a.K / BK;
+    Frag f0, f1;
+    // Step ks computes from stage ks%2 (first-quarter fragments in f0).  When the last
+    // quarter's fragments have been read the stage is free for step ks+2, and the other
+    // stage (requested a step ago) must have landed.
+    auto step = [&](auto issue_tag, int ks) {
+        constexpr bool ISSUE = decltype(issue_tag)::value;
+        const int cur = ks & 1;
+        read_q(cur, 1, f1);
+        mma_q(f0);
+        pace_quarter();
+        read_q(cur, 2, f0);
+        mma_q(f1);
+        pace_quarter();
+        read_q(cur, 3, f1);
+        mma_q(f0);
+        pace_quarter();
+        wait_vmcnt<0>();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if constexpr (ISSUE) issue(cur, ks + 2);
+        read_q(cur ^ 1, 0, f0);  // past the last step: a stale stage nobody uses
+        mma_q(f1);
+        constexpr int N_VM = ISSUE ? WL + XL : 0;
+#pragma unroll
+        for (int i = 0; i < N_MMA; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (2 * i < N_VM) __builtin_amdgcn_sched_group_barrier(0x010, 2, 0);
+            else if (i - (N_VM + 1) / 2 < N_DS) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+    };
+    using issue_t = std::integral_constant<bool, true>;
+    using drain_t = std::integral_constant<bool, false>;
+
+    issue(0, 0);
+    if (ksteps > 1) {
+        issue(1, 1);
+        wait_vmcnt<9>();
+    } else {
+        wait_vmcnt<0>();
+    }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    read_q(0, 0, f0);
+    int ks = 0;
+    for (; ks + 2 < ksteps; ++ks) step(issue_t{}, ks);
+    for (; ks < ksteps; ++ks) step(drain_t{}, ks);
+
+    epilogue<TN, TM, 1>(a, acc, lds, wave, lane, n0 + wn * 32 * TN, m0 + wm * 32 * TM);
+}
+
+int launch_wide(Args &a, hipStream_t st) {
+    a.tiles_m = (a.M + wide::BM - 1) / wide::BM;
+    a.tiles_n = (a.N + wide::BN - 1) / wide::BN;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w8a8_wide_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, wide::LDS_BYTES) != hipSuccess)
+            return fail(CMI_E_HIP, "cmi_gemm_w8a8: cannot reserve %d bytes of LDS", wide::LDS_BYTES);
+        configured = true;
+    }
+    gemm_w8a8_wide_kernel<<<dim3(a.tiles_m * a.tiles_n), dim3(512), wide::LDS_BYTES, st>>>(a);
+    return check_launch("cmi_gemm_w8a8");
+}
+
 }  // namespace
 
 extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws,
@@ -564,19 +736,27 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
     a.K = K;
     a.ldy = ldy;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    // Tile choice: how full the last round of workgroups is (256 CUs; one 256 x 256
-    // workgroup or two 128 x 128 workgroups per CU), times the measured steady-state
-    // advantage of the large tile.  CMI_GEMM_TILE=128|256 overrides (tests, tuning).
+    // Tile choice: how full the last round of workgroups is (256 CUs; one large workgroup or
+    // two 128 x 128 workgroups per CU) and how much of the tiles' area is real output, times
+    // the steady-state advantage of the larger tiles.  CMI_GEMM_TILE=128|256|320 overrides
+    // (tests, tuning).
     const char *force = getenv("CMI_GEMM_TILE");
-    bool use_big;
+    int pick;  // 128, 256 or 320: block tile along n
     if (force && force[0]) {
-        use_big = atoi(force) == 256;
+        pick = atoi(force);
     } else {
-        const double tb = (double)((M + 255) / 256) * ((N + 255) / 256);
-        const double tsm = (double)((M + 127) / 128) * ((N + 127) / 128);
-        const double eff_big = tb / (ceil(tb / 256.0) * 256.0) * 1.23;
-        const double eff_small = tsm / (ceil(tsm / 512.0) * 512.0);
-        use_big = eff_big > eff_small;
+        auto fill = [](double tiles, double slots) { return tiles / (ceil(tiles / slots) * slots); };
+        const double t128 = (double)((M + 127) / 128) * ((N + 127) / 128);
+        const double t256 = (double)((M + 255) / 256) * ((N + 255) / 256);
+        const double t320 = (double)((M + 255) / 256) * ((N + 319) / 320);
+        // useful fraction of the tiles' area times the measured steady-state advantage
+        const double area = (double)M * N;
+        const double e128 = fill(t128, 512.0) * area / (t128 * 128 * 128);
+        const double e256 = fill(t256, 256.0) * area / (t256 * 256 * 256) * 1.23;
+        const double e320 = fill(t320, 256.0) * area / (t320 * 256 * 320) * 1.30;
+        pick = e128 >= e256 && e128 >= e320 ? 128 : e256 >= e320 ? 256 : 320;
     }
+    if (pick == 320) return launch_wide(a, st);
+    const bool use_big = pick == 256;
     return use_big ? launch_big(a, st) : launch<2, 2, 2>(a, st);
 }

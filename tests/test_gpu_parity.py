@@ -154,9 +154,9 @@ def test_gemv_w8a16_lm_head_sampled_rows(orc):
 
 # ------------------------------------------------------------------ W8A8 GEMM
 
-@pytest.fixture(params=["auto", "128", "256"])
+@pytest.fixture(params=["auto", "128", "256", "320"])
 def gemm_tile(request, monkeypatch):
-    """Force the 128 x 128 or the 256 x 256 block-tile kernel (the library reads
+    """Force the 128 x 128, 256 x 256 or 256 x 320 block-tile kernel (the library reads
     CMI_GEMM_TILE on every call), or leave the choice to the library."""
     if request.param != "auto":
         monkeypatch.setenv("CMI_GEMM_TILE", request.param)
