@@ -35,7 +35,7 @@ def seeded(seed=1234):
 # --------------------------------------------------------------------- quant
 
 @pytest.mark.parametrize("m,k", [(1, 2560), (4, 2560), (16, 9728), (7, 200), (3, 25600),
-                                 (513, 2560), (5, 1001), (2, 70000), (1, 8)])
+                                 (513, 2560), (5, 1001), (2, 70000), (1, 8), (96, 65536)])
 def test_quant_bit_exact(orc, m, k):
     g = seeded()
     x = synth.activations(m, k, g, outliers=True)
