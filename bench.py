@@ -51,6 +51,9 @@ def parse_args():
     ap.add_argument("--prefill-only", action="store_true",
                     help="time only the W8A8 prefill GEMM (M=2048 and 8192, N=9728, K=2560): the profiling "
                          "target for that kernel; prints its own JSON line")
+    ap.add_argument("--w4a8-prefill-only", action="store_true",
+                    help="time only the W4A8 prefill GEMM (M=1024, N=25600, K=5120): the profiling target "
+                         "for that kernel; prints its own JSON line")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (known traffic, for scaling HBM counters)")
     return ap.parse_args()
@@ -117,6 +120,26 @@ def main() -> int:
             out[f"M{m}_N{n_}_K{k_}"] = {"gemm_us": round(t * 1e6, 2), "tops": round(tops, 1),
                                         "frac_of_int8_peak": round(tops / INT8_PEAK_TOPS, 4)}
         print(json.dumps({"metric": "W8A8 prefill GEMM int8 TOPS", "unit": "TOP/s", "w8a8_prefill_gemm": out}))
+        return 0
+
+    if args.w4a8_prefill_only:
+        m, n_, k_ = 1024, 25600, 5120
+        w = synth.int4_weight(n_, k_, gen)
+        d4 = torch.empty((n_, k_ // 2), dtype=torch.uint8, device=dev)
+        ds = torch.empty((n_, k_ // 128), dtype=torch.float32, device=dev)
+        lib.cmi_w4_repack(ptr(w.packed), ptr(w.scale), ptr(d4), ptr(ds), n_, k_, 128, cur_stream())
+        x = synth.activations(m, k_, gen)
+        xq = torch.empty((m, k_), dtype=torch.int8, device=dev)
+        xs = torch.empty(m, dtype=torch.float32, device=dev)
+        y = torch.empty((m, n_), dtype=torch.bfloat16, device=dev)
+        lib.cmi_quant_act_i8(ptr(x), ptr(xq), ptr(xs), m, k_, cur_stream())
+        t = timed(lambda: lib.cmi_gemm_w4a8(ptr(d4), ptr(ds), ptr(xq), ptr(xs), ptr(y), vp(0), m, n_, k_, 128,
+                                            cur_stream()), args.steps, args.warmup)
+        tops = synth.gemm_ops(m, n_, k_) / t / 1e12
+        print(json.dumps({"metric": "W4A8 prefill GEMM int8 TOPS", "unit": "TOP/s",
+                          "w4a8_prefill_gemm_M1024_N25600_K5120": {
+                              "us": round(t * 1e6, 2), "tops": round(tops, 1),
+                              "frac_of_int8_peak": round(tops / INT8_PEAK_TOPS, 4)}}))
         return 0
 
     # ------------------------------------------------------------ headline: decode GEMVs

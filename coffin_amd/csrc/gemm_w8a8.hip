@@ -27,6 +27,8 @@
 //     workgroups per CU (one's prologue/epilogue hides under the other's MFMAs).
 //   gemm_w8a8_big_kernel: 256 x 256 block tile, 8 wavefronts of 128 x 64, a ring
 //     of five single-operand LDS slots.  Half the L2 -> LDS bytes per MFMA.
+//   gemm_w8a8_wide_kernel: 256 x 320 block tile, 8 wavefronts of 64 x 160, two LDS
+//     stages; for shapes whose n extent tiles better by 320 (9728 = 30.4 x 320).
 //
 // The launcher picks by how well the tile count fills the 256 CUs.
 #include "common.hpp"
