@@ -184,16 +184,23 @@ __device__ __forceinline__ void epilogue(const Args &a, v16i32 (&acc)[TN][TM], i
                 }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // own tile only: no barrier needed
+        // RPI whole rows per iteration: lane -> (row r0, chunk c) once, then only
+        // the row advances, so LDS offsets are immediates and the global
+        // pointer moves by a fixed stride.
+        constexpr int RPI = 64 / CPR;
+        const int r0 = lane / CPR, c = lane - r0 * CPR;
+        const int n = nb + c * 8;
+        const bool lane_ok = r0 < RPI && n < a.N;
+        const bool whole = vec_ok && n + 7 < a.N;
+        const int8_t *src = park + r0 * PITCH + c * 16;
+        int m = mb + j0 * 32 + r0;
+        uint16_t *dst = a.y + (size_t)m * a.ldy + n;
+        const size_t dstep = (size_t)RPI * a.ldy;
 #pragma unroll
-        for (int p = 0; p < (32 * JP * CPR + 63) / 64; ++p) {
-            const int idx = p * 64 + lane;
-            const int ml = idx / CPR, c = idx - ml * CPR;
-            const int m = mb + j0 * 32 + ml;
-            const int n = nb + c * 8;
-            if (ml >= 32 * JP || m >= a.M || n >= a.N) continue;
-            const uint4 v = *reinterpret_cast<const uint4 *>(park + ml * PITCH + c * 16);
-            uint16_t *dst = a.y + (size_t)m * a.ldy + n;
-            if (vec_ok && n + 7 < a.N) {
+        for (int it = 0; it < (32 * JP + RPI - 1) / RPI; ++it, m += RPI, dst += dstep) {
+            if (!lane_ok || m >= a.M || (it * RPI + RPI > 32 * JP && it * RPI + r0 >= 32 * JP)) continue;
+            const uint4 v = *reinterpret_cast<const uint4 *>(src + it * RPI * PITCH);
+            if (whole) {
                 *reinterpret_cast<uint4 *>(dst) = v;
             } else {
                 const uint32_t w[4] = {v.x, v.y, v.z, v.w};
