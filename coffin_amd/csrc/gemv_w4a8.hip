@@ -343,7 +343,9 @@ extern "C" int cmi_gemv_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     CMI_REQUIRE(aligned(w4, 16) && aligned(xq, 16), CMI_E_ARG,
                 "cmi_gemv_w4a8: w4 and xq must be 16-byte aligned");
     if (gs == GS && N >= 1 && M >= 1) {
-        const int rc = gemv_w4a8_decode(w4, ws, nullptr, xq, xs, y, group_acc, nullptr, nullptr, M, N, K, stream);
+        // 1..2 rows: dot-product kernel; 3..16: group sums on the matrix pipe (measured faster from 3 up)
+        const int rc = M <= 2 ? gemv_w4a8_decode(w4, ws, nullptr, xq, xs, y, group_acc, nullptr, nullptr, M, N, K, stream)
+                              : gemv_w4a8_rows16(w4, ws, xq, xs, y, group_acc, M, N, K, stream);
         if (rc != CMI_E_UNSUPPORTED) return rc;
     }
     return run_gemv_w4a8("cmi_gemv_w4a8", w4, ws, xq, xs, nullptr, nullptr, nullptr, y, group_acc, M, N, K, gs,

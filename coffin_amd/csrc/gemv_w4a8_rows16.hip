@@ -1,0 +1,222 @@
+// W4A8 GEMV for 3..16 activation rows (speculative verify, small batches), from
+// already quantised activations, K <= 10240.
+//
+//   sum_g   = sum_{k in group g} xq[m,k] * (code(n,k) - 8)     int32, exact
+//   total   = fma((float)sum_g, ws[n,g], total)                 g = 0,1,.. from 0.f
+//   y[m,n]  = bf16(total * xs[m])
+//
+// HBM-bound on the packed weight, and meant to stay so: with 16 rows the
+// v_dot4_i32_i8 formulation costs ~240 vector instructions per 16 weight bytes
+// of a lane and runs at a quarter of memory speed.  The integer group sums are
+// exact in any order, so they are formed by v_mfma_i32_16x16x64_i8 instead --
+// 16 weight rows x 16 activation rows x 64 k per instruction -- which leaves the
+// vector ALU only the nibble split and the fp32 chain.
+//
+// A workgroup owns 16 weight rows; its wavefronts split K by 128-byte lines of
+// the weight rows (two groups of 128 k each), wavefront w taking lines w,
+// w+WAVES, ..  (Two 16-row tiles per workgroup, sharing the activation
+// registers, measured no faster.)  Lane l holds
+// weight row l%16 and the 32 k  128*g + 32*(l/16) ..  of a group: 16 packed bytes, whose low nibbles are k 8i..8i+3 and high nibbles
+// k 8i+4..8i+7 of dword i.  The matching activation bytes are dwords 0,2,4,6
+// and 1,3,5,7 of the 32 contiguous xq bytes of row l%16, so both MFMA operands
+// come out of plain 16-byte loads with no shuffling.  Codes stay unsigned; the
+// -8 is applied by two more MFMAs against a constant operand of -8s (the matrix
+// pipe is idle here).  Each wavefront parks its int32 group sums in LDS and,
+// after one barrier, thread (n, m) walks the groups in ascending order.
+#include "common.hpp"
+
+namespace {
+
+using namespace cmi;
+
+typedef int v4i32 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int GS = 128;
+constexpr int ROWS = 16;        // weight rows per workgroup = activation rows per MFMA
+constexpr int MAX_K = 10240;    // 40 lines: 8 wavefronts x 5
+
+struct Args {
+    const uint8_t *w4;
+    const float *ws;
+    const int8_t *xq;
+    const float *xs;
+    uint16_t *y;
+    int32_t *group_acc;
+    int M, N, K, G;
+};
+
+__host__ __device__ inline int lds_bytes(int G) { return G * 1024 + ROWS * G * 4; }
+
+// NLP: lines per wavefront.  WAVES: wavefronts per workgroup (4 or 8).
+// DUMP: also write the int32 group sums to a.group_acc.
+template <int NLP, int WAVES, bool DUMP>
+__global__ void __launch_bounds__(WAVES * 64)
+gemv_w4a8_rows16_kernel(const Args a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    int32_t *sums = reinterpret_cast<int32_t *>(lds);             // [G][64 lanes][4]
+    float *ws_lds = reinterpret_cast<float *>(lds + a.G * 1024);  // [16][G]
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int col = lane & 15, kq = lane >> 4;
+    const int n0 = blockIdx.x * ROWS;
+    const int nrow = min(n0 + col, a.N - 1);
+    const int mrow = min(col, a.M - 1);  // rows past M repeat the last one; their sums are dropped
+
+    // 1. activations of this wavefront's groups (L2 resident; asked for first because
+    //    memory answers in request order)
+    uint4 xa[NLP][2][2];
+    const int8_t *xrow = a.xq + (size_t)mrow * a.K + kq * 32;
+#pragma unroll
+    for (int i = 0; i < NLP; ++i)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int g = min(2 * (wave + i * WAVES) + h, a.G - 1);
+            const uint4 *p = reinterpret_cast<const uint4 *>(xrow + g * GS);
+            xa[i][h][0] = p[0];
+            xa[i][h][1] = p[1];
+        }
+    // 2. the scales of the 16 rows (contiguous), into registers until the weights are asked for
+    const int ws_total = min(ROWS, a.N - n0) * a.G;
+    constexpr int WSN = (ROWS * (MAX_K / GS) + WAVES * 64 - 1) / (WAVES * 64);
+    float wsreg[WSN];
+    {
+        const float *src = a.ws + (size_t)n0 * a.G;
+#pragma unroll
+        for (int i = 0; i < WSN; ++i) {
+            const int idx = threadIdx.x + i * (WAVES * 64);
+            wsreg[i] = idx < ws_total ? src[idx] : 0.f;
+        }
+    }
+    // 3. every weight byte of this wavefront
+    u32x4 w[NLP][2];
+    const uint8_t *wrow = a.w4 + (size_t)nrow * (a.K / 2) + kq * 16;
+#pragma unroll
+    for (int i = 0; i < NLP; ++i)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int g = min(2 * (wave + i * WAVES) + h, a.G - 1);
+            w[i][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wrow + g * (GS / 2)));
+        }
+#pragma unroll
+    for (int i = 0; i < WSN; ++i) {
+        const int idx = threadIdx.x + i * (WAVES * 64);
+        if (idx < ws_total) ws_lds[idx] = wsreg[i];
+    }
+
+    // 4. integer group sums: lane holds (n = col, m = 4*kq + v), v = 0..3
+    const v4i32 minus8 = {(int)0xF8F8F8F8u, (int)0xF8F8F8F8u, (int)0xF8F8F8F8u, (int)0xF8F8F8F8u};
+#pragma unroll
+    for (int i = 0; i < NLP; ++i)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int g = 2 * (wave + i * WAVES) + h;
+            if (g >= a.G) break;  // uniform per wavefront
+            const v4i32 x0 = {(int)xa[i][h][0].x, (int)xa[i][h][0].z, (int)xa[i][h][1].x, (int)xa[i][h][1].z};
+            const v4i32 x1 = {(int)xa[i][h][0].y, (int)xa[i][h][0].w, (int)xa[i][h][1].y, (int)xa[i][h][1].w};
+            const u32x4 ww = w[i][h];
+            const u32x4 lo = ww & 0x0F0F0F0Fu, hi = (ww >> 4) & 0x0F0F0F0Fu;
+            v4i32 acc = {0, 0, 0, 0};
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x0, minus8, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x1, minus8, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x0, __builtin_bit_cast(v4i32, lo), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x1, __builtin_bit_cast(v4i32, hi), acc, 0, 0, 0);
+            reinterpret_cast<v4i32 *>(sums)[g * 64 + lane] = acc;
+        }
+    __syncthreads();
+
+    // 5. fp32 chain over the groups, one thread per (n, m)
+    if (threadIdx.x < 256) {
+        const int p = threadIdx.x;
+        const int l = p >> 2, v = p & 3;
+        const int nn = l & 15, m = 4 * (l >> 4) + v;
+        const int n = n0 + nn;
+        if (n < a.N && m < a.M) {
+            const int32_t *sp = sums + p;
+            const float *wsn = ws_lds + nn * a.G;
+            float total = 0.f;
+            int g = 0;
+            for (; g + 4 <= a.G; g += 4) {
+                int sv[4];
+                float wv[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    sv[i] = sp[(g + i) * 256];
+                    wv[i] = wsn[g + i];
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if constexpr (DUMP) a.group_acc[((size_t)m * a.G + g + i) * a.N + n] = sv[i];
+                    total = fmaf((float)sv[i], wv[i], total);
+                }
+            }
+            for (; g < a.G; ++g) {
+                const int sg = sp[g * 256];
+                if constexpr (DUMP) a.group_acc[((size_t)m * a.G + g) * a.N + n] = sg;
+                total = fmaf((float)sg, wsn[g], total);
+            }
+            a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * a.xs[m]);
+        }
+    }
+}
+
+template <int NLP, int WAVES, bool DUMP>
+int launch_one(const Args &a, hipStream_t st) {
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_w4a8_rows16_kernel<NLP, WAVES, DUMP>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(MAX_K / GS)) != hipSuccess)
+            return fail(CMI_E_HIP, "cmi_gemv_w4a8: cannot reserve %d bytes of LDS", lds_bytes(MAX_K / GS));
+        configured = true;
+    }
+    const dim3 grid((a.N + ROWS - 1) / ROWS);
+    gemv_w4a8_rows16_kernel<NLP, WAVES, DUMP><<<grid, dim3(WAVES * 64), lds_bytes(a.G), st>>>(a);
+    return check_launch("cmi_gemv_w4a8");
+}
+
+template <int NLP, int WAVES>
+int launch(const Args &a, hipStream_t st) {
+    return a.group_acc ? launch_one<NLP, WAVES, true>(a, st) : launch_one<NLP, WAVES, false>(a, st);
+}
+
+}  // namespace
+
+namespace cmi {
+
+// Returns CMI_E_UNSUPPORTED without setting the error text when the shape is
+// outside this kernel's range (the caller then uses the general kernel).
+int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs, void *y,
+                     int32_t *group_acc, int M, int N, int K, void *stream) {
+    if (M < 1 || M > ROWS || K < GS || K > MAX_K || K % GS != 0 || N < 1) return CMI_E_UNSUPPORTED;
+    Args a;
+    a.w4 = w4;
+    a.ws = ws;
+    a.xq = xq;
+    a.xs = xs;
+    a.y = static_cast<uint16_t *>(y);
+    a.group_acc = group_acc;
+    a.M = M;
+    a.N = N;
+    a.K = K;
+    a.G = K / GS;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int lines = (a.G + 1) / 2;
+    // four wavefronts per workgroup up to 20 lines (measured faster than eight), eight beyond
+    if (lines <= 20) {
+        switch ((lines + 3) / 4) {
+            case 1: return launch<1, 4>(a, st);
+            case 2: return launch<2, 4>(a, st);
+            case 3: return launch<3, 4>(a, st);
+            case 4: return launch<4, 4>(a, st);
+            default: return launch<5, 4>(a, st);
+        }
+    }
+    switch ((lines + 7) / 8) {
+        case 3: return launch<3, 8>(a, st);
+        case 4: return launch<4, 8>(a, st);
+        default: return launch<5, 8>(a, st);
+    }
+}
+
+}  // namespace cmi

@@ -228,7 +228,11 @@ def _w4_case(orc, m, n, k, g):
 @pytest.mark.parametrize("m,n,k", [(1, 9728, 2560), (1, 2560, 9728), (4, 512, 256),
                                    (16, 2560, 9728), (16, 1024, 2560), (2, 333, 1280),
                                    (8, 4096, 2560), (1, 640, 25600), (3, 7, 128), (4, 2560, 4096),
-                                   (2, 9728, 2560), (1, 300, 10240)])
+                                   (2, 9728, 2560), (1, 300, 10240),
+                                   # 3..16 rows: every lines-per-wavefront variant, ragged N, odd group counts
+                                   (5, 9728, 2560), (16, 9728, 2560), (7, 37, 128), (9, 100, 384),
+                                   (16, 530, 1152), (12, 2560, 4096), (6, 300, 5120), (16, 256, 6656),
+                                   (13, 200, 8192), (16, 333, 10240), (5, 64, 10368), (16, 64, 12288)])
 def test_gemv_w4a8_bit_exact(orc, m, n, k):
     w4, ws, xq, xs, gacc_ref, y_ref = _w4_case(orc, m, n, k, seeded())
     gacc, y = G.w4a8(w4, ws, xq, xs, k, gemm=False)
