@@ -17,6 +17,8 @@ QWeight (int8)     1..16 (any entry)           int8 weight-only GEMV
 QWeight            > 16, linear / linear_m /   weight-only GEMV, 16 rows at a
                    linear_m_verify             time (numerics stay weight-only)
 QWeight            >= 64, linear_prefill       per-token quant + W8A8 MFMA GEMM
+QWeight            >= 2, linear_m_verify with  per-token quant + W8A8 (weight read
+                   COFFIN_AMD_W8A8_VERIFY=1    once up to 16 rows, tiled beyond)
 W4A8Weight         1..16                       per-token quant + W4A8 GEMV
 W4A8Weight         > 16                        per-token quant + W4A8 MFMA GEMM
 plain tensor       any                         torch ``F.linear`` (not quantized,
@@ -32,6 +34,7 @@ re-layout is a private copy made once per weight).
 from __future__ import annotations
 
 import ctypes
+import os
 import weakref
 
 import torch
@@ -45,6 +48,15 @@ GEMV_MAX_ROWS = 16
 #: int8 MFMA GEMM (the reference's corex backend draws the same line at 64,
 #: backends/corex/__init__.py:633,1655-1659).
 PREFILL_MIN_ROWS = 64
+
+#: ``linear_m_verify`` on int8 weights may answer with W8A8 arithmetic (per-token
+#: int8 activations) instead of the weight-only GEMV: the contract allows it
+#: (backends/protocol.py:152-155) and corex keeps the same switch, off by default,
+#: as ``COFFIN_COREX_W8A8_DP4A_VERIFY`` (backends/corex/__init__.py:119-131,
+#: 450-494).  Off by default here too, so verify and decode share their numerics
+#: unless asked; on, a 16-row verify of a 2560 -> 9728 projection takes 8 us
+#: instead of 32 (the weight is read once, the sums run on the matrix pipe).
+W8A8_VERIFY = os.environ.get("COFFIN_AMD_W8A8_VERIFY", "0").strip() == "1"
 #: W4A8 switches from the GEMV to the MFMA GEMM above this many rows.
 W4_GEMM_MIN_ROWS = 17
 #: Up to this many rows the W4A8 GEMV quantises its activations itself (one launch); the
@@ -218,7 +230,7 @@ def _dense(w, x: torch.Tensor) -> torch.Tensor:
     return F.linear(x.to(compute), dense).to(x.dtype)
 
 
-def _project(w, x: torch.Tensor, prefill: bool) -> torch.Tensor:
+def _project(w, x: torch.Tensor, prefill: bool, min_rows: int = PREFILL_MIN_ROWS) -> torch.Tensor:
     if not (_is_w4(w) or _is_q8(w)):
         return _dense(w, x)
     if not _on_gpu(x):
@@ -241,12 +253,12 @@ def _project(w, x: torch.Tensor, prefill: bool) -> torch.Tensor:
     rows = act.shape[0]
     if torch.cuda.current_device() != x.device.index:
         with torch.cuda.device(x.device):
-            return _project(w, x, prefill)
+            return _project(w, x, prefill, min_rows)
     if _is_w4(w):
         out = _rows_w4(w, act)
     elif rows == 0:
         out = torch.empty((0, int(w.n)), dtype=x.dtype, device=x.device)
-    elif prefill and rows >= PREFILL_MIN_ROWS:
+    elif prefill and rows >= min_rows:
         out = _gemm_q8(w, act)
     else:
         out = _gemv_q8(w, act)
@@ -264,7 +276,15 @@ def linear_m(w, x: torch.Tensor) -> torch.Tensor:
 
 
 def linear_m_verify(w, x: torch.Tensor) -> torch.Tensor:
-    """Speculative-verify batches; same numerics as :func:`linear_m` on this backend."""
+    """Speculative-verify batches: :func:`linear_m` numerics unless ``W8A8_VERIFY`` is set.
+
+    With the switch on, int8 weights with at least two bf16 rows on the GPU take
+    quantiser + W8A8 (same conditions as backends/corex/__init__.py:462-485:
+    ``QWeight`` only, rows >= 2, everything else falls back to ``linear_m``).
+    """
+    if (W8A8_VERIFY and _is_q8(w) and x.dim() == 2 and x.shape[0] >= 2 and _on_gpu(x)
+            and x.dtype == torch.bfloat16 and int(w.k) % 16 == 0 and x.shape[-1] == int(w.k)):
+        return _project(w, x, prefill=True, min_rows=2)
     return _project(w, x, prefill=False)
 
 

@@ -21,6 +21,10 @@ int check_launch(const char *what);
 // gemm_mfma.hip: register-staged W8A8 GEMM for K % 64 != 0 (see gemm_w8a8.hip for the fast path).
 int gemm_w8a8_generic(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws, void *y,
                       int32_t *acc_out, int M, int N, int K, int ldy, void *stream);
+// gemm_w8a8_rows16.hip: W8A8 for up to 16 rows with the weight read once (K % 128 == 0,
+// K <= 10240); CMI_E_UNSUPPORTED (no error text) outside that range.
+int gemm_w8a8_rows16(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws, void *y,
+                     int32_t *acc_out, int M, int N, int K, int ldy, void *stream);
 
 // gemv_w4a8_decode.hip: W4A8 GEMV for 1..4 rows, K <= 10240, from bf16 activations (x) or
 // quantised ones (xq, xs); returns CMI_E_UNSUPPORTED (no error text) for other shapes.

@@ -732,6 +732,12 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
     CMI_REQUIRE(K % 16 == 0, CMI_E_UNSUPPORTED, "cmi_gemm_w8a8: K=%d is not a multiple of 16", K);
     CMI_REQUIRE(aligned(xq, 16) && aligned(wq, 16), CMI_E_ARG,
                 "cmi_gemm_w8a8: xq and wq must be 16-byte aligned");
+    const char *force = getenv("CMI_GEMM_TILE");
+    if (M <= 16 && !(force && force[0])) {
+        // a verify-sized batch: read the weight once, GEMV style
+        const int rc = gemm_w8a8_rows16(xq, wq, xs, ws, y, acc_out, M, N, K, ldy, stream);
+        if (rc != CMI_E_UNSUPPORTED) return rc;
+    }
     if (K % BK != 0 || N < 8) return gemm_w8a8_generic(xq, wq, xs, ws, y, acc_out, M, N, K, ldy, stream);
     Args a;
     a.xq = xq;
@@ -749,7 +755,6 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
     // two 128 x 128 workgroups per CU) and how much of the tiles' area is real output, times
     // the steady-state advantage of the larger tiles.  CMI_GEMM_TILE=128|256|320 overrides
     // (tests, tuning).
-    const char *force = getenv("CMI_GEMM_TILE");
     int pick;  // 128, 256 or 320: block tile along n
     if (force && force[0]) {
         pick = atoi(force);

@@ -15,21 +15,23 @@
 // A workgroup owns 16 weight rows; its wavefronts split K by 128-byte lines of
 // the weight rows (two groups of 128 k each), wavefront w taking lines w,
 // w+WAVES, ..  (Two 16-row tiles per workgroup, sharing the activation
-// registers, measured no faster.)  Lane l holds
-// weight row l%16 and the 32 k  128*g + 32*(l/16) ..  of a group: 16 packed bytes, whose low nibbles are k 8i..8i+3 and high nibbles
-// k 8i+4..8i+7 of dword i.  The matching activation bytes are dwords 0,2,4,6
-// and 1,3,5,7 of the 32 contiguous xq bytes of row l%16, so both MFMA operands
-// come out of plain 16-byte loads with no shuffling.  Codes stay unsigned; the
-// -8 is applied by two more MFMAs against a constant operand of -8s (the matrix
-// pipe is idle here).  Each wavefront parks its int32 group sums in LDS and,
-// after one barrier, thread (n, m) walks the groups in ascending order.
-#include "common.hpp"
+// registers, measured no faster.)  For the MFMA lane l holds weight row l%16 and
+// the 32 k  128*g + 32*(l/16) ..  of a group: 16 packed bytes, whose low nibbles
+// are k 8i..8i+3 and high nibbles k 8i+4..8i+7 of dword i.  The matching
+// activation bytes are dwords 0,2,4,6 and 1,3,5,7 of the 32 contiguous xq bytes
+// of row l%16, so both operands are plain 16-byte pieces.  They are fetched as
+// whole cache lines and rearranged through a private LDS patch.  Codes stay
+// unsigned; the -8 is applied by two more MFMAs against a constant operand of
+// -8s (the matrix pipe is idle here).  Each wavefront parks its int32 group sums
+// in LDS and, after one barrier, thread (n, m) walks the groups in ascending
+// order.
+#include "rows16_tile.hpp"
 
 namespace {
 
 using namespace cmi;
+using namespace cmi::rows16;
 
-typedef int v4i32 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int GS = 128;
@@ -46,7 +48,8 @@ struct Args {
     int M, N, K, G;
 };
 
-__host__ __device__ inline int lds_bytes(int G) { return G * 1024 + ROWS * G * 4; }
+// group sums [G][64 lanes][4], scales [16][G], one rearrangement patch per wavefront
+__host__ __device__ inline int lds_bytes(int G, int waves) { return G * 1024 + ROWS * G * 4 + waves * PATCH_BYTES; }
 
 // NLP: lines per wavefront.  WAVES: wavefronts per workgroup (4 or 8).
 // DUMP: also write the int32 group sums to a.group_acc.
@@ -57,26 +60,30 @@ gemv_w4a8_rows16_kernel(const Args a) {
     int32_t *sums = reinterpret_cast<int32_t *>(lds);             // [G][64 lanes][4]
     float *ws_lds = reinterpret_cast<float *>(lds + a.G * 1024);  // [16][G]
 
+    uint8_t *patches = lds + a.G * 1024 + ROWS * a.G * 4;
+
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int col = lane & 15, kq = lane >> 4;
+    const int kq = lane >> 4;
     const int n0 = blockIdx.x * ROWS;
-    const int nrow = min(n0 + col, a.N - 1);
-    const int mrow = min(col, a.M - 1);  // rows past M repeat the last one; their sums are dropped
+    const int lines = (a.G + 1) / 2;
+    uint8_t *patch = patches + wave * PATCH_BYTES;
 
     // 1. activations of this wavefront's groups (L2 resident; asked for first because
-    //    memory answers in request order)
-    uint4 xa[NLP][2][2];
-    const int8_t *xrow = a.xq + (size_t)mrow * a.K + kq * 32;
+    //    memory answers in request order); rows past M repeat the last one, their sums are dropped
+    v4i32 xa[NLP][2][2];
 #pragma unroll
-    for (int i = 0; i < NLP; ++i)
+    for (int i = 0; i < NLP; ++i) {
+        const int line = wave + i * WAVES;
+        if (line >= lines) break;  // uniform per wavefront
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const int g = min(2 * (wave + i * WAVES) + h, a.G - 1);
-            const uint4 *p = reinterpret_cast<const uint4 *>(xrow + g * GS);
-            xa[i][h][0] = p[0];
-            xa[i][h][1] = p[1];
+            const int g = min(2 * line + h, a.G - 1);
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                xa[i][h][j] = *reinterpret_cast<const v4i32 *>(a.xq + tile_src(lane, j, 0, a.M - 1, a.K, g * GS));
         }
+    }
     // 2. the scales of the 16 rows (contiguous), into registers until the weights are asked for
     const int ws_total = min(ROWS, a.N - n0) * a.G;
     constexpr int WSN = (ROWS * (MAX_K / GS) + WAVES * 64 - 1) / (WAVES * 64);
@@ -90,32 +97,48 @@ gemv_w4a8_rows16_kernel(const Args a) {
         }
     }
     // 3. every weight byte of this wavefront
-    u32x4 w[NLP][2];
-    const uint8_t *wrow = a.w4 + (size_t)nrow * (a.K / 2) + kq * 16;
+    v4i32 w[NLP][2];
 #pragma unroll
-    for (int i = 0; i < NLP; ++i)
+    for (int i = 0; i < NLP; ++i) {
+        const int line = wave + i * WAVES;
+        if (line >= lines) break;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int g = min(2 * (wave + i * WAVES) + h, a.G - 1);
-            w[i][h] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wrow + g * (GS / 2)));
-        }
+        for (int j = 0; j < 2; ++j)
+            w[i][j] = __builtin_nontemporal_load(reinterpret_cast<const v4i32 *>(
+                a.w4 + tile_src(lane, j, n0, a.N - 1, a.K / 2, line * 128)));
+    }
 #pragma unroll
     for (int i = 0; i < WSN; ++i) {
         const int idx = threadIdx.x + i * (WAVES * 64);
         if (idx < ws_total) ws_lds[idx] = wsreg[i];
     }
 
-    // 4. integer group sums: lane holds (n = col, m = 4*kq + v), v = 0..3
-    const v4i32 minus8 = {(int)0xF8F8F8F8u, (int)0xF8F8F8F8u, (int)0xF8F8F8F8u, (int)0xF8F8F8F8u};
+    // 4. into the MFMA arrangement: activations pieces 2kq, 2kq+1 of row lane%16 per group
 #pragma unroll
-    for (int i = 0; i < NLP; ++i)
+    for (int i = 0; i < NLP; ++i) {
+        const int line = wave + i * WAVES;
+        if (line >= lines) break;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const int g = 2 * (wave + i * WAVES) + h;
+            tile_park(patch, lane, xa[i][h][0], xa[i][h][1]);
+            xa[i][h][0] = tile_take(patch, lane, 2 * kq);
+            xa[i][h][1] = tile_take(patch, lane, 2 * kq + 1);
+        }
+    }
+    // 5. integer group sums: lane holds (n = lane%16, m = 4*kq + v), v = 0..3
+    const v4i32 minus8 = {(int)0xF8F8F8F8u, (int)0xF8F8F8F8u, (int)0xF8F8F8F8u, (int)0xF8F8F8F8u};
+#pragma unroll
+    for (int i = 0; i < NLP; ++i) {
+        const int line = wave + i * WAVES;
+        if (line >= lines) break;
+        tile_park(patch, lane, w[i][0], w[i][1]);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int g = 2 * line + h;
             if (g >= a.G) break;  // uniform per wavefront
-            const v4i32 x0 = {(int)xa[i][h][0].x, (int)xa[i][h][0].z, (int)xa[i][h][1].x, (int)xa[i][h][1].z};
-            const v4i32 x1 = {(int)xa[i][h][0].y, (int)xa[i][h][0].w, (int)xa[i][h][1].y, (int)xa[i][h][1].w};
-            const u32x4 ww = w[i][h];
+            const u32x4 ww = __builtin_bit_cast(u32x4, tile_take(patch, lane, 4 * h + kq));
+            const v4i32 x0 = {xa[i][h][0].x, xa[i][h][0].z, xa[i][h][1].x, xa[i][h][1].z};
+            const v4i32 x1 = {xa[i][h][0].y, xa[i][h][0].w, xa[i][h][1].y, xa[i][h][1].w};
             const u32x4 lo = ww & 0x0F0F0F0Fu, hi = (ww >> 4) & 0x0F0F0F0Fu;
             v4i32 acc = {0, 0, 0, 0};
             acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x0, minus8, acc, 0, 0, 0);
@@ -124,9 +147,10 @@ gemv_w4a8_rows16_kernel(const Args a) {
             acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x1, __builtin_bit_cast(v4i32, hi), acc, 0, 0, 0);
             reinterpret_cast<v4i32 *>(sums)[g * 64 + lane] = acc;
         }
+    }
     __syncthreads();
 
-    // 5. fp32 chain over the groups, one thread per (n, m)
+    // 6. fp32 chain over the groups, one thread per (n, m)
     if (threadIdx.x < 256) {
         const int p = threadIdx.x;
         const int l = p >> 2, v = p & 3;
@@ -166,12 +190,12 @@ int launch_one(const Args &a, hipStream_t st) {
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_w4a8_rows16_kernel<NLP, WAVES, DUMP>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(MAX_K / GS)) != hipSuccess)
-            return fail(CMI_E_HIP, "cmi_gemv_w4a8: cannot reserve %d bytes of LDS", lds_bytes(MAX_K / GS));
+                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(MAX_K / GS, WAVES)) != hipSuccess)
+            return fail(CMI_E_HIP, "cmi_gemv_w4a8: cannot reserve %d bytes of LDS", lds_bytes(MAX_K / GS, WAVES));
         configured = true;
     }
     const dim3 grid((a.N + ROWS - 1) / ROWS);
-    gemv_w4a8_rows16_kernel<NLP, WAVES, DUMP><<<grid, dim3(WAVES * 64), lds_bytes(a.G), st>>>(a);
+    gemv_w4a8_rows16_kernel<NLP, WAVES, DUMP><<<grid, dim3(WAVES * 64), lds_bytes(a.G, WAVES), st>>>(a);
     return check_launch("cmi_gemv_w4a8");
 }
 
@@ -202,8 +226,12 @@ int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const
     a.G = K / GS;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int lines = (a.G + 1) / 2;
-    // four wavefronts per workgroup up to 20 lines (measured faster than eight), eight beyond
-    if (lines <= 20) {
+    // Eight wavefronts per workgroup beyond 20 lines, and up to ~640 workgroups (2.5 per compute
+    // unit) where a wavefront's chain of dependent steps is what is left to shorten (0.6-0.9 us
+    // faster at N = 2560..9728); four on larger grids (7 % faster at N = 151936).
+    const int grid = (N + ROWS - 1) / ROWS;
+    const bool eight = lines > 20 || (grid <= 640 && lines >= 8);
+    if (!eight) {
         switch ((lines + 3) / 4) {
             case 1: return launch<1, 4>(a, st);
             case 2: return launch<2, 4>(a, st);
@@ -213,6 +241,8 @@ int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const
         }
     }
     switch ((lines + 7) / 8) {
+        case 1: return launch<1, 8>(a, st);
+        case 2: return launch<2, 8>(a, st);
         case 3: return launch<3, 8>(a, st);
         case 4: return launch<4, 8>(a, st);
         default: return launch<5, 8>(a, st);

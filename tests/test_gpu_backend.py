@@ -97,6 +97,30 @@ def test_prefill_switches_to_w8a8_and_matches_the_oracle(orc):
     assert _rel(y, x.float() @ q.dequant(torch.float32).t()) < 1e-1
 
 
+@pytest.mark.parametrize("rows", [1, 2, 8, 16, 17, 40])
+def test_verify_switch_takes_w8a8_and_matches_the_oracle(orc, monkeypatch, rows):
+    """The opt-in W8A8 verify route (the counterpart of corex's COFFIN_COREX_W8A8_DP4A_VERIFY):
+    from two rows up the answer is the W8A8 oracle's, bit for bit; one row and the switch
+    being off keep the weight-only numerics."""
+    g = synth.generator()
+    q = _q8(1536, 2560, g)
+    x = synth.activations(rows, 2560, g, outliers=True).to(G.DEV)
+    off = backend.linear_m_verify(q, x)
+    assert (off.view(torch.int16) == backend.linear_m(q, x).view(torch.int16)).all()
+    monkeypatch.setattr(backend, "W8A8_VERIFY", True)
+    on = backend.linear_m_verify(q, x)
+    assert on.shape == off.shape and on.dtype == off.dtype and on.is_contiguous()
+    if rows < 2:
+        assert (on.view(torch.int16) == off.view(torch.int16)).all()
+        return
+    xq, xs = orc.quant_act_i8(G.bits(x))
+    _, y_ref = orc.gemm_w8a8(xq, q.wq.cpu().numpy(), xs, q.scale.cpu().numpy(), want_acc=False)
+    assert (G.bits(on) == y_ref).all()
+    # int4 weights and plain tensors are not affected by the switch
+    w = _w4(256, 2560, g)
+    assert (backend.linear_m_verify(w, x).view(torch.int16) == backend.linear_m(w, x).view(torch.int16)).all()
+
+
 @pytest.mark.parametrize("rows", [None, 1, 4, 16, 17, 64, 300])
 def test_w4_entries_match_the_oracle_bit_for_bit(orc, rows):
     g = synth.generator()

@@ -181,6 +181,29 @@ def test_gemm_w8a8_bit_exact(orc, gemm_tile, m, n, k):
     assert (y2.view(torch.int16) == y.view(torch.int16)).all()
 
 
+@pytest.mark.parametrize("m,n,k", [(16, 9728, 2560), (16, 2560, 9728), (1, 37, 128), (5, 530, 1152),
+                                   (9, 100, 384), (12, 2560, 4096), (16, 256, 10240), (7, 300, 5120),
+                                   (2, 6144, 2560), (16, 64, 6656)])
+def test_gemm_w8a8_verify_batches_bit_exact(orc, monkeypatch, m, n, k):
+    """Up to 16 rows take the read-the-weight-once kernel: exact against the oracle, and the
+    same bits as the tiled kernel gives for the same rows (also with a row stride)."""
+    monkeypatch.delenv("CMI_GEMM_TILE", raising=False)
+    g = seeded()
+    q = synth.int8_weight(n, k, g)
+    x = synth.activations(m, k, g, outliers=True)
+    xq, xs = orc.quant_act_i8(G.bits(x))
+    acc_ref, y_ref = orc.gemm_w8a8(xq, q.wq.numpy(), xs, q.scale.numpy())
+    args = (G.dev(xq), q.wq.to(G.DEV), G.dev(xs), q.scale.to(G.DEV))
+    acc, y = G.gemm_w8a8(*args)
+    assert (acc.cpu().numpy() == acc_ref).all()
+    assert (G.bits(y) == y_ref).all()
+    _, wide = G.gemm_w8a8(*args, want_acc=False, ldy=n + 8)
+    assert (G.bits(wide[:, :n]) == y_ref).all() and (wide[:, n:].float() == 0).all()
+    monkeypatch.setenv("CMI_GEMM_TILE", "128")
+    _, tiled = G.gemm_w8a8(*args, want_acc=False)
+    assert (tiled.view(torch.int16) == y.view(torch.int16)).all()
+
+
 def test_gemm_w8a8_golden_and_row_stride(orc, golden, gemm_tile):
     g = golden("gemm_w8a8")
     acc, y = G.gemm_w8a8(G.dev(g["xq"]), G.dev(g["wq"]), G.dev(g["xs"]), G.dev(g["ws"]))
