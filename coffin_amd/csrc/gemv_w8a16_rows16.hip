@@ -1,0 +1,198 @@
+// int8 weight-only GEMV for batches of up to 16 bf16 activation rows (batched
+// decode, speculative verify).
+//
+//   y[m,n] = bf16( (sum_k x[m,k] * (float)wq[n,k]) * ws[n] )        fp32 sums
+//
+// With one row the kernel is a stream of weight bytes and a few dot-product
+// instructions per 16 of them; with 16 rows the dot products alone (8 per row
+// and 16 weight bytes) run at a quarter of memory speed.  int8 -> bf16 is exact
+// and bf16 x bf16 products are exact in fp32, so here v_mfma_f32_16x16x32_bf16
+// forms the sums -- 16 weight rows x 16 activation rows x 32 k per instruction
+// -- and the vector ALU only widens the weight bytes.  The kernel stays a GEMV
+// in every other respect: the weight is read once, straight into registers, all
+// of a wavefront's bytes requested before anything else.
+//
+// A workgroup owns 16 weight rows; its wavefronts split K by 128-byte lines of
+// the weight rows (wavefront w takes lines w, w+WAVES, ..).  For the MFMA lane l
+// holds k  32*(l/16) .. +31  of a line for weight row l%16 (two 16-byte pieces)
+// and for activation row l%16 (four pieces); both are fetched as whole cache
+// lines and rearranged through private LDS patches.  The fp32 partial tiles of
+// the wavefronts are added in wavefront order through LDS, so a row's result
+// depends on K only, not on the batch it came in.
+#include "rows16_tile.hpp"
+
+namespace {
+
+using namespace cmi;
+using namespace cmi::rows16;
+
+typedef float v4f32 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int ROWS = 16;
+constexpr int LINE = 128;           // k per line
+constexpr int XPITCH = 256 + 16;    // activation patch: 16 rows x 256 bytes
+constexpr int XPATCH_BYTES = 16 * XPITCH;
+
+struct Args {
+    const int8_t *wq;
+    const float *ws;
+    const uint16_t *x;
+    uint16_t *y;
+    int M, N, K;
+};
+
+// Four int8 of a dword -> four bf16 (two dwords); exact.
+__device__ __forceinline__ void widen4(uint32_t w, uint32_t &lo, uint32_t &hi) {
+    const float f0 = (float)(int8_t)(w);
+    const float f1 = (float)(int8_t)(w >> 8);
+    const float f2 = (float)(int8_t)(w >> 16);
+    const float f3 = (float)(int8_t)(w >> 24);
+    // integers up to 128 in magnitude live in the upper 16 bits of their fp32 pattern
+    lo = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
+    hi = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
+}
+
+// NLP: lines per wavefront and round.  WAVES: wavefronts per workgroup.  ROUNDS: 1, or 2 for
+// K above 128*NLP*WAVES (the second round's bytes are requested line by line as the first
+// round frees their registers; asking for all weight bytes at the start took 179 registers
+// and measured slower).
+template <int NLP, int WAVES, int ROUNDS>
+__global__ void __launch_bounds__(WAVES * 64)
+gemv_w8a16_rows16_kernel(const Args a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    float(*partial)[64][4] = reinterpret_cast<float(*)[64][4]>(lds);  // [WAVES][64][4]
+    uint8_t *patches = lds + WAVES * 1024;                            // per wavefront: weights, activations
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kq = lane >> 4;
+    const int n0 = blockIdx.x * ROWS;
+    const int lines = a.K / LINE;
+    uint8_t *wpatch = patches + wave * (PATCH_BYTES + XPATCH_BYTES), *xpatch = wpatch + PATCH_BYTES;
+    const uint8_t *xbytes = reinterpret_cast<const uint8_t *>(a.x);
+    auto line_of = [&](int r, int i) { return (r * NLP + i) * WAVES + wave; };
+
+    // Activations first (L2 resident; memory answers in request order), then every weight byte.
+    // An activation line is 256 bytes: parts 0 and 1, each fetched as two half tiles; rows past
+    // M repeat the last one, their sums are dropped.
+    v4i32 xr[NLP][4], wr[NLP][2];
+    auto request_x = [&](int r, int i) {
+        const int line = line_of(r, i);
+        if (line >= lines) return;  // uniform per wavefront
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            xr[i][q] = *reinterpret_cast<const v4i32 *>(
+                xbytes + tile_src(lane, q & 1, 0, a.M - 1, (size_t)a.K * 2, line * 256 + (q >> 1) * 128));
+    };
+    auto request_w = [&](int r, int i) {
+        const int line = line_of(r, i);
+        if (line >= lines) return;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            wr[i][h] = __builtin_nontemporal_load(
+                reinterpret_cast<const v4i32 *>(a.wq + tile_src(lane, h, n0, a.N - 1, a.K, line * LINE)));
+    };
+#pragma unroll
+    for (int i = 0; i < NLP; ++i) request_x(0, i);
+#pragma unroll
+    for (int i = 0; i < NLP; ++i) request_w(0, i);
+
+    // the accumulator of lane l holds (n = l%16, m = 4*kq + v), v = 0..3
+    v4f32 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < ROUNDS; ++r) {
+        // activations into the MFMA arrangement: row lane%16, bytes 64*kq .. +63 of the line
+#pragma unroll
+        for (int i = 0; i < NLP; ++i) {
+            if (line_of(r, i) >= lines) break;
+            uint8_t *p = xpatch + (lane >> 3) * XPITCH + (lane & 7) * 16;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                *reinterpret_cast<v4i32 *>(p + (q & 1) * 8 * XPITCH + (q >> 1) * 128) = xr[i][q];
+            const uint8_t *t = xpatch + (lane & 15) * XPITCH + kq * 64;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) xr[i][q] = *reinterpret_cast<const v4i32 *>(t + q * 16);
+        }
+        // weights: rearrange, widen, multiply
+#pragma unroll
+        for (int i = 0; i < NLP; ++i) {
+            if (line_of(r, i) >= lines) break;
+            tile_park(wpatch, lane, wr[i][0], wr[i][1]);
+            const v4i32 w0 = tile_take(wpatch, lane, 2 * kq), w1 = tile_take(wpatch, lane, 2 * kq + 1);
+            const uint32_t d[8] = {(uint32_t)w0.x, (uint32_t)w0.y, (uint32_t)w0.z, (uint32_t)w0.w,
+                                   (uint32_t)w1.x, (uint32_t)w1.y, (uint32_t)w1.z, (uint32_t)w1.w};
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {  // k = 32*kq + 8*s .. +7 of the line
+                uint32_t b[4];
+                widen4(d[2 * s], b[0], b[1]);
+                widen4(d[2 * s + 1], b[2], b[3]);
+                const v4i32 bw = {(int)b[0], (int)b[1], (int)b[2], (int)b[3]};
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xr[i][s]),
+                                                              __builtin_bit_cast(bf16x8, bw), acc, 0, 0, 0);
+            }
+            if (r + 1 < ROUNDS) {
+                request_x(r + 1, i);
+                request_w(r + 1, i);
+            }
+        }
+    }
+    *reinterpret_cast<v4f32 *>(&partial[wave][lane][0]) = acc;
+    __syncthreads();
+
+    if (threadIdx.x < 256) {
+        const int l = threadIdx.x >> 2, v = threadIdx.x & 3;
+        const int n = n0 + (l & 15), m = 4 * (l >> 4) + v;
+        if (n < a.N && m < a.M) {
+            float total = partial[0][l][v];
+#pragma unroll
+            for (int wv = 1; wv < WAVES; ++wv) total += partial[wv][l][v];
+            a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * a.ws[n]);
+        }
+    }
+}
+
+template <int NLP, int WAVES, int ROUNDS = 1>
+int launch(const Args &a, hipStream_t st) {
+    constexpr int LDS_BYTES = WAVES * (1024 + PATCH_BYTES + XPATCH_BYTES);
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_w8a16_rows16_kernel<NLP, WAVES, ROUNDS>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
+            return fail(CMI_E_HIP, "cmi_gemv_w8a16: cannot reserve %d bytes of LDS", LDS_BYTES);
+        configured = true;
+    }
+    const dim3 grid((a.N + ROWS - 1) / ROWS);
+    gemv_w8a16_rows16_kernel<NLP, WAVES, ROUNDS><<<grid, dim3(WAVES * 64), LDS_BYTES, st>>>(a);
+    return check_launch("cmi_gemv_w8a16");
+}
+
+}  // namespace
+
+namespace cmi {
+
+// Returns CMI_E_UNSUPPORTED without setting the error text when the shape is
+// outside this kernel's range (the caller then uses the dot-product kernel).
+int gemv_w8a16_rows16(const int8_t *wq, const float *ws, const void *x, void *y, int M, int N, int K,
+                      void *stream) {
+    if (M < 1 || M > ROWS || N < 1 || K < LINE || K % LINE != 0 || K > 80 * LINE) return CMI_E_UNSUPPORTED;
+    Args a;
+    a.wq = wq;
+    a.ws = ws;
+    a.x = static_cast<const uint16_t *>(x);
+    a.y = static_cast<uint16_t *>(y);
+    a.M = M;
+    a.N = N;
+    a.K = K;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int lines = K / LINE;
+    // eight wavefronts (shorter chains of dependent steps) up to 2048 workgroups, four beyond
+    // (2560 -> 151936: 72 us against 84)
+    if (lines <= 8) return launch<2, 4>(a, st);
+    if (lines <= 20 && (N + ROWS - 1) / ROWS > 2048) return launch<5, 4>(a, st);
+    if (lines <= 24) return launch<3, 8>(a, st);
+    if (lines <= 40) return launch<5, 8>(a, st);
+    return launch<5, 8, 2>(a, st);
+}
+
+}  // namespace cmi

@@ -78,7 +78,15 @@ def test_int8_entries_agree_with_dequant_matmul(rows):
     assert (a.view(torch.int16) == b.view(torch.int16)).all()
     if rows is not None and rows > 1:
         one = backend.linear(q, x[rows - 1])
-        assert (one.view(torch.int16) == a[rows - 1].view(torch.int16)).all()
+        if rows == 2:
+            # one and two rows share the dot-product kernel and its summation order
+            assert (one.view(torch.int16) == a[rows - 1].view(torch.int16)).all()
+        else:
+            # from three rows the sums run on the matrix pipe: same value to fp32 summation noise
+            assert _rel(a[rows - 1], one.float()) < 1e-2
+            # and a row does not depend on which rows travel with it (chunks of 16 included)
+            first = backend.linear_m(q, x[:3].contiguous())
+            assert (first.view(torch.int16) == a[:3].view(torch.int16)).all()
 
 
 def test_prefill_switches_to_w8a8_and_matches_the_oracle(orc):
