@@ -239,7 +239,7 @@ def main() -> int:
             # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this same
             # command (summary under profiles/); it only describes the default workload
             "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if (M == 1 and not args.no_graph) else None,
-            "kernel": "gemv_w8a16_kernel",
+            "kernel": "gemv_w8a16_kernel" if args.rows <= 2 else "gemv_w8a16_rows16_kernel",
             "avg_launch_us": round(step_s / n_launch * 1e6, 3),
             "algorithmic_bytes_per_launch": round(bytes_per_step / n_launch),
         },
@@ -331,6 +331,28 @@ def main() -> int:
                                       "quant_plus_gemm_us": round(tb * 1e6, 2)}
         extra["w8a8_prefill_gemm"] = mm
         extra["w8a8_prefill_int8_TOPS_M2048_N9728"] = mm["M2048_N9728_K2560"]["tops"]
+
+        # W8A8 on a verify-sized batch (16 rows): quantiser + the read-once kernel, weights rotated
+        # through enough copies that none is answered from cache
+        vf = {}
+        for name, n_, k_ in shapes:
+            copies = max(2, int(6e8 // (n_ * k_)))
+            ws_ = [synth.int8_weight(n_, k_, gen) for _ in range(copies)]
+            m = 16
+            x = synth.activations(m, k_, gen)
+            xq = torch.empty((m, k_), dtype=torch.int8, device=dev)
+            xs = torch.empty(m, dtype=torch.float32, device=dev)
+            y = torch.empty((m, n_), dtype=torch.bfloat16, device=dev)
+            def verify(ws_=ws_, x=x, xq=xq, xs=xs, y=y, m=m, n_=n_, k_=k_):
+                st = cur_stream()
+                for q in ws_:
+                    lib.cmi_quant_act_i8(ptr(x), ptr(xq), ptr(xs), m, k_, st)
+                    lib.cmi_gemm_w8a8(ptr(xq), ptr(q.wq), ptr(xs), ptr(q.scale), ptr(y), vp(0), m, n_, k_, n_, st)
+            t = timed(verify, 5) / copies
+            vf[name] = {"us": round(t * 1e6, 2), "GBps": round(n_ * k_ / t / 1e9, 1)}
+            del ws_
+        extra["w8a8_verify_M16_quant_plus_gemm"] = vf
+        torch.cuda.empty_cache()
 
         # W4A8 prefill GEMM, larger dense shape
         m, n_, k_ = 1024, 25600, 5120

@@ -105,7 +105,7 @@ gemv_w4a8_rows16_kernel(const Args a) {
 #pragma unroll
         for (int j = 0; j < 2; ++j)
             w[i][j] = __builtin_nontemporal_load(reinterpret_cast<const v4i32 *>(
-                a.w4 + tile_src(lane, j, n0, a.N - 1, a.K / 2, line * 128)));
+                a.w4 + tile_src<true>(lane, j, n0, a.N - 1, a.K / 2, line * 128)));
     }
 #pragma unroll
     for (int i = 0; i < WSN; ++i) {

@@ -16,12 +16,15 @@ typedef int v4i32 __attribute__((ext_vector_type(4)));
 constexpr int TILE_PITCH = 144;             // 128 + 16: the 16 rows of a column read hit 16 different bank groups
 constexpr int PATCH_BYTES = 16 * TILE_PITCH;
 
-// Global side: byte offset of this lane's piece in the half tile `half` (rows 8*half ..),
-// rows clamped to `last_row`, the piece clamped to stay inside a row of `row_bytes`.
+// Global side: byte offset of this lane's piece in the half tile `half` (rows 8*half ..) of the
+// line starting at byte `line_byte` of each row; rows clamped to `last_row`.  CLAMP: also keep
+// the piece inside a row of `row_bytes` (rows that end in the middle of a line).
+template <bool CLAMP = false>
 __device__ __forceinline__ size_t tile_src(int lane, int half, int first_row, int last_row, size_t row_bytes,
                                            int line_byte) {
     const int row = min(first_row + 8 * half + (lane >> 3), last_row);
-    const int off = min(line_byte + (lane & 7) * 16, (int)row_bytes - 16);
+    int off = line_byte + (lane & 7) * 16;
+    if (CLAMP) off = min(off, (int)row_bytes - 16);
     return (size_t)row * row_bytes + off;
 }
 
