@@ -2,6 +2,8 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 #include <stdint.h>
 
 #include "../../include/coffin_mi355.h"
@@ -12,6 +14,9 @@ namespace cmi {
 void set_error(const char *fmt, ...);
 int fail(int code, const char *fmt, ...);
 int check_launch(const char *what);
+// Raise a kernel's dynamic-LDS limit to `bytes` on the current device, once per device
+// (`devices`: one bit per device ordinal, owned by the call site).  CMI_OK or CMI_E_HIP.
+int reserve_lds(const void *kernel, int bytes, std::atomic<uint64_t> &devices, const char *who);
 
 #define CMI_REQUIRE(cond, code, ...)                 \
     do {                                             \

@@ -289,13 +289,10 @@ int launch(GemmArgs &a, hipStream_t st, const char *what) {
     a.tiles_m = (a.M + BM - 1) / BM;
     a.tiles_n = (a.N + BN - 1) / BN;
     const size_t lds = 2 * STAGE_BYTES + (W4 ? WS_BYTES : 0);
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel<W4>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-            return fail(CMI_E_HIP, "%s: cannot reserve %zu bytes of LDS", what, lds);
-        configured = true;
-    }
+    static std::atomic<uint64_t> devices{0};
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_kernel<W4>),
+                                   (int)lds, devices, what))
+        return rc;
     gemm_kernel<W4><<<dim3(a.tiles_m * a.tiles_n), dim3(THREADS), lds, st>>>(a);
     return check_launch(what);
 }

@@ -312,15 +312,13 @@ extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     a.G = K / BK;
     a.tiles_m = (M + BM - 1) / BM;
     a.tiles_n = (N + BN - 1) / BN;
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w4a8_kernel<false>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess ||
-            hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w4a8_kernel<true>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
-            return fail(CMI_E_HIP, "cmi_gemm_w4a8: cannot reserve %d bytes of LDS", LDS_BYTES);
-        configured = true;
-    }
+    static std::atomic<uint64_t> devices[2];
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w4a8_kernel<false>),
+                                   LDS_BYTES, devices[0], "cmi_gemm_w4a8"))
+        return rc;
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w4a8_kernel<true>),
+                                   LDS_BYTES, devices[1], "cmi_gemm_w4a8"))
+        return rc;
     const dim3 grid(a.tiles_m * a.tiles_n), block(THREADS);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (group_acc) gemm_w4a8_kernel<true><<<grid, block, LDS_BYTES, st>>>(a);

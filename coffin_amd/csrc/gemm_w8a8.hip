@@ -364,13 +364,10 @@ int launch(Args &a, hipStream_t st) {
     using C = Cfg<TN, TM, NST>;
     a.tiles_m = (a.M + C::BM - 1) / C::BM;
     a.tiles_n = (a.N + C::BN - 1) / C::BN;
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w8a8_pipe_kernel<TN, TM, NST>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES) != hipSuccess)
-            return fail(CMI_E_HIP, "cmi_gemm_w8a8: cannot reserve %d bytes of LDS", C::LDS_BYTES);
-        configured = true;
-    }
+    static std::atomic<uint64_t> devices{0};
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_pipe_kernel<TN, TM, NST>),
+                                   C::LDS_BYTES, devices, "cmi_gemm_w8a8"))
+        return rc;
     gemm_w8a8_pipe_kernel<TN, TM, NST><<<dim3(a.tiles_m * a.tiles_n), dim3(THREADS), C::LDS_BYTES, st>>>(a);
     return check_launch("cmi_gemm_w8a8");
 }
@@ -544,13 +541,10 @@ gemm_w8a8_big_kernel(const Args a) {
 int launch_big(Args &a, hipStream_t st) {
     a.tiles_m = (a.M + big::BM - 1) / big::BM;
     a.tiles_n = (a.N + big::BN - 1) / big::BN;
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w8a8_big_kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, big::LDS_BYTES) != hipSuccess)
-            return fail(CMI_E_HIP, "cmi_gemm_w8a8: cannot reserve %d bytes of LDS", big::LDS_BYTES);
-        configured = true;
-    }
+    static std::atomic<uint64_t> devices{0};
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_big_kernel),
+                                   big::LDS_BYTES, devices, "cmi_gemm_w8a8"))
+        return rc;
     gemm_w8a8_big_kernel<<<dim3(a.tiles_m * a.tiles_n), dim3(512), big::LDS_BYTES, st>>>(a);
     return check_launch("cmi_gemm_w8a8");
 }
@@ -709,13 +703,10 @@ gemm_w8a8_wide_kernel(const Args a) {
 int launch_wide(Args &a, hipStream_t st) {
     a.tiles_m = (a.M + wide::BM - 1) / wide::BM;
     a.tiles_n = (a.N + wide::BN - 1) / wide::BN;
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_w8a8_wide_kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, wide::LDS_BYTES) != hipSuccess)
-            return fail(CMI_E_HIP, "cmi_gemm_w8a8: cannot reserve %d bytes of LDS", wide::LDS_BYTES);
-        configured = true;
-    }
+    static std::atomic<uint64_t> devices{0};
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_wide_kernel),
+                                   wide::LDS_BYTES, devices, "cmi_gemm_w8a8"))
+        return rc;
     gemm_w8a8_wide_kernel<<<dim3(a.tiles_m * a.tiles_n), dim3(512), wide::LDS_BYTES, st>>>(a);
     return check_launch("cmi_gemm_w8a8");
 }

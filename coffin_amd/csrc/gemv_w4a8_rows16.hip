@@ -187,13 +187,10 @@ gemv_w4a8_rows16_kernel(const Args a) {
 
 template <int NLP, int WAVES, bool DUMP>
 int launch_one(const Args &a, hipStream_t st) {
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_w4a8_rows16_kernel<NLP, WAVES, DUMP>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes(MAX_K / GS, WAVES)) != hipSuccess)
-            return fail(CMI_E_HIP, "cmi_gemv_w4a8: cannot reserve %d bytes of LDS", lds_bytes(MAX_K / GS, WAVES));
-        configured = true;
-    }
+    static std::atomic<uint64_t> devices{0};
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w4a8_rows16_kernel<NLP, WAVES, DUMP>),
+                                   lds_bytes(MAX_K / GS, WAVES), devices, "cmi_gemv_w4a8"))
+        return rc;
     const dim3 grid((a.N + ROWS - 1) / ROWS);
     gemv_w4a8_rows16_kernel<NLP, WAVES, DUMP><<<grid, dim3(WAVES * 64), lds_bytes(a.G, WAVES), st>>>(a);
     return check_launch("cmi_gemv_w4a8");

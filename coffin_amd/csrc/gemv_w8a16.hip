@@ -416,13 +416,10 @@ int launch(GemvArgs &a, hipStream_t st) {
     const dim3 block(64 * a.uw * a.teams);
     const size_t lds = (XLDS ? 16 * (size_t)xlds_vectors(M, a.M, a.K, a.units * a.unit) : 0) +
                        (MODE == 0 ? 0 : sizeof(float) * a.teams * a.units * R * M);
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_w8a16_kernel<M, R, CHT, MODE, XLDS>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024) != hipSuccess)
-            return fail(CMI_E_HIP, "cmi_gemv_w8a16: cannot reserve LDS");
-        configured = true;
-    }
+    static std::atomic<uint64_t> devices{0};
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w8a16_kernel<M, R, CHT, MODE, XLDS>),
+                                   128 * 1024, devices, "cmi_gemv_w8a16"))
+        return rc;
     gemv_w8a16_kernel<M, R, CHT, MODE, XLDS><<<grid, block, lds, st>>>(a);
     return check_launch("cmi_gemv_w8a16");
 }

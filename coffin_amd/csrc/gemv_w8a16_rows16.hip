@@ -155,13 +155,10 @@ gemv_w8a16_rows16_kernel(const Args a) {
 template <int NLP, int WAVES, int ROUNDS = 1>
 int launch(const Args &a, hipStream_t st) {
     constexpr int LDS_BYTES = WAVES * (1024 + PATCH_BYTES + XPATCH_BYTES);
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_w8a16_rows16_kernel<NLP, WAVES, ROUNDS>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
-            return fail(CMI_E_HIP, "cmi_gemv_w8a16: cannot reserve %d bytes of LDS", LDS_BYTES);
-        configured = true;
-    }
+    static std::atomic<uint64_t> devices{0};
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w8a16_rows16_kernel<NLP, WAVES, ROUNDS>),
+                                   LDS_BYTES, devices, "cmi_gemv_w8a16"))
+        return rc;
     const dim3 grid((a.N + ROWS - 1) / ROWS);
     gemv_w8a16_rows16_kernel<NLP, WAVES, ROUNDS><<<grid, dim3(WAVES * 64), LDS_BYTES, st>>>(a);
     return check_launch("cmi_gemv_w8a16");

@@ -31,6 +31,17 @@ int check_launch(const char *what) {
     return CMI_OK;
 }
 
+int reserve_lds(const void *kernel, int bytes, std::atomic<uint64_t> &devices, const char *who) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return fail(CMI_E_HIP, "%s: no current device", who);
+    const uint64_t bit = 1ull << (dev & 63);
+    if (devices.load(std::memory_order_acquire) & bit) return CMI_OK;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess)
+        return fail(CMI_E_HIP, "%s: cannot reserve %d bytes of LDS", who, bytes);
+    devices.fetch_or(bit, std::memory_order_release);
+    return CMI_OK;
+}
+
 }  // namespace cmi
 
 extern "C" int cmi_abi_version(void) { return 1; }
