@@ -147,6 +147,27 @@ def test_w4_entries_match_the_oracle_bit_for_bit(orc, rows):
     assert _rel(y.reshape(ref.shape), ref) < 5e-2
 
 
+def test_tied_embedding_on_the_gpu(orc):
+    """Row gather on the device gives the oracle's dequantised rows; the projection is the
+    native GEMV on the same weight (ops/embed.py:64-104)."""
+    from coffin_amd import embed
+    g = synth.generator()
+    q = _q8(3000, 2560, g)
+    emb = embed.TiedEmbedding(q)
+    ids = torch.tensor([7, 2999, 0, 7, 1234], device=G.DEV)
+    rows = emb.lookup(ids)
+    want = orc.qweight_dequant_bf16(q.wq.cpu().numpy(), q.scale.cpu().numpy())[ids.cpu().numpy()]
+    assert rows.dtype == torch.bfloat16 and (G.bits(rows) == want).all()
+    x = synth.activations(1, 2560, g).to(G.DEV)[0]
+    assert (emb(x).view(torch.int16) == backend.linear(q, x).view(torch.int16)).all()
+    w = _w4(512, 2560, g)
+    emb4 = embed.TiedEmbedding(w)
+    dense = orc.w4_dequant_f32(w.packed.cpu().numpy(), w.scale.cpu().numpy(), 2560)
+    ids4 = torch.tensor([0, 511, 100], device=G.DEV)
+    assert (G.bits(emb4.lookup(ids4)) == orc.bf16_from_f32(dense[ids4.cpu().numpy()])).all()
+    assert (emb4(x).view(torch.int16) == backend.linear(w, x).view(torch.int16)).all()
+
+
 def test_outputs_are_fresh_and_inputs_untouched():
     g = synth.generator()
     q, w = _q8(256, 512, g), _w4(256, 512, g)

@@ -12,7 +12,7 @@ import numpy as np
 import pytest
 import torch
 
-from coffin_amd import _native, backend, contract, gemv, synth
+from coffin_amd import _native, backend, contract, embed, gemv, synth
 from coffin_amd.weights import (QWeight, W4A8Weight, dequantize_projection,
                                 quantize_projection)
 
@@ -172,6 +172,38 @@ def test_gemv_group_fuses_and_splits():
         gemv.GEMVGroup([qa, wa], ops=rec)
     dense = gemv.GEMVGroup([torch.ones(2, 4), torch.zeros(3, 4)], ops=rec)
     assert dense.g.w.shape == (5, 4)
+
+
+def test_tied_embedding_lookup_dequantises_only_the_gathered_rows(orc):
+    """ops/embed.py:64-81: bf16 rows whatever the storage, equal to the oracle's dequantisation
+    of those rows; the projection side goes through GEMV with the same weight."""
+    g = synth.generator()
+    ids = torch.tensor([5, 0, 39, 5, 17])
+    q = synth.int8_weight(40, 96, g)
+    emb = embed.TiedEmbedding(q, ops=Recorder())
+    assert emb.shape == (40, 96) and emb.gemv.q is q and emb.w is None
+    rows = emb.lookup(ids)
+    assert rows.dtype == torch.bfloat16 and rows.shape == (5, 96)
+    want = orc.qweight_dequant_bf16(q.wq.numpy(), q.scale.numpy())[ids.numpy()]
+    assert (rows.view(torch.int16).numpy().view(np.uint16) == want).all()
+
+    w4 = synth.int4_weight(40, 256, g)
+    emb4 = embed.TiedEmbedding(w4, ops=Recorder())
+    assert emb4.shape == (40, 256) and emb4.gemv.q4 is w4
+    rows4 = emb4.lookup(ids)
+    dense = orc.w4_dequant_f32(w4.packed.numpy(), w4.scale.numpy(), 256)[ids.numpy()]
+    assert rows4.dtype == torch.bfloat16
+    assert (rows4.view(torch.int16).numpy().view(np.uint16) == orc.bf16_from_f32(dense)).all()
+
+    plain = torch.randn(12, 8, generator=g)
+    embp = embed.TiedEmbedding(plain, ops=Recorder())
+    assert embp.shape == (12, 8)
+    assert (embp.lookup(torch.tensor([3, 3, 11])) == plain[[3, 3, 11]].to(torch.bfloat16)).all()
+    # both projection entries hand the weight to the table
+    rec = Recorder()
+    proj = embed.TiedEmbedding(q, ops=rec)
+    assert proj(torch.zeros(96)).shape == (40,) and proj.prefill(torch.zeros(9, 96)).shape == (9, 40)
+    assert [c[0] for c in rec.calls] == ["linear", "linear_prefill"]
 
 
 # --------------------------------------------------------------- adapters, CPU
