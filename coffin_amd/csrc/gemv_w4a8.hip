@@ -79,7 +79,8 @@ gemv_w4a8_kernel(const W4Args a) {
 #pragma unroll
         for (int m = 0; m < M; ++m) {
             const float amax = fmaxf(fmaxf(part[m * 4], part[m * 4 + 1]), fmaxf(part[m * 4 + 2], part[m * 4 + 3]));
-            const float sc = quant_scale(amax);
+            const RowScale rs = row_scale(amax);
+            const float sc = rs.sc;
             if (threadIdx.x == 0) {
                 xs_lds[m] = sc;
                 if (a.xs_out && blockIdx.x == 0 && m < a.M) a.xs_out[m] = sc;
@@ -88,7 +89,7 @@ gemv_w4a8_kernel(const W4Args a) {
             for (int j = 0; j < XV; ++j) {
                 const int idx = threadIdx.x + j * 256;
                 if (idx < xvecs) {
-                    const uint2 q = quant8(v[m][j], sc);
+                    const uint2 q = quant8(v[m][j], rs);
                     reinterpret_cast<uint2 *>(xq_lds + (size_t)m * a.K)[idx] = q;
                     if (a.xq_out && blockIdx.x == 0 && m < a.M)
                         reinterpret_cast<uint2 *>(a.xq_out + (size_t)m * a.K)[idx] = q;

@@ -163,7 +163,8 @@ gemv_w4a8_decode_kernel(const Args a) {
         for (int m = 0; m < M; ++m) {
             const float amax =
                 fmaxf(fmaxf(part[m * 4], part[m * 4 + 1]), fmaxf(part[m * 4 + 2], part[m * 4 + 3]));
-            const float sc = quant_scale(amax);
+            const RowScale rs = row_scale(amax);
+            const float sc = rs.sc;
             if (threadIdx.x == 0) {
                 xs_lds[m] = sc;
                 if (a.xs_out && blockIdx.x == 0 && m < a.M) a.xs_out[m] = sc;
@@ -172,7 +173,7 @@ gemv_w4a8_decode_kernel(const Args a) {
             for (int j = 0; j < XVN; ++j) {
                 if (j * 256 >= xvecs) break;  // uniform
                 const int idx = threadIdx.x + j * 256;
-                const uint2 q = quant8(v[m][j], sc);
+                const uint2 q = quant8(v[m][j], rs);
                 // four consecutive vectors (adjacent lanes) = one chunk
                 int s8 = __builtin_amdgcn_sdot4((int)q.x, 0x01010101, 0, false);
                 s8 = __builtin_amdgcn_sdot4((int)q.y, 0x01010101, s8, false);

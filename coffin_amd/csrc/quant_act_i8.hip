@@ -46,19 +46,21 @@ quant_act_i8_vec(const uint4 *__restrict__ x, uint2 *__restrict__ q, float *__re
 #pragma unroll
         for (int i = 0; i < VPT; ++i) amax = absmax8(v[i], amax);
         amax = block_max(amax, smem);
-        const float sc = quant_scale(amax);
+        const RowScale rs = row_scale(amax);
+        const float sc = rs.sc;
         if (threadIdx.x == 0) s[row] = sc;
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
             const int idx = threadIdx.x + i * QUANT_THREADS;
-            if (idx < nvec) qr[idx] = quant8(v[i], sc);
+            if (idx < nvec) qr[idx] = quant8(v[i], rs);
         }
     } else {
         for (int idx = threadIdx.x; idx < nvec; idx += QUANT_THREADS) amax = absmax8(xr[idx], amax);
         amax = block_max(amax, smem);
-        const float sc = quant_scale(amax);
+        const RowScale rs = row_scale(amax);
+        const float sc = rs.sc;
         if (threadIdx.x == 0) s[row] = sc;
-        for (int idx = threadIdx.x; idx < nvec; idx += QUANT_THREADS) qr[idx] = quant8(xr[idx], sc);
+        for (int idx = threadIdx.x; idx < nvec; idx += QUANT_THREADS) qr[idx] = quant8(xr[idx], rs);
     }
 }
 
@@ -74,10 +76,11 @@ quant_act_i8_scalar(const uint16_t *__restrict__ x, int8_t *__restrict__ q,
     for (int k = threadIdx.x; k < K; k += QUANT_THREADS)
         amax = fmaxf(amax, fabsf(bf16_bits_to_f32(xr[k])));
     amax = block_max(amax, smem);
-    const float sc = quant_scale(amax);
+    const RowScale rs = row_scale(amax);
+    const float sc = rs.sc;
     if (threadIdx.x == 0) s[row] = sc;
     for (int k = threadIdx.x; k < K; k += QUANT_THREADS)
-        qr[k] = (int8_t)quant1(bf16_bits_to_f32(xr[k]), sc);
+        qr[k] = (int8_t)quant1(bf16_bits_to_f32(xr[k]), rs);
 }
 
 }  // namespace

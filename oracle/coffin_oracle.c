@@ -127,6 +127,50 @@ void orc_quant_act_i8(const uint16_t *x, int64_t M, int64_t K, int8_t *q,
     }
 }
 
+/* Proof obligation of the GPU quantiser, checked by exhaustion rather than by
+ * argument.  The kernels do not divide per element: with r = 1.0f / sc (one IEEE
+ * division per row) they form
+ *     q0 = x * r;  e = fma(-q0, sc, x);  q1 = fma(e, r, q0)
+ * and round q1.  This counts the (amax, x) pairs for which that differs from
+ * rintf(x / sc) clamped to +-127 -- over every scale a row can have (amax = any
+ * finite non-negative bf16 with bit pattern in [amax_lo, amax_hi)) and every
+ * finite bf16 x with |x| <= amax.  With check_quotient != 0 the quotients
+ * themselves must agree bit for bit wherever x / sc is a normal number.
+ * Must return 0. */
+int64_t orc_quant_division_mismatches(int32_t amax_lo, int32_t amax_hi, int32_t check_quotient) {
+    int64_t bad = 0;
+    if (amax_lo < 0) amax_lo = 0;
+    if (amax_hi > 0x7F80) amax_hi = 0x7F80;
+#pragma omp parallel for schedule(dynamic, 64) reduction(+ : bad)
+    for (int32_t a = amax_lo; a < amax_hi; ++a) {
+        const float amax = bf16_to_f32((uint16_t)a);
+        const float sc = fmaxf(amax, 1e-5f) / 127.0f;
+        const float r = 1.0f / sc;
+        for (int32_t xb = 0; xb <= a; ++xb) {
+            for (int sign = 0; sign < 2; ++sign) {
+                const float x = bf16_to_f32((uint16_t)(xb | (sign << 15)));
+                const float ref_q = x / sc;
+                float ref = rintf(ref_q);
+                ref = fminf(fmaxf(ref, -127.f), 127.f);
+                const float q0 = x * r;
+                const float e = fmaf(-q0, sc, x);
+                const float q1 = fmaf(e, r, q0);
+                float got = rintf(q1);
+                got = fminf(fmaxf(got, -127.f), 127.f);
+                int differ = (int)got != (int)ref;
+                if (check_quotient && fabsf(ref_q) >= 1.17549435e-38f) {
+                    uint32_t u0, u1;
+                    memcpy(&u0, &ref_q, 4);
+                    memcpy(&u1, &q1, 4);
+                    differ |= u0 != u1;
+                }
+                bad += differ;
+            }
+        }
+    }
+    return bad;
+}
+
 /* ------------------------------------------------ R7: W4 pack / unpack */
 
 /* tools/quant_disk_w4a8.py:45-89 (quantize_projection), group_size along K:

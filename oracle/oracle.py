@@ -119,6 +119,15 @@ def w4_dequant_f32(packed: np.ndarray, scale: np.ndarray, k: int,
 
 # --------------------------------------------------------- activation quant R3
 
+def quant_division_mismatches(amax_lo: int = 0, amax_hi: int = 0x7F80, check_quotient: bool = True) -> int:
+    """Pairs (row absmax, element) for which the kernels' division-free rounding
+    (one reciprocal per row, two fused multiply-adds per element) differs from
+    ``rint(x / s)`` of backends/reference/__init__.py:386-389; exhaustive over bf16."""
+    fn = lib().orc_quant_division_mismatches
+    fn.restype = ctypes.c_int64
+    return int(fn(ctypes.c_int32(amax_lo), ctypes.c_int32(amax_hi), ctypes.c_int32(int(check_quotient))))
+
+
 def quant_act_i8(x_bf16: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
     """R3, backends/reference/__init__.py:386-389.  x bf16 bits [M,K] -> (q, s)."""
     m, k = x_bf16.shape

@@ -68,6 +68,26 @@ def test_quant_full_prefill_size_properties():
     assert (q2 == q[100:164]).all() and (s2 == s[100:164]).all()
 
 
+def test_quant_act_rows_with_non_finite_values_keep_the_division(orc):
+    """A row holding inf or nan has no finite scale; such rows take the per-element division
+    so that they keep giving what the reference statement gives (finite rows beside them
+    are unaffected)."""
+    g = seeded()
+    x = synth.activations(6, 512, g).float()
+    x[1, 7] = float("inf")
+    x[3, 100] = float("-inf")
+    x[4, 5] = float("nan")
+    xb = x.to(torch.bfloat16)
+    q, s = G.quant(xb.to(G.DEV))
+    q_ref, s_ref = orc.quant_act_i8(G.bits(xb))
+    finite = [0, 2, 5]
+    assert (q.cpu().numpy()[finite] == q_ref[finite]).all() and (s.cpu().numpy()[finite] == s_ref[finite]).all()
+    # inf rows: scale inf, finite elements quantise to 0 exactly as x / inf does
+    for r, c in ((1, 7), (3, 100)):
+        row = q.cpu().numpy()[r]
+        assert np.isinf(s.cpu().numpy()[r]) and (np.delete(row, c) == 0).all()
+
+
 # ------------------------------------------------------- int8 weight-only GEMV
 
 def _w8a16_case(orc, m, n, k, g):

@@ -112,6 +112,15 @@ def test_quant_act_uses_division_not_reciprocal(orc):
     assert found > 0, "no discriminating input found; widen the search"
 
 
+def test_quantiser_rounding_without_per_element_division_is_exhaustively_exact(orc):
+    """The GPU kernels divide once per row (rc = 1/s) and round fma(fma(-x*rc, s, x), rc, x*rc)
+    instead of x / s.  Every (row absmax, element) pair of finite bf16 values -- about 1e9 --
+    gives the same int8 as the division; the quotients themselves are allowed to differ in
+    the last bit (they do, in a fraction of a percent of the pairs), the integers are not."""
+    assert orc.quant_division_mismatches(0, 0x7F80, check_quotient=False) == 0
+    assert orc.quant_division_mismatches(0x3F00, 0x3F10, check_quotient=True) > 0
+
+
 def test_quant_act_matches_torch_engine(orc):
     g = torch.Generator().manual_seed(1234)
     x = torch.randn(33, 2560, generator=g)
