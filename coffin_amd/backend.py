@@ -64,15 +64,32 @@ W4_GEMM_MIN_ROWS = 17
 #: than the separate quantiser launch.
 W4_FUSED_MAX_ROWS = 1
 
-_vp = ctypes.c_void_p
+def _vp(address: int) -> int:
+    """Pointer argument: the entry points declare ``void *`` (``argtypes``), so a plain int passes."""
+    return address
 
 
-def _ptr(t: torch.Tensor | None) -> ctypes.c_void_p:
-    return _vp(t.data_ptr()) if t is not None else _vp(0)
+def _ptr(t: torch.Tensor | None) -> int:
+    return t.data_ptr() if t is not None else 0
 
 
-def _stream() -> ctypes.c_void_p:
-    return _vp(torch.cuda.current_stream().cuda_stream)
+# The adapters run once per projection and token; what they do on the host is part of the decode
+# path (corex measured 36 us per call for its W4A8 adapter, backends/corex/__init__.py:580-585).
+# ``torch.cuda.current_stream()`` builds a Stream object through three layers of Python (several
+# microseconds); the raw getter behind it returns the handle directly.
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
+def _stream() -> int:
+    """Handle of torch's current stream on the current device."""
+    if _raw_stream is not None:
+        return _raw_stream(_current_device())
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _current_device() -> int:
+    return _raw_device() if _raw_device is not None else torch.cuda.current_device()
 
 
 def _is_w4(w) -> bool:
@@ -153,63 +170,93 @@ def _w4_operands(w):
 
 # ------------------------------------------------------------------- kernels
 
-def _quantize_rows(act: torch.Tensor, xq: torch.Tensor, xs: torch.Tensor) -> None:
-    rows, k = act.shape
-    _native.check(_native.load().cmi_quant_act_i8(_ptr(act), _ptr(xq), _ptr(xs), rows, k,
-                                                  _stream()), "quant_act_i8")
+def _quantize_rows(act: torch.Tensor, xq: torch.Tensor, xs: torch.Tensor, rows: int, k: int) -> None:
+    rc = _native.load().cmi_quant_act_i8(act.data_ptr(), xq.data_ptr(), xs.data_ptr(), rows, k, _stream())
+    if rc:
+        _native.check(rc, "quant_act_i8")
 
 
-def _gemv_q8(w, act: torch.Tensor) -> torch.Tensor:
-    wq, scale = _q8_operands(w)
-    n, k = wq.shape
-    rows = act.shape[0]
-    out = torch.empty((rows, n), dtype=torch.bfloat16, device=act.device)
-    lib = _native.load()
+class _Record:
+    """What the adapters need of one quantized weight, resolved once: operand addresses in
+    device layout, shape, device.  Holds no strong reference to the caller's tensors."""
+
+    __slots__ = ("kind", "src", "src2", "a", "b", "n", "k", "gs", "dev")
+
+
+#: id(weight object) -> _Record; an entry is trusted only while the tensors it was
+#: built from are still the ones the weight object holds.
+_RECORDS: dict = {}
+_RECORDS_MAX = 8192
+
+
+def _lookup(w) -> _Record | None:
+    rec = _RECORDS.get(id(w))
+    if rec is None:
+        return None
+    try:
+        first = w.wq if rec.kind == 8 else w.packed
+        if rec.src() is first and rec.src2() is w.scale:
+            return rec
+    except AttributeError:
+        pass
+    return None
+
+
+def _make_record(w) -> _Record:
+    rec = _Record()
+    if _is_w4(w):
+        w4, ws = _w4_operands(w)
+        rec.kind, rec.src, rec.a, rec.b = 4, weakref.ref(w.packed), w4.data_ptr(), ws.data_ptr()
+        rec.n, rec.k, rec.gs, rec.dev = int(w.n), int(w.k), int(w.group_size), w.packed.device
+    else:
+        wq, scale = _q8_operands(w)
+        rec.kind, rec.src, rec.a, rec.b = 8, weakref.ref(w.wq), wq.data_ptr(), scale.data_ptr()
+        rec.n, rec.k, rec.gs, rec.dev = int(wq.shape[0]), int(wq.shape[1]), 0, w.wq.device
+    rec.src2 = weakref.ref(w.scale)
+    if len(_RECORDS) >= _RECORDS_MAX:
+        _RECORDS.clear()
+    _RECORDS[id(w)] = rec
+    return rec
+
+
+def _gemv_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> None:
+    n, k = rec.n, rec.k
+    fn = _native.load().cmi_gemv_w8a16
     stream = _stream()
+    x0, y0 = act.data_ptr(), out.data_ptr()
     for lo in range(0, rows, GEMV_MAX_ROWS):
         m = min(GEMV_MAX_ROWS, rows - lo)
-        _native.check(lib.cmi_gemv_w8a16(_ptr(wq), _ptr(scale), _vp(act.data_ptr() + lo * k * 2),
-                                         _vp(out.data_ptr() + lo * n * 2), m, n, k, stream),
-                      "gemv_w8a16")
-    return out
+        rc = fn(rec.a, rec.b, x0 + lo * k * 2, y0 + lo * n * 2, m, n, k, stream)
+        if rc:
+            _native.check(rc, "gemv_w8a16")
 
 
-def _gemm_q8(w, act: torch.Tensor) -> torch.Tensor:
-    wq, scale = _q8_operands(w)
-    n, k = wq.shape
-    rows = act.shape[0]
+def _gemm_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> None:
+    n, k = rec.n, rec.k
     xq, xs = _scratch(rows, k, act.device)
-    out = torch.empty((rows, n), dtype=torch.bfloat16, device=act.device)
-    _quantize_rows(act, xq, xs)
-    _native.check(_native.load().cmi_gemm_w8a8(_ptr(xq), _ptr(wq), _ptr(xs), _ptr(scale),
-                                               _ptr(out), _vp(0), rows, n, k, n, _stream()),
+    _quantize_rows(act, xq, xs, rows, k)
+    _native.check(_native.load().cmi_gemm_w8a8(_ptr(xq), rec.a, _ptr(xs), rec.b,
+                                               _ptr(out), 0, rows, n, k, n, _stream()),
                   "gemm_w8a8")
-    return out
 
 
-def _rows_w4(w, act: torch.Tensor) -> torch.Tensor:
-    n, k, gs = int(w.n), int(w.k), int(w.group_size)
-    rows = act.shape[0]
-    w4, ws = _w4_operands(w)
-    out = torch.empty((rows, n), dtype=torch.bfloat16, device=act.device)
-    if rows == 0:
-        return out
+def _rows_w4(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> None:
+    n, k, gs = rec.n, rec.k, rec.gs
     lib = _native.load()
     if rows <= W4_FUSED_MAX_ROWS:
         # decode: one launch, activations quantised inside the GEMV (same bits)
-        rc = lib.cmi_gemv_w4a8_bf16(_ptr(w4), _ptr(ws), _ptr(act), _ptr(out), _vp(0), _vp(0), _vp(0),
+        rc = lib.cmi_gemv_w4a8_bf16(rec.a, rec.b, act.data_ptr(), out.data_ptr(), 0, 0, 0,
                                     rows, n, k, gs, _stream())
         if rc == 0:
-            return out
+            return
         if rc != _native.E_UNSUPPORTED:
             _native.check(rc, "gemv_w4a8_bf16")
     xq, xs = _scratch(rows, k, act.device)
-    _quantize_rows(act, xq, xs)
+    _quantize_rows(act, xq, xs, rows, k)
     fn, what = ((lib.cmi_gemm_w4a8, "gemm_w4a8") if rows >= W4_GEMM_MIN_ROWS
                 else (lib.cmi_gemv_w4a8, "gemv_w4a8"))
-    _native.check(fn(_ptr(w4), _ptr(ws), _ptr(xq), _ptr(xs), _ptr(out), _vp(0), rows, n, k, gs,
+    _native.check(fn(rec.a, rec.b, _ptr(xq), _ptr(xs), out.data_ptr(), 0, rows, n, k, gs,
                      _stream()), what)
-    return out
 
 
 # ------------------------------------------------------------------ dispatch
@@ -231,38 +278,43 @@ def _dense(w, x: torch.Tensor) -> torch.Tensor:
 
 
 def _project(w, x: torch.Tensor, prefill: bool, min_rows: int = PREFILL_MIN_ROWS) -> torch.Tensor:
-    if not (_is_w4(w) or _is_q8(w)):
+    rec = _lookup(w)
+    if rec is None and not (_is_w4(w) or _is_q8(w)):
         return _dense(w, x)
-    if not _on_gpu(x):
+    dev = x.device
+    if dev.type != "cuda":
         # A CPU tensor cannot reach the kernels and this backend has no CPU
         # path for quantized weights: refuse instead of answering slowly.
         raise ValueError("coffin_amd: quantized weights need activations on the GPU, "
                          f"got {x.device}")
     if x.dtype != torch.bfloat16:
         return _dense(w, x)
-    k = int(w.k)
-    if x.dim() not in (1, 2) or x.shape[-1] != k:
+    k = rec.k if rec is not None else int(w.k)
+    nd = x.dim()
+    if nd not in (1, 2) or x.shape[-1] != k:
         raise ValueError(f"projection expects [K] or [M, K] activations with K={k}, "
                          f"got {tuple(x.shape)}")
-    wdev = (w.packed if _is_w4(w) else w.wq).device
-    if x.device != wdev:
+    wdev = rec.dev if rec is not None else (w.packed if _is_w4(w) else w.wq).device
+    if dev != wdev:
         raise ValueError(f"weight on {wdev} and activation on {x.device} must share a device")
-    act = x if x.dim() == 2 else x.unsqueeze(0)
-    if not act.is_contiguous():
-        act = act.contiguous()
-    rows = act.shape[0]
-    if torch.cuda.current_device() != x.device.index:
-        with torch.cuda.device(x.device):
+    if _current_device() != dev.index:
+        with torch.cuda.device(dev):
             return _project(w, x, prefill, min_rows)
-    if _is_w4(w):
-        out = _rows_w4(w, act)
-    elif rows == 0:
-        out = torch.empty((0, int(w.n)), dtype=x.dtype, device=x.device)
+    if rec is None:
+        rec = _make_record(w)
+    act = x if x.is_contiguous() else x.contiguous()
+    rows = 1 if nd == 1 else x.shape[0]
+    # a [K] activation is one row answered as [N]: no view juggling on the decode path
+    out = torch.empty((rec.n,) if nd == 1 else (rows, rec.n), dtype=torch.bfloat16, device=dev)
+    if rows == 0:
+        return out
+    if rec.kind == 4:
+        _rows_w4(rec, act, rows, out)
     elif prefill and rows >= min_rows:
-        out = _gemm_q8(w, act)
+        _gemm_q8(rec, act, rows, out)
     else:
-        out = _gemv_q8(w, act)
-    return out[0] if x.dim() == 1 else out
+        _gemv_q8(rec, act, rows, out)
+    return out
 
 
 def linear(w, x: torch.Tensor) -> torch.Tensor:
@@ -313,7 +365,7 @@ def kv_quant(x: torch.Tensor, out_q: torch.Tensor, out_s: torch.Tensor) -> torch
         out_q.copy_(torch.round(xf / s.unsqueeze(-1)).clamp_(-127, 127).to(torch.int8))
         return out_q
     with torch.cuda.device(x.device):
-        _quantize_rows(x, out_q, out_s)
+        _quantize_rows(x, out_q, out_s, x.shape[0], x.shape[1])
     return out_q
 
 
