@@ -222,6 +222,27 @@ def test_adapter_answers_dense_and_refuses_cpu_quantized():
     assert set(backend.native_table()) == set(contract.Ops.NAMES)
 
 
+def test_weight_records_are_cached_weakly_and_revalidated():
+    """The adapters resolve a weight's operand addresses once; the cached record must stop
+    being trusted when the weight object swaps a tensor, and must not keep weights alive."""
+    import gc
+    import weakref
+    g = synth.generator()
+    q = synth.int8_weight(6, 32, g)
+    rec = backend._make_record(q)
+    assert backend._lookup(q) is rec and (rec.kind, rec.n, rec.k) == (8, 6, 32)
+    assert rec.a == q.wq.data_ptr() and rec.b == q.scale.data_ptr()
+    q.wq = q.wq.clone()                      # same object, new tensor: record is stale
+    assert backend._lookup(q) is None
+    rec2 = backend._make_record(q)
+    assert backend._lookup(q) is rec2 and rec2.a == q.wq.data_ptr()
+    alive = weakref.ref(q.wq)
+    del q, rec, rec2
+    gc.collect()
+    assert alive() is None                   # the cache holds weak references only
+    assert backend._lookup(torch.zeros(2, 2)) is None
+
+
 def test_kv_quant_torch_branch_matches_oracle(orc):
     g = synth.generator()
     x = synth.activations(5, 96, g)
