@@ -168,6 +168,40 @@ def test_tied_embedding_on_the_gpu(orc):
     assert (emb4(x).view(torch.int16) == backend.linear(w, x).view(torch.int16)).all()
 
 
+def test_adapters_replay_inside_a_captured_graph():
+    """A decode step is captured once and replayed (the callers' engines do that): every
+    replay, with fresh activation contents in the same buffers, must equal the eager answer."""
+    g = synth.generator()
+    q, w = _q8(1024, 2560, g), _w4(768, 2560, g)
+    x1 = synth.activations(1, 2560, g).to(G.DEV)[0].contiguous()
+    x16 = synth.activations(16, 2560, g).to(G.DEV)
+    x100 = synth.activations(100, 2560, g).to(G.DEV)
+
+    def step():
+        return (backend.linear(q, x1), backend.linear(w, x1), backend.linear_m(q, x16),
+                backend.linear_m(w, x16), backend.linear_prefill(q, x100), backend.linear_prefill(w, x100))
+
+    step()                                   # warm-up: lazy library state, scratch buffers
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+        with torch.cuda.graph(graph, stream=side):
+            outs = step()
+    torch.cuda.current_stream().wait_stream(side)
+    for seed in (1, 2, 3):
+        gg = synth.generator(seed)
+        x1.copy_(synth.activations(1, 2560, gg)[0])
+        x16.copy_(synth.activations(16, 2560, gg))
+        x100.copy_(synth.activations(100, 2560, gg))
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(outs, step()):
+            assert (got.view(torch.int16) == want.view(torch.int16)).all()
+
+
 def test_outputs_are_fresh_and_inputs_untouched():
     g = synth.generator()
     q, w = _q8(256, 512, g), _w4(256, 512, g)
