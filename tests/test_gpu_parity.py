@@ -184,6 +184,38 @@ def test_gemv_w8a16_lm_head_sampled_rows(orc):
     assert (np.abs(got - exact[0]) <= np.abs(exact[0]) * WEIGHT_ONLY_EXACT_REL + 1e-6).all()
 
 
+def test_sixteen_row_kernels_at_lm_head_size_sampled_columns(orc):
+    """The three 16-row kernels on the largest weight of the model (151936 x 2560, 9496
+    workgroups): sampled output columns against the oracle -- weight-only within the exact-sum
+    bound, W8A8 and W4A8 bit for bit."""
+    _, n, k = synth.LM_HEAD
+    g = synth.generator(1234, G.DEV)
+    cols = torch.cat([torch.randint(0, n, (384,), generator=torch.Generator().manual_seed(7)),
+                      torch.tensor([0, 15, 16, n - 17, n - 1])]).to(G.DEV)
+    x = synth.activations(16, k, g, outliers=True)
+    xq, xs = orc.quant_act_i8(G.bits(x))
+
+    q = synth.int8_weight(n, k, g)
+    wq_s, ws_s = q.wq[cols].cpu().numpy(), q.scale[cols].cpu().numpy()
+    y = G.gemv_w8a16(q.wq, q.scale, x)
+    exact = orc.gemv_w8a16_exact(wq_s, ws_s, G.bits(x))
+    got = y[:, cols].float().cpu().numpy()
+    assert (np.abs(got - exact) <= np.abs(exact) * WEIGHT_ONLY_EXACT_REL + 1e-6).all()
+
+    _, y8 = G.gemm_w8a8(G.dev(xq), q.wq, G.dev(xs), q.scale, want_acc=False)
+    _, y8_ref = orc.gemm_w8a8(xq, wq_s, xs, ws_s, want_acc=False)
+    assert (G.bits(y8[:, cols].contiguous()) == y8_ref).all()
+    del q, y, y8
+    torch.cuda.empty_cache()
+
+    w = synth.int4_weight(n, k, g)
+    w4, ws4 = G.w4_repack(w.packed, w.scale, k)
+    _, y4 = G.w4a8(w4, ws4, G.dev(xq), G.dev(xs), k, gemm=False, want_acc=False)
+    _, y4_ref = orc.linear_w4a8(xq, xs, w.packed[:, cols].contiguous().cpu().numpy(),
+                                w.scale[:, cols].contiguous().cpu().numpy(), k, 128)
+    assert (G.bits(y4[:, cols].contiguous()) == y4_ref).all()
+
+
 # ------------------------------------------------------------------ W8A8 GEMM
 
 @pytest.fixture(params=["auto", "128", "256", "320"])
