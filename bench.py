@@ -45,6 +45,9 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--rows", type=int, default=1, help="activation rows M of the headline workload")
+    ap.add_argument("--mfma", action="store_true",
+                    help="headline workload through cmi_gemv_w8a16_mfma (the verify / short-prefill kernel) "
+                         "instead of the dot-product GEMV; meant for --rows 3..16")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary configurations")
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the CPU baseline leg (0 = skip)")
@@ -162,23 +165,29 @@ def main() -> int:
     def step_bytes(m):
         return sum(synth.gemv_bytes(m, n_, k_) for *_, n_, k_ in launches)
 
-    def run_step(m):
+    def run_step(m, mfma=False):
+        # mfma: the matrix-pipe GEMV that verify and short prefill chunks take (rows of a batch
+        # independent of each other, not bit-identical to the single-row call); otherwise the
+        # dot-product GEMV of linear / linear_m
         st = cur_stream()
+        fn = lib.cmi_gemv_w8a16_mfma if mfma else lib.cmi_gemv_w8a16
         for wq, sc, x, y, n_, k_ in launches:
-            rc = lib.cmi_gemv_w8a16(ptr(wq), ptr(sc), ptr(x), ptr(y), m, n_, k_, st)
+            rc = fn(ptr(wq), ptr(sc), ptr(x), ptr(y), m, n_, k_, st)
             if rc:
                 _native.check(rc, "cmi_gemv_w8a16")
 
-    def make_runner(m):
+    def make_runner(m, mfma=False):
         """Eager launcher, or a HIP graph of one step checked against the eager result."""
+        def step_fn(rows):
+            run_step(rows, mfma)
         if args.no_graph:
-            return (lambda: run_step(m)), "eager"
-        run_step(m)
+            return (lambda: step_fn(m)), "eager"
+        step_fn(m)
         torch.cuda.synchronize()
         want = [y[:m].clone() for *_, y, _, _ in launches[:4]] + [launches[-1][3][:m].clone()]
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            run_step(m)
+            step_fn(m)
         for _ in range(3):
             for *_, y, _, _ in launches:
                 y[:m].zero_()
@@ -189,7 +198,7 @@ def main() -> int:
                 raise RuntimeError("HIP graph replay differs from the eager step")
         return graph.replay, "hipgraph"
 
-    runner, launch_mode = make_runner(M)
+    runner, launch_mode = make_runner(M, args.mfma)
     for _ in range(args.warmup):
         runner()
     torch.cuda.synchronize()
@@ -239,7 +248,7 @@ def main() -> int:
             # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this same
             # command (summary under profiles/); it only describes the default workload
             "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if (M == 1 and not args.no_graph) else None,
-            "kernel": "gemv_w8a16_kernel" if args.rows <= 2 else "gemv_w8a16_rows16_kernel",
+            "kernel": "gemv_w8a16_rows16_kernel" if args.mfma else "gemv_w8a16_kernel",
             "avg_launch_us": round(step_s / n_launch * 1e6, 3),
             "algorithmic_bytes_per_launch": round(bytes_per_step / n_launch),
         },
@@ -255,6 +264,11 @@ def main() -> int:
             r, _ = make_runner(m)
             t = timed(r, max(3, args.steps // 2), warm=2)
             extra[f"decode_gemv_int8_M{m}_GBps"] = round(step_bytes(m) / t / 1e9, 1)
+        # the same step through the matrix-pipe GEMV (linear_m_verify, short linear_prefill chunks)
+        for m in (4, 8, 16):
+            r, _ = make_runner(m, True)
+            t = timed(r, max(3, args.steps // 2), warm=2)
+            extra[f"verify_gemv_int8_mfma_M{m}_GBps"] = round(step_bytes(m) / t / 1e9, 1)
         # per-shape kernel time, weights rotated through > 1 GB so HBM serves them
         per_shape = {}
         for name, n_, k_ in shapes + [synth.LM_HEAD]:

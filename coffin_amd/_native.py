@@ -24,6 +24,7 @@ _vp, _ci = ctypes.c_void_p, ctypes.c_int
 SIGNATURES: dict[str, list] = {
     "cmi_quant_act_i8": [_vp, _vp, _vp, _ci, _ci, _vp],
     "cmi_gemv_w8a16": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp],
+    "cmi_gemv_w8a16_mfma": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp],
     "cmi_w4_repack": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp],
     "cmi_gemv_w4a8": [_vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cmi_gemv_w4a8_bf16": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],

@@ -13,9 +13,10 @@ Routing, by storage type first (never by op name), then by row count:
 =================  ==========================  =================================
 weight             rows                        kernel
 =================  ==========================  =================================
-QWeight (int8)     1..16 (any entry)           int8 weight-only GEMV
-QWeight            > 16, linear / linear_m /   weight-only GEMV, 16 rows at a
-                   linear_m_verify             time (numerics stay weight-only)
+QWeight (int8)     linear, linear_m            int8 weight-only dot-product GEMV, 16
+                                               rows at a time (row r == linear(x[r]))
+QWeight            >= 3, linear_m_verify and   weight-only GEMV on the matrix pipe,
+                   linear_prefill below 64     16 rows at a time
 QWeight            >= 64, linear_prefill       per-token quant + W8A8 MFMA GEMM
 QWeight            >= 2, linear_m_verify with  per-token quant + W8A8 (weight read
                    COFFIN_AMD_W8A8_VERIFY=1    once up to 16 rows, tiled beyond)
@@ -57,6 +58,18 @@ PREFILL_MIN_ROWS = 64
 #: unless asked; on, a 16-row verify of a 2560 -> 9728 projection takes 8 us
 #: instead of 32 (the weight is read once, the sums run on the matrix pipe).
 W8A8_VERIFY = os.environ.get("COFFIN_AMD_W8A8_VERIFY", "0").strip() == "1"
+#: Static-batch decode owes its users "row r of a batch equals the single-row call on x[r]", bit
+#: for bit (models/qwen35/batch.py:19-22: a batched and an unbatched request must give the same
+#: numbers), so ``linear`` and ``linear_m`` on int8 weights stay on the dot-product GEMV, whose
+#: summation order depends on K only.  ``linear_m_verify`` (which may use a path of its own,
+#: backends/protocol.py:152-155) and short ``linear_prefill`` chunks do not carry that obligation
+#: and take the matrix-pipe GEMV from three rows up: 3-4 times faster at 8-16 rows, same
+#: weight-only arithmetic, last-place differences from fp32 summation order.
+#: ``COFFIN_AMD_BATCH_MFMA=1`` gives ``linear_m`` the fast kernel too, for deployments that prefer
+#: batch throughput to bitwise agreement between batched and unbatched requests.
+BATCH_MFMA = os.environ.get("COFFIN_AMD_BATCH_MFMA", "0").strip() == "1"
+#: Rows from which the matrix-pipe GEMV beats the dot-product one (measured on every layer shape).
+MFMA_MIN_ROWS = 3
 #: W4A8 switches from the GEMV to the MFMA GEMM above this many rows.
 W4_GEMM_MIN_ROWS = 17
 #: Up to this many rows the W4A8 GEMV quantises its activations itself (one launch); the
@@ -219,13 +232,18 @@ def _make_record(w) -> _Record:
     return rec
 
 
-def _gemv_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> None:
+def _gemv_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor, mfma: bool = False) -> None:
     n, k = rec.n, rec.k
-    fn = _native.load().cmi_gemv_w8a16
+    lib = _native.load()
+    exact = lib.cmi_gemv_w8a16
+    fast = lib.cmi_gemv_w8a16_mfma if mfma and rows >= MFMA_MIN_ROWS and k % 128 == 0 and k <= 10240 else None
     stream = _stream()
     x0, y0 = act.data_ptr(), out.data_ptr()
     for lo in range(0, rows, GEMV_MAX_ROWS):
         m = min(GEMV_MAX_ROWS, rows - lo)
+        # every chunk of a fast call takes the fast kernel, also a short last one: a row's bits
+        # must not depend on where the batch happened to be cut
+        fn = fast if fast is not None else exact
         rc = fn(rec.a, rec.b, x0 + lo * k * 2, y0 + lo * n * 2, m, n, k, stream)
         if rc:
             _native.check(rc, "gemv_w8a16")
@@ -277,7 +295,8 @@ def _dense(w, x: torch.Tensor) -> torch.Tensor:
     return F.linear(x.to(compute), dense).to(x.dtype)
 
 
-def _project(w, x: torch.Tensor, prefill: bool, min_rows: int = PREFILL_MIN_ROWS) -> torch.Tensor:
+def _project(w, x: torch.Tensor, prefill: bool, min_rows: int = PREFILL_MIN_ROWS,
+             mfma: bool = False) -> torch.Tensor:
     rec = _lookup(w)
     if rec is None and not (_is_w4(w) or _is_q8(w)):
         return _dense(w, x)
@@ -299,7 +318,7 @@ def _project(w, x: torch.Tensor, prefill: bool, min_rows: int = PREFILL_MIN_ROWS
         raise ValueError(f"weight on {wdev} and activation on {x.device} must share a device")
     if _current_device() != dev.index:
         with torch.cuda.device(dev):
-            return _project(w, x, prefill, min_rows)
+            return _project(w, x, prefill, min_rows, mfma)
     if rec is None:
         rec = _make_record(w)
     act = x if x.is_contiguous() else x.contiguous()
@@ -313,7 +332,7 @@ def _project(w, x: torch.Tensor, prefill: bool, min_rows: int = PREFILL_MIN_ROWS
     elif prefill and rows >= min_rows:
         _gemm_q8(rec, act, rows, out)
     else:
-        _gemv_q8(rec, act, rows, out)
+        _gemv_q8(rec, act, rows, out, mfma)
     return out
 
 
@@ -323,26 +342,30 @@ def linear(w, x: torch.Tensor) -> torch.Tensor:
 
 
 def linear_m(w, x: torch.Tensor) -> torch.Tensor:
-    """``linear_m(w, x[M, K]) -> [M, N]``: one weight read serves all rows."""
-    return _project(w, x, prefill=False)
+    """``linear_m(w, x[M, K]) -> [M, N]``: one weight read serves all rows; row r carries the bits
+    of ``linear(w, x[r])`` (unless ``BATCH_MFMA`` trades that for speed)."""
+    return _project(w, x, prefill=False, mfma=BATCH_MFMA)
 
 
 def linear_m_verify(w, x: torch.Tensor) -> torch.Tensor:
-    """Speculative-verify batches: :func:`linear_m` numerics unless ``W8A8_VERIFY`` is set.
+    """Speculative-verify batches.
 
-    With the switch on, int8 weights with at least two bf16 rows on the GPU take
-    quantiser + W8A8 (same conditions as backends/corex/__init__.py:462-485:
-    ``QWeight`` only, rows >= 2, everything else falls back to ``linear_m``).
+    int8 weights: weight-only arithmetic on the matrix-pipe GEMV from three rows up (a row's
+    bits do not depend on the batch, but are not those of ``linear``); with ``W8A8_VERIFY``
+    set, at least two bf16 rows on the GPU take quantiser + W8A8 instead (same conditions as
+    backends/corex/__init__.py:462-485: ``QWeight`` only, rows >= 2).  int4 weights: as
+    ``linear_m`` (exact integer sums, one summation order everywhere).
     """
     if (W8A8_VERIFY and _is_q8(w) and x.dim() == 2 and x.shape[0] >= 2 and _on_gpu(x)
             and x.dtype == torch.bfloat16 and int(w.k) % 16 == 0 and x.shape[-1] == int(w.k)):
         return _project(w, x, prefill=True, min_rows=2)
-    return _project(w, x, prefill=False)
+    return _project(w, x, prefill=False, mfma=True)
 
 
 def linear_prefill(w, x: torch.Tensor) -> torch.Tensor:
-    """``linear_prefill(w, x[C, K]) -> [C, N]``: the GEMM regime (W8A8 from 64 rows up)."""
-    return _project(w, x, prefill=True)
+    """``linear_prefill(w, x[C, K]) -> [C, N]``: the GEMM regime (W8A8 from 64 rows up; shorter
+    chunks of int8 weights stay weight-only, on the matrix-pipe GEMV)."""
+    return _project(w, x, prefill=True, mfma=True)
 
 
 def kv_quant(x: torch.Tensor, out_q: torch.Tensor, out_s: torch.Tensor) -> torch.Tensor:

@@ -40,11 +40,6 @@ int gemv_w4a8_decode(const uint8_t *w4, const float *ws, const void *x, const in
 // sums on the matrix pipe; CMI_E_UNSUPPORTED (no error text) outside that range.
 int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs, void *y,
                      int32_t *group_acc, int M, int N, int K, void *stream);
-// gemv_w8a16_rows16.hip: int8 weight-only GEMV for up to 16 rows with the sums on the matrix pipe
-// (K % 128 == 0); CMI_E_UNSUPPORTED (no error text) outside that range.
-int gemv_w8a16_rows16(const int8_t *wq, const float *ws, const void *x, void *y, int M, int N, int K,
-                      void *stream);
-
 static inline bool aligned(const void *p, uintptr_t a) {
     return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
 }

@@ -480,11 +480,6 @@ extern "C" int cmi_gemv_w8a16(const int8_t *wq, const float *ws, const void *x, 
     CMI_REQUIRE(K % 16 == 0, CMI_E_UNSUPPORTED, "cmi_gemv_w8a16: K=%d is not a multiple of 16", K);
     CMI_REQUIRE(aligned(wq, 16) && aligned(x, 16) && aligned(y, 2) && aligned(ws, 4), CMI_E_ARG,
                 "cmi_gemv_w8a16: wq and x must be 16-byte aligned");
-    if (M >= 3) {
-        // three rows and more: sums on the matrix pipe (faster from 3 rows up on every shape measured)
-        const int rc = gemv_w8a16_rows16(wq, ws, x, y, M, N, K, stream);
-        if (rc != CMI_E_UNSUPPORTED) return rc;
-    }
     const Plan p = make_plan(M, N, K);
     GemvArgs a;
     a.wq = wq;

@@ -18,7 +18,11 @@
 // and for activation row l%16 (four pieces); both are fetched as whole cache
 // lines and rearranged through private LDS patches.  The fp32 partial tiles of
 // the wavefronts are added in wavefront order through LDS, so a row's result
-// depends on K only, not on the batch it came in.
+// depends on K only, not on the batch it came in -- but it is not the bit
+// pattern of the dot-product kernel behind cmi_gemv_w8a16 (different fp32
+// summation order), which is why this kernel has an entry point of its own:
+// callers that owe their users "a batched row equals the single-row call"
+// (static-batch decode) stay on cmi_gemv_w8a16.
 #include "rows16_tile.hpp"
 
 namespace {
@@ -157,22 +161,24 @@ int launch(const Args &a, hipStream_t st) {
     constexpr int LDS_BYTES = WAVES * (1024 + PATCH_BYTES + XPATCH_BYTES);
     static std::atomic<uint64_t> devices{0};
     if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w8a16_rows16_kernel<NLP, WAVES, ROUNDS>),
-                                   LDS_BYTES, devices, "cmi_gemv_w8a16"))
+                                   LDS_BYTES, devices, "cmi_gemv_w8a16_mfma"))
         return rc;
     const dim3 grid((a.N + ROWS - 1) / ROWS);
     gemv_w8a16_rows16_kernel<NLP, WAVES, ROUNDS><<<grid, dim3(WAVES * 64), LDS_BYTES, st>>>(a);
-    return check_launch("cmi_gemv_w8a16");
+    return check_launch("cmi_gemv_w8a16_mfma");
 }
 
 }  // namespace
 
-namespace cmi {
-
-// Returns CMI_E_UNSUPPORTED without setting the error text when the shape is
-// outside this kernel's range (the caller then uses the dot-product kernel).
-int gemv_w8a16_rows16(const int8_t *wq, const float *ws, const void *x, void *y, int M, int N, int K,
-                      void *stream) {
-    if (M < 1 || M > ROWS || N < 1 || K < LINE || K % LINE != 0 || K > 80 * LINE) return CMI_E_UNSUPPORTED;
+extern "C" int cmi_gemv_w8a16_mfma(const int8_t *wq, const float *ws, const void *x, void *y, int M, int N,
+                                   int K, void *stream) {
+    CMI_REQUIRE(wq && ws && x && y, CMI_E_ARG, "cmi_gemv_w8a16_mfma: null pointer");
+    CMI_REQUIRE(M >= 1 && M <= ROWS, CMI_E_UNSUPPORTED, "cmi_gemv_w8a16_mfma: M=%d outside 1..16", M);
+    CMI_REQUIRE(N >= 1 && K >= 1, CMI_E_ARG, "cmi_gemv_w8a16_mfma: bad shape N=%d K=%d", N, K);
+    CMI_REQUIRE(K % LINE == 0 && K <= 80 * LINE, CMI_E_UNSUPPORTED,
+                "cmi_gemv_w8a16_mfma: K=%d is not a multiple of 128 up to 10240 (use cmi_gemv_w8a16)", K);
+    CMI_REQUIRE(aligned(wq, 16) && aligned(x, 16) && aligned(y, 2) && aligned(ws, 4), CMI_E_ARG,
+                "cmi_gemv_w8a16_mfma: wq and x must be 16-byte aligned");
     Args a;
     a.wq = wq;
     a.ws = ws;
@@ -191,5 +197,3 @@ int gemv_w8a16_rows16(const int8_t *wq, const float *ws, const void *x, void *y,
     if (lines <= 40) return launch<5, 8>(a, st);
     return launch<5, 8, 2>(a, st);
 }
-
-}  // namespace cmi

@@ -56,6 +56,20 @@ int cmi_quant_act_i8(const void *x, int8_t *q, float *s, int M, int K, void *str
 int cmi_gemv_w8a16(const int8_t *wq, const float *ws, const void *x, void *y,
                    int M, int N, int K, void *stream);
 
+/* The same product for a batch with the sums on the matrix pipe
+ * (v_mfma_f32_16x16x32_bf16; int8 -> bf16 is exact), 1 <= M <= 16,
+ * K % 128 == 0, K <= 10240 (else CMI_E_UNSUPPORTED: use cmi_gemv_w8a16).
+ * 3-4 times faster than cmi_gemv_w8a16 at 8-16 rows.  A row's bits depend on K
+ * only, not on the rows it travels with, but differ from cmi_gemv_w8a16's in
+ * the last place (fp32 summation order): for callers without the
+ * "batched row == single-row call" obligation of static-batch decode
+ * (models/qwen35/batch.py:19-22) -- speculative verify, whose entry may use a
+ * path of its own (backends/protocol.py:152-155), and short prefill chunks.
+ * Stands where gemv_nk_i8_m is used for those callers
+ * (backends/corex/__init__.py:495-546). */
+int cmi_gemv_w8a16_mfma(const int8_t *wq, const float *ws, const void *x, void *y,
+                        int M, int N, int K, void *stream);
+
 /* One-time re-layout of a W4A8Weight for the device kernels.
  *   in : packed u8 [ceil(K/2), N] (low nibble = even k, code = q+8) and
  *        scale fp32 [K/gs, N]      (w4a8_weights.py:14-20,28-53)

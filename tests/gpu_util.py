@@ -40,12 +40,13 @@ def quant(x: torch.Tensor):
     return q, s
 
 
-def gemv_w8a16(wq, ws, x):
+def gemv_w8a16(wq, ws, x, mfma: bool = False):
+    """The dot-product GEMV, or (mfma) the matrix-pipe one for batches."""
     m, k = x.shape
     n = wq.shape[0]
     y = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
-    _native.check(_native.load().cmi_gemv_w8a16(ptr(wq), ptr(ws), ptr(x), ptr(y), m, n, k, stream()),
-                  "gemv_w8a16")
+    fn = _native.load().cmi_gemv_w8a16_mfma if mfma else _native.load().cmi_gemv_w8a16
+    _native.check(fn(ptr(wq), ptr(ws), ptr(x), ptr(y), m, n, k, stream()), "gemv_w8a16")
     return y
 
 

@@ -73,20 +73,32 @@ def test_int8_entries_agree_with_dequant_matmul(rows):
         y = fn(q, x)
         assert y.dtype == x.dtype and y.shape == ref.shape and y.is_contiguous()
         assert _rel(y, ref) < BF16_TOL
-    # weight-only entries are bit-identical to each other whatever the batch
+    # decode entries are bit-identical to each other whatever the batch (the static-batch contract)
     a, b = backend.linear(q, x), backend.linear_m(q, x)
     assert (a.view(torch.int16) == b.view(torch.int16)).all()
     if rows is not None and rows > 1:
         one = backend.linear(q, x[rows - 1])
-        if rows == 2:
-            # one and two rows share the dot-product kernel and its summation order
-            assert (one.view(torch.int16) == a[rows - 1].view(torch.int16)).all()
+        assert (one.view(torch.int16) == a[rows - 1].view(torch.int16)).all()
+        # verify and short prefill chunks take the matrix-pipe GEMV from three rows up: the same
+        # bits from both entries, independent of the rows that travel along (chunks of 16 included)
+        v, p = backend.linear_m_verify(q, x), backend.linear_prefill(q, x)
+        assert (v.view(torch.int16) == p.view(torch.int16)).all()
+        if rows >= 3:
+            first = backend.linear_m_verify(q, x[:3].contiguous())
+            assert (first.view(torch.int16) == v[:3].view(torch.int16)).all()
         else:
-            # from three rows the sums run on the matrix pipe: same value to fp32 summation noise
-            assert _rel(a[rows - 1], one.float()) < 1e-2
-            # and a row does not depend on which rows travel with it (chunks of 16 included)
-            first = backend.linear_m(q, x[:3].contiguous())
-            assert (first.view(torch.int16) == a[:3].view(torch.int16)).all()
+            assert (v.view(torch.int16) == a.view(torch.int16)).all()
+
+
+def test_batch_switch_gives_linear_m_the_matrix_pipe_kernel(monkeypatch):
+    g = synth.generator()
+    q = _q8(512, 2560, g)
+    x = synth.activations(8, 2560, g).to(G.DEV)
+    exact = backend.linear_m(q, x)
+    monkeypatch.setattr(backend, "BATCH_MFMA", True)
+    fast = backend.linear_m(q, x)
+    assert (fast.view(torch.int16) == backend.linear_m_verify(q, x).view(torch.int16)).all()
+    assert _rel(fast, exact.float()) < 1e-2
 
 
 def test_prefill_switches_to_w8a8_and_matches_the_oracle(orc):
@@ -97,9 +109,10 @@ def test_prefill_switches_to_w8a8_and_matches_the_oracle(orc):
     xq, xs = orc.quant_act_i8(G.bits(x))
     _, y_ref = orc.gemm_w8a8(xq, q.wq.cpu().numpy(), xs, q.scale.cpu().numpy(), want_acc=False)
     assert (G.bits(y) == y_ref).all()
-    # below the threshold prefill keeps weight-only numerics
+    # below the threshold prefill keeps weight-only numerics (matrix-pipe GEMV, as verify does)
     small = backend.linear_prefill(q, x[:63].contiguous())
-    assert (small.view(torch.int16) == backend.linear_m(q, x[:63].contiguous()).view(torch.int16)).all()
+    assert (small.view(torch.int16) == backend.linear_m_verify(q, x[:63].contiguous()).view(torch.int16)).all()
+    assert _rel(small, backend.linear_m(q, x[:63].contiguous()).float()) < 1e-2
     # and the W8A8 answer is the unquantised product up to int8 activation noise (rows
     # with a x20 outlier have a 20x coarser step, hence the loose bound)
     assert _rel(y, x.float() @ q.dequant(torch.float32).t()) < 1e-1
@@ -114,7 +127,10 @@ def test_verify_switch_takes_w8a8_and_matches_the_oracle(orc, monkeypatch, rows)
     q = _q8(1536, 2560, g)
     x = synth.activations(rows, 2560, g, outliers=True).to(G.DEV)
     off = backend.linear_m_verify(q, x)
-    assert (off.view(torch.int16) == backend.linear_m(q, x).view(torch.int16)).all()
+    if rows < 3:
+        assert (off.view(torch.int16) == backend.linear_m(q, x).view(torch.int16)).all()
+    else:                                    # weight-only either way, summation order differs
+        assert _rel(off, backend.linear_m(q, x).float()) < 1e-2
     monkeypatch.setattr(backend, "W8A8_VERIFY", True)
     on = backend.linear_m_verify(q, x)
     assert on.shape == off.shape and on.dtype == off.dtype and on.is_contiguous()

@@ -90,12 +90,24 @@ def test_quant_act_rows_with_non_finite_values_keep_the_division(orc):
 
 # ------------------------------------------------------- int8 weight-only GEMV
 
-def _w8a16_case(orc, m, n, k, g):
+def _w8a16_case(orc, m, n, k, g, mfma=False):
     q = synth.int8_weight(n, k, g)
     x = synth.activations(m, k, g)
     wq, ws = q.wq.numpy(), q.scale.numpy()
-    y = G.gemv_w8a16(q.wq.to(G.DEV), q.scale.to(G.DEV), x.to(G.DEV))
+    y = G.gemv_w8a16(q.wq.to(G.DEV), q.scale.to(G.DEV), x.to(G.DEV), mfma=mfma)
     return wq, ws, x, y
+
+
+def _assert_weight_only_tolerance(orc, wq, ws, x, y):
+    got = y.float().cpu().numpy()
+    ref = orc.bf16_to_f32(orc.linear_qweight(wq, ws, G.bits(x)))
+    exact = orc.gemv_w8a16_exact(wq, ws, G.bits(x))
+    rms = float(np.sqrt((ref.astype(np.float64) ** 2).mean()))
+    ulp = np.abs(ref) * 2.0 ** -7
+    assert (np.abs(got - ref) <= WEIGHT_ONLY_TOL_RMS * rms + ulp).all()
+    assert (np.abs(got - exact) <= np.abs(exact) * WEIGHT_ONLY_EXACT_REL + 1e-5 * rms).all()
+    # the stated metric itself, on the un-narrowed side: rms error stays far below 1e-2
+    assert float(np.sqrt(((got - exact) ** 2).mean())) / rms < 3e-3
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 9728, 2560), (1, 2560, 9728), (4, 4096, 2560),
@@ -107,15 +119,17 @@ def _w8a16_case(orc, m, n, k, g):
                                    (16, 200, 12800), (5, 2560, 9728)])
 def test_gemv_w8a16_within_tolerance(orc, m, n, k):
     wq, ws, x, y = _w8a16_case(orc, m, n, k, seeded())
-    got = y.float().cpu().numpy()
-    ref = orc.bf16_to_f32(orc.linear_qweight(wq, ws, G.bits(x)))
-    exact = orc.gemv_w8a16_exact(wq, ws, G.bits(x))
-    rms = float(np.sqrt((ref.astype(np.float64) ** 2).mean()))
-    ulp = np.abs(ref) * 2.0 ** -7
-    assert (np.abs(got - ref) <= WEIGHT_ONLY_TOL_RMS * rms + ulp).all()
-    assert (np.abs(got - exact) <= np.abs(exact) * WEIGHT_ONLY_EXACT_REL + 1e-5 * rms).all()
-    # the stated metric itself, on the un-narrowed side: rms error stays far below 1e-2
-    assert float(np.sqrt(((got - exact) ** 2).mean())) / rms < 3e-3
+    _assert_weight_only_tolerance(orc, wq, ws, x, y)
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 9728, 2560), (5, 2560, 9728), (7, 37, 128), (9, 100, 384),
+                                   (16, 64, 10240), (6, 530, 1152), (1, 333, 2560), (3, 2560, 4096),
+                                   (16, 1024, 5120), (12, 640, 3072), (2, 96, 8192), (16, 300, 6656)])
+def test_gemv_w8a16_mfma_within_tolerance(orc, m, n, k):
+    """The matrix-pipe GEMV: same tolerance bars as the dot-product kernel, every
+    lines-per-wavefront variant, one and two rounds, ragged N."""
+    wq, ws, x, y = _w8a16_case(orc, m, n, k, seeded(), mfma=True)
+    _assert_weight_only_tolerance(orc, wq, ws, x, y)
 
 
 def test_gemv_w8a16_golden(golden):
@@ -129,24 +143,36 @@ def test_gemv_w8a16_golden(golden):
 
 @pytest.mark.parametrize("n,k", [(4096, 2560), (2560, 9728), (1000, 4112), (512, 5120), (300, 7168),
                                  (777, 10368), (64, 128)])
-def test_gemv_w8a16_rows_do_not_depend_on_the_batch(n, k):
-    """A row's bits depend on K and on the kernel family only: up to 2 rows (dot-product
-    kernel) every row equals the single-row call; from 3 rows (matrix-pipe kernel, or the
-    dot-product kernel where K is not a multiple of 128 or above 10240) every row equals
-    the same row of the 16-row call."""
+def test_gemv_w8a16_batched_row_equals_single_row(n, k):
+    """The contract of static-batch decode (models/qwen35/batch.py:19-22): row r of a batched
+    call carries the bits of the single-row call on x[r], whatever the batch."""
     g = seeded()
     q = synth.int8_weight(n, k, g)
     wq, ws = q.wq.to(G.DEV), q.scale.to(G.DEV)
     x = synth.activations(16, k, g).to(G.DEV)
     single = torch.cat([G.gemv_w8a16(wq, ws, x[i:i + 1].contiguous()) for i in range(16)])
-    full = G.gemv_w8a16(wq, ws, x)
-    y = G.gemv_w8a16(wq, ws, x[:2].contiguous())
-    assert (y.view(torch.int16) == single[:2].view(torch.int16)).all()
-    for m in (3, 4, 5, 8, 9, 13):
+    for m in (2, 3, 4, 5, 8, 9, 16):
         y = G.gemv_w8a16(wq, ws, x[:m].contiguous())
+        assert (y.view(torch.int16) == single[:m].view(torch.int16)).all(), m
+
+
+@pytest.mark.parametrize("n,k", [(4096, 2560), (2560, 9728), (512, 5120), (300, 6656), (64, 128)])
+def test_gemv_w8a16_mfma_rows_do_not_depend_on_the_batch(n, k):
+    """The matrix-pipe GEMV makes the weaker promise: a row's bits depend on K only, not on
+    the rows it travels with (also one row alone); against the dot-product kernel the
+    difference is fp32 summation noise."""
+    g = seeded()
+    q = synth.int8_weight(n, k, g)
+    wq, ws = q.wq.to(G.DEV), q.scale.to(G.DEV)
+    x = synth.activations(16, k, g).to(G.DEV)
+    full = G.gemv_w8a16(wq, ws, x, mfma=True)
+    for m in (1, 2, 3, 5, 8, 13):
+        y = G.gemv_w8a16(wq, ws, x[:m].contiguous(), mfma=True)
         assert (y.view(torch.int16) == full[:m].view(torch.int16)).all(), m
-    # the two families agree to fp32 summation noise
-    assert ((full.float() - single.float()).abs() <= single.float().abs() * 2.0 ** -7 + 1e-4).all()
+    last = G.gemv_w8a16(wq, ws, x[15:16].contiguous(), mfma=True)
+    assert (last.view(torch.int16) == full[15:16].view(torch.int16)).all()
+    exact_kernel = G.gemv_w8a16(wq, ws, x)
+    assert ((full.float() - exact_kernel.float()).abs() <= exact_kernel.float().abs() * 2.0 ** -7 + 1e-4).all()
 
 
 def test_gemv_w8a16_decode_layer_full_size_properties():
@@ -197,7 +223,7 @@ def test_sixteen_row_kernels_at_lm_head_size_sampled_columns(orc):
 
     q = synth.int8_weight(n, k, g)
     wq_s, ws_s = q.wq[cols].cpu().numpy(), q.scale[cols].cpu().numpy()
-    y = G.gemv_w8a16(q.wq, q.scale, x)
+    y = G.gemv_w8a16(q.wq, q.scale, x, mfma=True)
     exact = orc.gemv_w8a16_exact(wq_s, ws_s, G.bits(x))
     got = y[:, cols].float().cpu().numpy()
     assert (np.abs(got - exact) <= np.abs(exact) * WEIGHT_ONLY_EXACT_REL + 1e-6).all()

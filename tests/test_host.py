@@ -265,7 +265,7 @@ def _declared_symbols() -> list[str]:
 def test_library_exports_every_declared_symbol():
     lib = _native.load()
     names = _declared_symbols()
-    assert len(names) == 9
+    assert len(names) == 10
     for name in names:
         assert getattr(lib, name) is not None
     assert set(_native.SIGNATURES) | {"cmi_abi_version", "cmi_last_error"} == set(names)
@@ -277,6 +277,11 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     null, one = ctypes.c_void_p(0), ctypes.c_void_p(256)
     assert lib.cmi_quant_act_i8(null, one, one, 1, 8, null) == _native.E_ARG
     assert "null pointer" in _native.last_error()
+    assert lib.cmi_gemv_w8a16_mfma(one, one, one, one, 17, 8, 128, null) == _native.E_UNSUPPORTED
+    assert lib.cmi_gemv_w8a16_mfma(one, one, one, one, 4, 8, 64, null) == _native.E_UNSUPPORTED
+    assert lib.cmi_gemv_w8a16_mfma(one, one, one, one, 4, 8, 10368, null) == _native.E_UNSUPPORTED
+    assert "multiple of 128" in _native.last_error()
+    assert lib.cmi_gemv_w8a16_mfma(null, one, one, one, 4, 8, 128, null) == _native.E_ARG
     assert lib.cmi_gemv_w8a16(one, one, one, one, 17, 8, 16, null) == _native.E_UNSUPPORTED
     assert "outside 1..16" in _native.last_error()
     assert lib.cmi_gemv_w8a16(one, one, one, one, 1, 8, 24, null) == _native.E_UNSUPPORTED
