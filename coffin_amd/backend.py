@@ -65,8 +65,10 @@ W8A8_VERIFY = os.environ.get("COFFIN_AMD_W8A8_VERIFY", "0").strip() == "1"
 #: backends/protocol.py:152-155) and short ``linear_prefill`` chunks do not carry that obligation
 #: and take the matrix-pipe GEMV from three rows up: 3-4 times faster at 8-16 rows, same
 #: weight-only arithmetic, last-place differences from fp32 summation order.
-#: ``COFFIN_AMD_BATCH_MFMA=1`` gives ``linear_m`` the fast kernel too, for deployments that prefer
-#: batch throughput to bitwise agreement between batched and unbatched requests.
+#: ``COFFIN_AMD_BATCH_MFMA=1`` moves *every* int8 weight-only call -- ``linear`` included, one row
+#: included -- to the matrix-pipe GEMV: the contract holds again (one kernel family, a row's bits
+#: independent of its batch), static batches of 4-16 requests run 1.5-3.8 times faster, and
+#: single-stream decode pays for it (9.3 us instead of 6.3 us for 2560 -> 9728).  A deployment choice.
 BATCH_MFMA = os.environ.get("COFFIN_AMD_BATCH_MFMA", "0").strip() == "1"
 #: Rows from which the matrix-pipe GEMV beats the dot-product one (measured on every layer shape).
 MFMA_MIN_ROWS = 3
@@ -236,7 +238,8 @@ def _gemv_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor, mfma
     n, k = rec.n, rec.k
     lib = _native.load()
     exact = lib.cmi_gemv_w8a16
-    fast = lib.cmi_gemv_w8a16_mfma if mfma and rows >= MFMA_MIN_ROWS and k % 128 == 0 and k <= 10240 else None
+    fast = (lib.cmi_gemv_w8a16_mfma
+            if mfma and (BATCH_MFMA or rows >= MFMA_MIN_ROWS) and k % 128 == 0 and k <= 10240 else None)
     stream = _stream()
     x0, y0 = act.data_ptr(), out.data_ptr()
     for lo in range(0, rows, GEMV_MAX_ROWS):
@@ -338,12 +341,12 @@ def _project(w, x: torch.Tensor, prefill: bool, min_rows: int = PREFILL_MIN_ROWS
 
 def linear(w, x: torch.Tensor) -> torch.Tensor:
     """``linear(w, x) -> y``: ``x`` ``[K]`` or ``[C, K]``, ``y`` ``[N]`` or ``[C, N]``, dtype of ``x``."""
-    return _project(w, x, prefill=False)
+    return _project(w, x, prefill=False, mfma=BATCH_MFMA)
 
 
 def linear_m(w, x: torch.Tensor) -> torch.Tensor:
     """``linear_m(w, x[M, K]) -> [M, N]``: one weight read serves all rows; row r carries the bits
-    of ``linear(w, x[r])`` (unless ``BATCH_MFMA`` trades that for speed)."""
+    of ``linear(w, x[r])`` (in either setting of ``BATCH_MFMA``: both entries switch together)."""
     return _project(w, x, prefill=False, mfma=BATCH_MFMA)
 
 

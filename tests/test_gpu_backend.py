@@ -90,15 +90,22 @@ def test_int8_entries_agree_with_dequant_matmul(rows):
             assert (v.view(torch.int16) == a.view(torch.int16)).all()
 
 
-def test_batch_switch_gives_linear_m_the_matrix_pipe_kernel(monkeypatch):
+def test_batch_switch_moves_every_weight_only_call_to_the_matrix_pipe(monkeypatch):
+    """COFFIN_AMD_BATCH_MFMA: one kernel family for linear, linear_m, verify and short prefill,
+    so the static-batch contract (row r == single-row call) holds in that setting too."""
     g = synth.generator()
     q = _q8(512, 2560, g)
     x = synth.activations(8, 2560, g).to(G.DEV)
     exact = backend.linear_m(q, x)
     monkeypatch.setattr(backend, "BATCH_MFMA", True)
     fast = backend.linear_m(q, x)
-    assert (fast.view(torch.int16) == backend.linear_m_verify(q, x).view(torch.int16)).all()
     assert _rel(fast, exact.float()) < 1e-2
+    for fn in (backend.linear, backend.linear_m_verify, backend.linear_prefill):
+        assert (fn(q, x).view(torch.int16) == fast.view(torch.int16)).all()
+    for r in (0, 3, 7):
+        assert (backend.linear(q, x[r]).view(torch.int16) == fast[r].view(torch.int16)).all()
+    two = backend.linear_m(q, x[:2].contiguous())
+    assert (two.view(torch.int16) == fast[:2].view(torch.int16)).all()
 
 
 def test_prefill_switches_to_w8a8_and_matches_the_oracle(orc):
