@@ -68,7 +68,7 @@ W8A8_VERIFY = os.environ.get("COFFIN_AMD_W8A8_VERIFY", "0").strip() == "1"
 #: ``COFFIN_AMD_BATCH_MFMA=1`` moves *every* int8 weight-only call -- ``linear`` included, one row
 #: included -- to the matrix-pipe GEMV: the contract holds again (one kernel family, a row's bits
 #: independent of its batch), static batches of 4-16 requests run 1.5-3.8 times faster, and
-#: single-stream decode pays for it (9.3 us instead of 6.3 us for 2560 -> 9728).  A deployment choice.
+#: single-stream decode pays for it (7.9 us instead of 6.3 us for 2560 -> 9728).  A deployment choice.
 BATCH_MFMA = os.environ.get("COFFIN_AMD_BATCH_MFMA", "0").strip() == "1"
 #: Rows from which the matrix-pipe GEMV beats the dot-product one (measured on every layer shape).
 MFMA_MIN_ROWS = 3

@@ -81,9 +81,20 @@ gemv_w8a16_rows16_kernel(const Args a) {
     // An activation line is 256 bytes: parts 0 and 1, each fetched as two half tiles; rows past
     // M repeat the last one, their sums are dropped.
     v4i32 xr[NLP][4], wr[NLP][2];
+    // One or two activation rows: every lane's row is one of two, so the MFMA arrangement (row
+    // lane%16, bytes 64*kq .. +63 of the line) can be loaded as it is -- the requests collapse
+    // onto a few cache lines -- and the LDS rearrangement is skipped.
+    const bool direct_x = a.M <= 2;
+    const uint8_t *xdirect = xbytes + (size_t)min(lane & 15, a.M - 1) * a.K * 2 + kq * 64;
     auto request_x = [&](int r, int i) {
         const int line = line_of(r, i);
         if (line >= lines) return;  // uniform per wavefront
+        if (direct_x) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                xr[i][q] = *reinterpret_cast<const v4i32 *>(xdirect + line * 256 + q * 16);
+            return;
+        }
 #pragma unroll
         for (int q = 0; q < 4; ++q)
             xr[i][q] = *reinterpret_cast<const v4i32 *>(
@@ -109,7 +120,7 @@ gemv_w8a16_rows16_kernel(const Args a) {
         // activations into the MFMA arrangement: row lane%16, bytes 64*kq .. +63 of the line
 #pragma unroll
         for (int i = 0; i < NLP; ++i) {
-            if (line_of(r, i) >= lines) break;
+            if (direct_x || line_of(r, i) >= lines) break;
             uint8_t *p = xpatch + (lane >> 3) * XPITCH + (lane & 7) * 16;
 #pragma unroll
             for (int q = 0; q < 4; ++q)
