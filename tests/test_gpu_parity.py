@@ -461,3 +461,54 @@ def test_entry_points_raise_on_unsupported_shapes():
         G.w4a8(torch.zeros((8, 128), dtype=torch.uint8, device=G.DEV), torch.ones((8, 4), device=G.DEV),
                torch.zeros((1, 256), dtype=torch.int8, device=G.DEV), torch.ones(1, device=G.DEV),
                256, gemm=False, gs=64)
+
+
+# ------------------------------------------------------ seeded random shape sweep
+
+def _rand_shapes(seed, count, m_hi, n_hi, k_step, k_hi):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        m = int(rng.integers(1, m_hi + 1))
+        n = int(rng.integers(1, n_hi + 1))
+        k = int(rng.integers(1, k_hi // k_step + 1)) * k_step
+        out.append((m, n, k))
+    return out
+
+
+def test_random_shapes_every_kernel_against_the_oracle(orc):
+    """A seeded sweep over ragged shapes (rows, columns and K drawn independently) through every
+    entry point: the integer paths bit for bit, the weight-only paths within their bound.  One
+    process, small sizes: the oracle is the slow side."""
+    g = seeded(99)
+    # quantiser: vector path (K % 8 == 0) and scalar path (any K)
+    for m, _, k in _rand_shapes(1, 12, 40, 1, 8, 3000) + _rand_shapes(2, 6, 9, 1, 1, 700):
+        x = synth.activations(m, k, g, outliers=True)
+        q, s = G.quant(x.to(G.DEV))
+        q_ref, s_ref = orc.quant_act_i8(G.bits(x))
+        assert (q.cpu().numpy() == q_ref).all() and (s.cpu().numpy() == s_ref).all(), ("quant", m, k)
+    # int8 weight-only: dot-product kernel (K % 16) and matrix-pipe kernel (K % 128)
+    for mfma, shapes in ((False, _rand_shapes(3, 10, 16, 200, 16, 4096)),
+                         (True, _rand_shapes(4, 10, 16, 200, 128, 10240))):
+        for m, n, k in shapes:
+            wq, ws, x, y = _w8a16_case(orc, m, n, k, g, mfma=mfma)
+            exact = orc.gemv_w8a16_exact(wq, ws, G.bits(x))
+            got = y.float().cpu().numpy()
+            rms = float(np.sqrt((exact.astype(np.float64) ** 2).mean())) + 1e-30
+            assert (np.abs(got - exact) <= np.abs(exact) * WEIGHT_ONLY_EXACT_REL + 1e-5 * rms).all(), (mfma, m, n, k)
+    # W8A8: read-once kernel up to 16 rows, tiled / generic kernels beyond; K % 16
+    for m, n, k in _rand_shapes(5, 8, 16, 300, 128, 4096) + _rand_shapes(6, 8, 300, 300, 16, 1536):
+        q = synth.int8_weight(n, k, g)
+        x = synth.activations(m, k, g, outliers=True)
+        xq, xs = orc.quant_act_i8(G.bits(x))
+        acc_ref, y_ref = orc.gemm_w8a8(xq, q.wq.numpy(), xs, q.scale.numpy())
+        acc, y = G.gemm_w8a8(G.dev(xq), q.wq.to(G.DEV), G.dev(xs), q.scale.to(G.DEV))
+        assert (acc.cpu().numpy() == acc_ref).all() and (G.bits(y) == y_ref).all(), ("w8a8", m, n, k)
+    # W4A8: GEMV kernels (1..16 rows), fused quantiser (1..4 rows), GEMM (any rows); K % 128
+    for m, n, k in _rand_shapes(7, 10, 16, 200, 128, 5120) + _rand_shapes(8, 6, 150, 200, 128, 1536):
+        w4, ws, xq, xs, gacc_ref, y_ref = _w4_case(orc, m, n, k, g)
+        if m <= 16:
+            gacc, y = G.w4a8(w4, ws, xq, xs, k, gemm=False)
+            assert (gacc.cpu().numpy() == gacc_ref).all() and (G.bits(y) == y_ref).all(), ("w4 gemv", m, n, k)
+        gacc, y = G.w4a8(w4, ws, xq, xs, k, gemm=True)
+        assert (gacc.cpu().numpy() == gacc_ref).all() and (G.bits(y) == y_ref).all(), ("w4 gemm", m, n, k)
