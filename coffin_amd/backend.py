@@ -75,9 +75,11 @@ MFMA_MIN_ROWS = 3
 #: W4A8 switches from the GEMV to the MFMA GEMM above this many rows.
 W4_GEMM_MIN_ROWS = 17
 #: Up to this many rows the W4A8 GEMV quantises its activations itself (one launch); the
-#: kernel takes up to 4, but from 2 rows on every workgroup redoing the divisions costs more
-#: than the separate quantiser launch.
+#: kernel takes up to 4, but from 2 rows on every workgroup redoing the quantisation costs more
+#: than the separate quantiser launch -- except on long rows (K > 5120), where two rows still
+#: win (10.8 us against 12.7 us at 9728 -> 2560).
 W4_FUSED_MAX_ROWS = 1
+W4_FUSED_MAX_ROWS_LONG_K = 2
 
 def _vp(address: int) -> int:
     """Pointer argument: the entry points declare ``void *`` (``argtypes``), so a plain int passes."""
@@ -264,7 +266,7 @@ def _gemm_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> N
 def _rows_w4(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> None:
     n, k, gs = rec.n, rec.k, rec.gs
     lib = _native.load()
-    if rows <= W4_FUSED_MAX_ROWS:
+    if rows <= (W4_FUSED_MAX_ROWS_LONG_K if k > 5120 else W4_FUSED_MAX_ROWS):
         # decode: one launch, activations quantised inside the GEMV (same bits)
         rc = lib.cmi_gemv_w4a8_bf16(rec.a, rec.b, act.data_ptr(), out.data_ptr(), 0, 0, 0,
                                     rows, n, k, gs, _stream())

@@ -36,10 +36,11 @@ int gemm_w8a8_rows16(const int8_t *xq, const int8_t *wq, const float *xs, const 
 int gemv_w4a8_decode(const uint8_t *w4, const float *ws, const void *x, const int8_t *xq, const float *xs,
                      void *y, int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
                      void *stream);
-// gemv_w4a8_rows16.hip: W4A8 GEMV for up to 16 already quantised rows, K <= 10240, integer
-// sums on the matrix pipe; CMI_E_UNSUPPORTED (no error text) outside that range.
-int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs, void *y,
-                     int32_t *group_acc, int M, int N, int K, void *stream);
+// gemv_w4a8_rows16.hip: W4A8 GEMV for up to 16 quantised rows (xq, xs) or up to 4 bf16 rows (x,
+// quantised in the kernel), K <= 10240, integer sums on the matrix pipe; CMI_E_UNSUPPORTED (no error text) outside that range.
+int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs, const void *x,
+                     void *y, int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
+                     void *stream);
 static inline bool aligned(const void *p, uintptr_t a) {
     return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
 }

@@ -346,7 +346,7 @@ extern "C" int cmi_gemv_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     if (gs == GS && N >= 1 && M >= 1) {
         // 1..2 rows: dot-product kernel; 3..16: group sums on the matrix pipe (measured faster from 3 up)
         const int rc = M <= 2 ? gemv_w4a8_decode(w4, ws, nullptr, xq, xs, y, group_acc, nullptr, nullptr, M, N, K, stream)
-                              : gemv_w4a8_rows16(w4, ws, xq, xs, y, group_acc, M, N, K, stream);
+                              : gemv_w4a8_rows16(w4, ws, xq, xs, nullptr, y, group_acc, nullptr, nullptr, M, N, K, stream);
         if (rc != CMI_E_UNSUPPORTED) return rc;
     }
     return run_gemv_w4a8("cmi_gemv_w4a8", w4, ws, xq, xs, nullptr, nullptr, nullptr, y, group_acc, M, N, K, gs,
@@ -365,8 +365,14 @@ extern "C" int cmi_gemv_w4a8_bf16(const uint8_t *w4, const float *ws, const void
     CMI_REQUIRE(N >= 1 && K >= GS, CMI_E_ARG, "cmi_gemv_w4a8_bf16: bad shape N=%d K=%d", N, K);
     CMI_REQUIRE(gs == GS, CMI_E_UNSUPPORTED, "cmi_gemv_w4a8_bf16: group size %d, kernels are built for %d", gs, GS);
     CMI_REQUIRE(K % GS == 0, CMI_E_UNSUPPORTED, "cmi_gemv_w4a8_bf16: K=%d is not a multiple of %d", K, GS);
-    // the decode kernel (whole rows requested up front) where it applies, else the general one
-    const int rc = gemv_w4a8_decode(w4, ws, x, nullptr, nullptr, y, group_acc, xq_out, xs_out, M, N, K, stream);
+    // long rows: the matrix-pipe kernel with the quantiser folded in (the dot-product kernel shares
+    // such rows among wavefronts and its fp32 chain serialises: 10.5 us at 9728 -> 2560); else the
+    // decode kernel (whole rows requested up front) where it applies, else the general one
+    int rc = CMI_E_UNSUPPORTED;
+    if (K > 5120)
+        rc = gemv_w4a8_rows16(w4, ws, nullptr, nullptr, x, y, group_acc, xq_out, xs_out, M, N, K, stream);
+    if (rc != CMI_E_UNSUPPORTED) return rc;
+    rc = gemv_w4a8_decode(w4, ws, x, nullptr, nullptr, y, group_acc, xq_out, xs_out, M, N, K, stream);
     if (rc != CMI_E_UNSUPPORTED) return rc;
     return run_gemv_w4a8("cmi_gemv_w4a8_bf16", w4, ws, nullptr, nullptr, x, xq_out, xs_out, y, group_acc, M, N, K,
                          gs, stream);

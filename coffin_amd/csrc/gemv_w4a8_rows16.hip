@@ -25,6 +25,7 @@
 // -8s (the matrix pipe is idle here).  Each wavefront parks its int32 group sums
 // in LDS and, after one barrier, thread (n, m) walks the groups in ascending
 // order.
+#include "quant_math.hpp"
 #include "rows16_tile.hpp"
 
 namespace {
@@ -38,22 +39,33 @@ constexpr int GS = 128;
 constexpr int ROWS = 16;        // weight rows per workgroup = activation rows per MFMA
 constexpr int MAX_K = 10240;    // 40 lines: 8 wavefronts x 5
 
+constexpr int FUSED_ROWS = 4;   // rows the kernel quantises itself (bf16 activations in)
+constexpr int FUSED_XV = 3;     // 16-byte bf16 vectors per thread and row: K <= 3 * 8 * threads
+
 struct Args {
     const uint8_t *w4;
     const float *ws;
-    const int8_t *xq;
+    const int8_t *xq;     // quantised activations and their scales, or
     const float *xs;
+    const uint16_t *x;    // bf16 activations (FUSED), with optional copies of what was quantised
+    int8_t *xq_out;
+    float *xs_out;
     uint16_t *y;
     int32_t *group_acc;
     int M, N, K, G;
 };
 
-// group sums [G][64 lanes][4], scales [16][G], one rearrangement patch per wavefront
-__host__ __device__ inline int lds_bytes(int G, int waves) { return G * 1024 + ROWS * G * 4 + waves * PATCH_BYTES; }
+// group sums [G][64 lanes][4], scales [16][G], one rearrangement patch per wavefront; FUSED adds
+// the int8 rows [4][K], their scales and the per-wavefront maxima
+__host__ __device__ inline int lds_bytes(int G, int waves, bool fused = false) {
+    return G * 1024 + ROWS * G * 4 + waves * PATCH_BYTES + (fused ? FUSED_ROWS * G * GS + 256 : 0);
+}
 
 // NLP: lines per wavefront.  WAVES: wavefronts per workgroup (4 or 8).
 // DUMP: also write the int32 group sums to a.group_acc.
-template <int NLP, int WAVES, bool DUMP>
+// FUSED: activations arrive as bf16 (up to 4 rows) and every workgroup quantises them itself
+//        with the arithmetic of cmi_quant_act_i8 while its weights travel.
+template <int NLP, int WAVES, bool DUMP, bool FUSED>
 __global__ void __launch_bounds__(WAVES * 64)
 gemv_w4a8_rows16_kernel(const Args a) {
     extern __shared__ __align__(16) uint8_t lds[];
@@ -61,6 +73,9 @@ gemv_w4a8_rows16_kernel(const Args a) {
     float *ws_lds = reinterpret_cast<float *>(lds + a.G * 1024);  // [16][G]
 
     uint8_t *patches = lds + a.G * 1024 + ROWS * a.G * 4;
+    int8_t *xq_lds = reinterpret_cast<int8_t *>(patches + WAVES * PATCH_BYTES);             // FUSED: [4][K]
+    float *xs_lds = reinterpret_cast<float *>(patches + WAVES * PATCH_BYTES + FUSED_ROWS * a.K);  // [4]
+    float *part = xs_lds + 8;                                                                // [4][WAVES]
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -72,16 +87,32 @@ gemv_w4a8_rows16_kernel(const Args a) {
     // 1. activations of this wavefront's groups (L2 resident; asked for first because
     //    memory answers in request order); rows past M repeat the last one, their sums are dropped
     v4i32 xa[NLP][2][2];
+    uint4 xv[FUSED ? FUSED_ROWS : 1][FUSED ? FUSED_XV : 1];
+    const int xvecs = a.K / 8;
+    if constexpr (FUSED) {
 #pragma unroll
-    for (int i = 0; i < NLP; ++i) {
-        const int line = wave + i * WAVES;
-        if (line >= lines) break;  // uniform per wavefront
+        for (int m = 0; m < FUSED_ROWS; ++m) {
+            if (m >= a.M) break;  // uniform
+            const uint4 *xg = reinterpret_cast<const uint4 *>(a.x + (size_t)m * a.K);
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int g = min(2 * line + h, a.G - 1);
+            for (int j = 0; j < FUSED_XV; ++j) {
+                const int idx = threadIdx.x + j * (WAVES * 64);
+                xv[m][j] = idx < xvecs ? xg[idx] : make_uint4(0, 0, 0, 0);
+            }
+        }
+    } else {
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                xa[i][h][j] = *reinterpret_cast<const v4i32 *>(a.xq + tile_src(lane, j, 0, a.M - 1, a.K, g * GS));
+        for (int i = 0; i < NLP; ++i) {
+            const int line = wave + i * WAVES;
+            if (line >= lines) break;  // uniform per wavefront
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int g = min(2 * line + h, a.G - 1);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    xa[i][h][j] =
+                        *reinterpret_cast<const v4i32 *>(a.xq + tile_src(lane, j, 0, a.M - 1, a.K, g * GS));
+            }
         }
     }
     // 2. the scales of the 16 rows (contiguous), into registers until the weights are asked for
@@ -113,16 +144,67 @@ gemv_w4a8_rows16_kernel(const Args a) {
         if (idx < ws_total) ws_lds[idx] = wsreg[i];
     }
 
-    // 4. into the MFMA arrangement: activations pieces 2kq, 2kq+1 of row lane%16 per group
+    // 4. activations into the MFMA arrangement: row lane%16, bytes 32*kq .. +31 of each group
+    if constexpr (FUSED) {
+        // quantise the rows into LDS first (same bits as cmi_quant_act_i8), then read the pieces
 #pragma unroll
-    for (int i = 0; i < NLP; ++i) {
-        const int line = wave + i * WAVES;
-        if (line >= lines) break;
+        for (int m = 0; m < FUSED_ROWS; ++m) {
+            if (m >= a.M) break;  // uniform
+            float amax = 0.f;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            tile_park(patch, lane, xa[i][h][0], xa[i][h][1]);
-            xa[i][h][0] = tile_take(patch, lane, 2 * kq);
-            xa[i][h][1] = tile_take(patch, lane, 2 * kq + 1);
+            for (int j = 0; j < FUSED_XV; ++j)
+                if (j * (WAVES * 64) < xvecs) amax = absmax8(xv[m][j], amax);  // uniform
+            amax = wave_max_to_lane63(amax);
+            if (lane == 63) part[m * WAVES + wave] = amax;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int m = 0; m < FUSED_ROWS; ++m) {
+            if (m >= a.M) break;  // uniform
+            float amax = part[m * WAVES];
+#pragma unroll
+            for (int wv = 1; wv < WAVES; ++wv) amax = fmaxf(amax, part[m * WAVES + wv]);
+            const RowScale rs = row_scale(amax);
+            if (threadIdx.x == 0) {
+                xs_lds[m] = rs.sc;
+                if (a.xs_out && blockIdx.x == 0) a.xs_out[m] = rs.sc;
+            }
+#pragma unroll
+            for (int j = 0; j < FUSED_XV; ++j) {
+                const int idx = threadIdx.x + j * (WAVES * 64);
+                if (j * (WAVES * 64) >= xvecs) break;  // uniform
+                const uint2 q = quant8(xv[m][j], rs);
+                if (idx < xvecs) {
+                    reinterpret_cast<uint2 *>(xq_lds + (size_t)m * a.K)[idx] = q;
+                    if (a.xq_out && blockIdx.x == 0)
+                        reinterpret_cast<uint2 *>(a.xq_out + (size_t)m * a.K)[idx] = q;
+                }
+            }
+        }
+        __syncthreads();
+        const int8_t *xrow = xq_lds + (size_t)min(lane & 15, min(a.M, FUSED_ROWS) - 1) * a.K + kq * 32;
+#pragma unroll
+        for (int i = 0; i < NLP; ++i) {
+            const int line = wave + i * WAVES;
+            if (line >= lines) break;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int g = min(2 * line + h, a.G - 1);
+                xa[i][h][0] = *reinterpret_cast<const v4i32 *>(xrow + g * GS);
+                xa[i][h][1] = *reinterpret_cast<const v4i32 *>(xrow + g * GS + 16);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < NLP; ++i) {
+            const int line = wave + i * WAVES;
+            if (line >= lines) break;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                tile_park(patch, lane, xa[i][h][0], xa[i][h][1]);
+                xa[i][h][0] = tile_take(patch, lane, 2 * kq);
+                xa[i][h][1] = tile_take(patch, lane, 2 * kq + 1);
+            }
         }
     }
     // 5. integer group sums: lane holds (n = lane%16, m = 4*kq + v), v = 0..3
@@ -180,41 +262,54 @@ gemv_w4a8_rows16_kernel(const Args a) {
                 if constexpr (DUMP) a.group_acc[((size_t)m * a.G + g) * a.N + n] = sg;
                 total = fmaf((float)sg, wsn[g], total);
             }
-            a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * a.xs[m]);
+            const float xsm = FUSED ? xs_lds[m] : a.xs[m];
+            a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * xsm);
         }
     }
 }
 
-template <int NLP, int WAVES, bool DUMP>
+template <int NLP, int WAVES, bool DUMP, bool FUSED>
 int launch_one(const Args &a, hipStream_t st) {
     static std::atomic<uint64_t> devices{0};
-    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w4a8_rows16_kernel<NLP, WAVES, DUMP>),
-                                   lds_bytes(MAX_K / GS, WAVES), devices, "cmi_gemv_w4a8"))
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w4a8_rows16_kernel<NLP, WAVES, DUMP, FUSED>),
+                                   lds_bytes(MAX_K / GS, WAVES, FUSED), devices, "cmi_gemv_w4a8"))
         return rc;
     const dim3 grid((a.N + ROWS - 1) / ROWS);
-    gemv_w4a8_rows16_kernel<NLP, WAVES, DUMP><<<grid, dim3(WAVES * 64), lds_bytes(a.G, WAVES), st>>>(a);
+    gemv_w4a8_rows16_kernel<NLP, WAVES, DUMP, FUSED>
+        <<<grid, dim3(WAVES * 64), lds_bytes(a.G, WAVES, FUSED), st>>>(a);
     return check_launch("cmi_gemv_w4a8");
 }
 
 template <int NLP, int WAVES>
 int launch(const Args &a, hipStream_t st) {
-    return a.group_acc ? launch_one<NLP, WAVES, true>(a, st) : launch_one<NLP, WAVES, false>(a, st);
+    if (a.x) {
+        if (a.K > FUSED_XV * 8 * WAVES * 64) return CMI_E_UNSUPPORTED;
+        return a.group_acc ? launch_one<NLP, WAVES, true, true>(a, st) : launch_one<NLP, WAVES, false, true>(a, st);
+    }
+    return a.group_acc ? launch_one<NLP, WAVES, true, false>(a, st) : launch_one<NLP, WAVES, false, false>(a, st);
 }
 
 }  // namespace
 
 namespace cmi {
 
-// Returns CMI_E_UNSUPPORTED without setting the error text when the shape is
-// outside this kernel's range (the caller then uses the general kernel).
-int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs, void *y,
-                     int32_t *group_acc, int M, int N, int K, void *stream) {
-    if (M < 1 || M > ROWS || K < GS || K > MAX_K || K % GS != 0 || N < 1) return CMI_E_UNSUPPORTED;
+// Exactly one of xq/xs (quantised rows, up to 16) and x (bf16 rows, up to 4: the kernel quantises
+// them itself and copies what it used to xq_out / xs_out when given) is set.  Returns
+// CMI_E_UNSUPPORTED without setting the error text when the shape is outside this kernel's range
+// (the caller then uses another kernel).
+int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs, const void *x,
+                     void *y, int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
+                     void *stream) {
+    if (M < 1 || M > (x ? FUSED_ROWS : ROWS) || K < GS || K > MAX_K || K % GS != 0 || N < 1)
+        return CMI_E_UNSUPPORTED;
     Args a;
     a.w4 = w4;
     a.ws = ws;
     a.xq = xq;
     a.xs = xs;
+    a.x = static_cast<const uint16_t *>(x);
+    a.xq_out = xq_out;
+    a.xs_out = xs_out;
     a.y = static_cast<uint16_t *>(y);
     a.group_acc = group_acc;
     a.M = M;
