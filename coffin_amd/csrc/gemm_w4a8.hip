@@ -21,6 +21,9 @@
 //   - the integer accumulators restart every step (first MFMA of a group takes
 //     C = 0); the flush is 64 converts + 64 fmas per lane and step, which is why
 //     two workgroups share a CU: one flushes while the other multiplies.
+#include <cmath>
+#include <cstdlib>
+
 #include "common.hpp"
 
 #include <type_traits>
@@ -289,6 +292,8 @@ gemm_w4a8_kernel(const Args a) {
 
 }  // namespace
 
+static inline int a_ceil(int a, int b) { return (a + b - 1) / b; }
+
 extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs,
                              void *y, int32_t *group_acc, int M, int N, int K, int gs,
                              void *stream) {
@@ -299,6 +304,28 @@ extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     CMI_REQUIRE(K % BK == 0, CMI_E_UNSUPPORTED, "cmi_gemm_w4a8: K=%d is not a multiple of %d", K, BK);
     CMI_REQUIRE(aligned(xq, 16) && aligned(w4, 16), CMI_E_ARG,
                 "cmi_gemm_w4a8: xq and w4 must be 16-byte aligned");
+    // Few rows: the tile pipeline is latency-bound (K/128 steps of ~1.2 us whatever M is), while the
+    // matrix-pipe GEMV reads the weight once per 16 rows at memory speed; same integer sums, same
+    // fp32 chain, same bits.  Cost model fitted to measurements on the layer shapes (us).
+    const char *force = getenv("CMI_GEMM_TILE");
+    if (M <= 256 && K <= 10240 && !(force && force[0])) {
+        const double steps = K / 128.0;
+        const double tiles = (double)a_ceil(M, BM) * a_ceil(N, BN);
+        const double t_tiled = 3.0 + steps * 1.17 * ceil(tiles / 512.0);
+        const double t_rows16 = a_ceil(M, 16) * (3.6 + (double)N * K / 2 / 4.2e6 + steps * 0.025);
+        if (t_rows16 < t_tiled) {
+            const int G = K / BK;
+            for (int lo = 0; lo < M; lo += 16) {
+                const int m = M - lo < 16 ? M - lo : 16;
+                const int rc = gemv_w4a8_rows16(w4, ws, xq + (size_t)lo * K, xs + lo, nullptr,
+                                                static_cast<uint16_t *>(y) + (size_t)lo * N,
+                                                group_acc ? group_acc + (size_t)lo * G * N : nullptr, nullptr,
+                                                nullptr, m, N, K, stream);
+                if (rc != CMI_OK) return rc == CMI_E_UNSUPPORTED ? fail(rc, "cmi_gemm_w4a8: internal dispatch") : rc;
+            }
+            return CMI_OK;
+        }
+    }
     Args a;
     a.xq = xq;
     a.w4 = w4;

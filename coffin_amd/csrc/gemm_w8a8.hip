@@ -729,6 +729,25 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
         const int rc = gemm_w8a8_rows16(xq, wq, xs, ws, y, acc_out, M, N, K, ldy, stream);
         if (rc != CMI_E_UNSUPPORTED) return rc;
     }
+    if (M > 16 && M <= 256 && K % 128 == 0 && K <= 10240 && !(force && force[0])) {
+        // Few rows: the tile pipeline is latency-bound (K/128 steps of ~0.9 us whatever M is), the
+        // read-once kernel runs at memory speed per 16 rows; same bits.  Cost model fitted to
+        // measurements on the layer shapes (us).
+        const double steps = K / 128.0;
+        const double tiles = (double)((M + 127) / 128) * ((N + 127) / 128);
+        const double t_tiled = 2.5 + steps * 0.9 * ceil(tiles / 512.0);
+        const double t_rows16 = ((M + 15) / 16) * (3.2 + (double)N * K / 6.0e6);
+        if (t_rows16 < t_tiled) {
+            for (int lo = 0; lo < M; lo += 16) {
+                const int m = M - lo < 16 ? M - lo : 16;
+                const int rc = gemm_w8a8_rows16(xq + (size_t)lo * K, wq, xs + lo, ws,
+                                                static_cast<uint16_t *>(y) + (size_t)lo * ldy,
+                                                acc_out ? acc_out + (size_t)lo * N : nullptr, m, N, K, ldy, stream);
+                if (rc != CMI_OK) return rc == CMI_E_UNSUPPORTED ? fail(rc, "cmi_gemm_w8a8: internal dispatch") : rc;
+            }
+            return CMI_OK;
+        }
+    }
     if (K % BK != 0 || N < 8) return gemm_w8a8_generic(xq, wq, xs, ws, y, acc_out, M, N, K, ldy, stream);
     Args a;
     a.xq = xq;
