@@ -730,12 +730,12 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
         if (rc != CMI_E_UNSUPPORTED) return rc;
     }
     if (M > 16 && M <= 256 && K % 128 == 0 && K <= 10240 && !(force && force[0])) {
-        // Few rows: the tile pipeline is latency-bound (K/128 steps of ~0.9 us whatever M is), the
-        // read-once kernel runs at memory speed per 16 rows; same bits.  Cost model fitted to
-        // measurements on the layer shapes (us).
+        // Few rows: the tile pipeline is latency-bound (K/128 dependent steps of ~0.5 us with three
+        // LDS stages, ~0.9 us with two, whatever M is), the read-once kernel runs at memory speed per
+        // 16 rows; same bits.  Cost model fitted to measurements on the layer shapes (us).
         const double steps = K / 128.0;
         const double tiles = (double)((M + 127) / 128) * ((N + 127) / 128);
-        const double t_tiled = 2.5 + steps * 0.9 * ceil(tiles / 512.0);
+        const double t_tiled = 2.5 + steps * (tiles <= 256 ? 0.5 : 0.9 * ceil(tiles / 512.0));
         const double t_rows16 = ((M + 15) / 16) * (3.2 + (double)N * K / 6.0e6);
         if (t_rows16 < t_tiled) {
             for (int lo = 0; lo < M; lo += 16) {
@@ -782,5 +782,11 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
     }
     if (pick == 320) return launch_wide(a, st);
     const bool use_big = pick == 256;
-    return use_big ? launch_big(a, st) : launch<2, 2, 2>(a, st);
+    if (use_big) return launch_big(a, st);
+    // Up to one 128 x 128 workgroup per CU the launch is a chain of K/128 dependent steps: a third
+    // LDS stage (96 KiB, one workgroup per CU anyway) puts two steps of loads in flight (-20 % at
+    // K = 2560, -33 % at K = 9728); with two workgroups per CU it measured slower.
+    const int tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+    if (tiles128 <= 256) return launch<2, 2, 3>(a, st);
+    return launch<2, 2, 2>(a, st);
 }
