@@ -45,6 +45,25 @@ class QWeight:
             scale[lo:hi] = s
         return cls(wq, scale)
 
+    @classmethod
+    def from_kn(cls, wt: torch.Tensor, scale: torch.Tensor) -> "QWeight":
+        """Wrap an int8 ``[K, N]`` buffer without copying (int8_weights.py:271-305).
+
+        ``wq`` becomes the transposed view, strides ``(1, N)``.  The MI355X
+        kernels stream ``[N, K]`` rows, so the backend adapter makes its own
+        row-major copy of such a weight the first time it is used.
+        """
+        if wt.dim() != 2 or wt.dtype != torch.int8:
+            raise ValueError(f"packed int8 weight must be 2-D int8, got "
+                             f"{tuple(wt.shape)} {wt.dtype}")
+        if scale.dim() != 1 or scale.dtype != torch.float32:
+            raise ValueError("scale must be 1-D fp32")
+        if int(scale.numel()) != int(wt.shape[1]):
+            raise ValueError(f"scale holds {scale.numel()} values for N = {int(wt.shape[1])}")
+        if not wt.is_contiguous():
+            raise ValueError("packed [K, N] weight must be contiguous")
+        return cls(wt.t(), scale)
+
     def dequant(self, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
         """Dense ``[N, K]``: one fp32 product, one narrowing (int8_weights.py:359)."""
         return (self.wq.to(torch.float32) * self.scale.unsqueeze(1)).to(dtype)

@@ -61,6 +61,19 @@ def test_reference_linear_assertions_on_device():
     assert _rel(backend.linear_prefill(q, X[:3]), X[:3] @ dense.t()) < FP32_TOL
 
 
+def test_kn_stored_weight_gives_the_bits_of_the_row_major_one():
+    # QWeight.from_kn hands the adapter a transposed view; it answers from one private row-major copy
+    g = synth.generator()
+    q = _q8(1536, 2560, g)
+    kn = QWeight.from_kn(q.wq.t().contiguous(), q.scale)
+    for rows in (1, 4, 16, 96):
+        x = synth.activations(rows, 2560, g).to(G.DEV)
+        for fn in (backend.linear_m, backend.linear_m_verify, backend.linear_prefill):
+            a, b = fn(q, x), fn(kn, x)
+            assert (a.view(torch.int16) == b.view(torch.int16)).all(), (fn.__name__, rows)
+    assert (backend.linear(q, x[0]).view(torch.int16) == backend.linear(kn, x[0]).view(torch.int16)).all()
+
+
 @pytest.mark.parametrize("rows", [None, 1, 2, 8, 16, 17, 40])
 def test_int8_entries_agree_with_dequant_matmul(rows):
     g = synth.generator()

@@ -70,6 +70,25 @@ def test_qweight_matches_oracle_and_surface(orc):
     assert (z.wq == 0).all() and torch.isfinite(z.scale).all()
 
 
+def test_qweight_from_kn_is_a_view_and_validates():
+    # int8_weights.py:271-305: a [K, N] buffer wrapped without a copy; wq is the transposed view
+    g = synth.generator()
+    q = synth.int8_weight(12, 40, g)
+    wt = q.wq.t().contiguous()
+    v = QWeight.from_kn(wt, q.scale)
+    assert (v.n, v.k) == (12, 40) and v.wq.stride() == (1, 12)
+    assert v.wq.data_ptr() == wt.data_ptr() and (v.wq == q.wq).all()
+    assert (v.dequant(torch.float32) == q.dequant(torch.float32)).all()
+    with pytest.raises(ValueError, match="2-D int8"):
+        QWeight.from_kn(wt.float(), q.scale)
+    with pytest.raises(ValueError, match="1-D fp32"):
+        QWeight.from_kn(wt, q.scale.double())
+    with pytest.raises(ValueError, match="N = 12"):
+        QWeight.from_kn(wt, q.scale[:5])
+    with pytest.raises(ValueError, match="contiguous"):
+        QWeight.from_kn(q.wq.t(), q.scale)
+
+
 def test_w4_weight_matches_oracle_and_validates(orc):
     g = synth.generator()
     w = synth.dense_weight(20, 200, g)                     # K not a multiple of the group
