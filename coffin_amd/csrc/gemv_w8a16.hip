@@ -61,6 +61,7 @@ struct GemvArgs {
     uint32_t xvecs_rcp;  // ceil(2^32 / (K/8)): idx / (K/8) == umulhi(idx, xvecs_rcp) for idx < 2^16
     int nblocks;    // ceil(N / R)
     int uw;         // wavefronts of a team (they stride over the units)
+    uint32_t uw_rcp;  // ceil(2^16 / uw)
     int teams;      // row blocks per workgroup
 };
 
@@ -108,8 +109,10 @@ __host__ __device__ constexpr int xlds_vectors(int mt, int rows, int K, int segs
 // 4 wavefronts per SIMD need; a spill inside the K loop costs a memory round trip each).
 constexpr int m_tile(int m) { return m < 4 ? m : 4; }
 
-// 16-byte vectors of activations each thread carries from global memory to LDS.
+// 16-byte vectors of activations each thread can carry from global memory to LDS, and the
+// short variant compiled for one or two rows of ordinary width (K up to 4096 at four wavefronts).
 constexpr int xstage_vectors(int m) { return m <= 1 ? 8 : m <= 2 ? 16 : m <= 4 ? 20 : 8; }
+constexpr int xstage_short(int m) { return m <= 1 ? 2 : m <= 2 ? 4 : xstage_vectors(m); }
 
 template <int M, int CHT>
 struct XStage {
@@ -126,13 +129,16 @@ struct WStage {
 // MODE 2: general: units walked in pipelined sub-trips.
 // XLDS: the workgroup stages the activations in LDS; otherwise each wavefront
 //       reads them from global memory (only when they do not fit).
-template <int M, int R, int CHT, int MODE, bool XLDS>
+// XV: 16-byte vectors of activations each thread carries from global memory to LDS.
+template <int M, int R, int CHT, int MODE, bool XLDS, int XV>
 __global__ void __launch_bounds__(64 * block_waves(M), simd_waves(M, CHT))
 gemv_w8a16_kernel(const GemvArgs a) {
     extern __shared__ uint4 smem[];  // staged activations (XLDS, see xlds_vectors), then unit totals
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int team = wave / a.uw;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: row addresses stay scalar
+    // a single unit means one wavefront per team; otherwise wave / uw through a 16-bit reciprocal
+    // (exact for the at most 16 wavefronts of a workgroup)
+    const int team = MODE == 0 ? wave : (int)(((uint32_t)wave * a.uw_rcp) >> 16);
     const int rb = blockIdx.x * a.teams + team;
     const bool idle = rb >= a.nblocks;  // only in the last workgroup
     int u = wave - team * a.uw;         // unit in hand; the team's wavefronts stride over units
@@ -141,12 +147,12 @@ gemv_w8a16_kernel(const GemvArgs a) {
     float *unit_total = reinterpret_cast<float *>(smem + (XLDS ? xlds_vectors(M, a.M, a.K, segs) : 0)) +
                         team * a.units * (R * M);
 
-    const u32x4 *wrow[R];
+    const int8_t *wrow[R];  // uniform per wavefront
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         int n = rb * R + r;
         n = n < a.N ? n : a.N - 1;
-        wrow[r] = reinterpret_cast<const u32x4 *>(a.wq + (size_t)n * a.K);
+        wrow[r] = a.wq + (size_t)n * a.K;
     }
 
     // Loads are unconditional: a dead chunk's address is clamped to the row's
@@ -158,7 +164,8 @@ gemv_w8a16_kernel(const GemvArgs a) {
 #pragma unroll
             for (int j = 0; j < CHT; ++j) {
                 const int chunk = (unit_idx * a.unit + t * CHT + j) * 64 + lane;
-                s.w[r][j] = __builtin_nontemporal_load(wrow[r] + min(chunk, a.nchunks - 1));
+                s.w[r][j] = __builtin_nontemporal_load(
+                    reinterpret_cast<const u32x4 *>(wrow[r] + (uint32_t)min(chunk, a.nchunks - 1) * 16u));
             }
     };
     constexpr int MT = m_tile(M), MH = M / MT;
@@ -232,11 +239,12 @@ gemv_w8a16_kernel(const GemvArgs a) {
     // wavefront waits for must have been requested before the long weight
     // stream), then all first-trip weights, then the LDS hand-over: the copy and
     // its barrier run in the shadow of the weight latency.
-    constexpr int XV = xstage_vectors(M);
     uint4 xstage[XV];
     const int xtotal = a.M * xvecs;
     if constexpr (XLDS) {
         const uint4 *xg = reinterpret_cast<const uint4 *>(a.x);
+        // (the zero of the idle threads also keeps the compiler from moving a load down to the
+        // predicated LDS store that consumes it, behind the weight requests)
 #pragma unroll
         for (int j = 0; j < XV; ++j) {
             const int idx = threadIdx.x + j * blockDim.x;
@@ -245,11 +253,16 @@ gemv_w8a16_kernel(const GemvArgs a) {
     }
     WStage<R, CHT> w0;
     load_w(w0, min(u, a.units - 1), 0);
+    // Row scales: uniform per wavefront, but fetched as vector loads behind the weights (the
+    // opaque zero keeps the address in a vector register).  As scalar loads they would share the
+    // LDS counter and sit in front of the barrier of the activation hand-over.
+    int vzero = 0;
+    asm volatile("" : "+v"(vzero));
     float scale[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         const int n = rb * R + r;
-        scale[r] = a.ws[n < a.N ? n : a.N - 1];
+        scale[r] = a.ws[(n < a.N ? n : a.N - 1) + vzero];
     }
     if constexpr (XLDS) {
 #pragma unroll
@@ -258,13 +271,14 @@ gemv_w8a16_kernel(const GemvArgs a) {
             // Within a segment (64 chunks of 16 weights) the first halves of all chunks
             // come first, then the second halves: a wavefront's 16-byte reads are then
             // contiguous across lanes (no bank conflicts).
+            const bool mine = idx < xtotal;
             if constexpr (M >= 4) {
                 const int row = __umulhi((uint32_t)idx, a.xvecs_rcp);
                 const int v = idx - row * xvecs;
                 const int seg = v >> 7, half = v & 1, c = (v & 127) >> 1;
-                if (idx < xtotal) smem[(seg * M + row) * 128 + half * 64 + c] = xstage[j];
+                if (mine) smem[(seg * M + row) * 128 + half * 64 + c] = xstage[j];
             } else {
-                if (idx < xtotal) smem[idx] = xstage[j];  // little LDS traffic: plain order
+                if (mine) smem[idx] = xstage[j];  // little LDS traffic: plain order
             }
         }
         if constexpr (M >= 4) {
@@ -400,9 +414,22 @@ Plan make_plan(int M, int N, int K) {
     const int subtrips = (unit + p.cht - 1) / p.cht;
     p.cht = (unit + subtrips - 1) / subtrips;
     p.mode = subtrips > 1 ? 2 : units > 1 ? 1 : 0;
-    p.r = 2;
-    (void)N;
+    // Two weight rows per wavefront share the activation fragments.  A single row of a small
+    // weight is latency-bound instead: one row per wavefront halves the arithmetic left to do
+    // when a wavefront's last bytes arrive (4096 -> 2560: 4.4 -> 4.1 us); from ~20 MB on the
+    // launch is throughput-bound and the shared fragments win.
+    p.r = (M == 1 && p.mode == 0 && (size_t)N * K <= ((size_t)20 << 20)) ? 1 : 2;
     return p;
+}
+
+template <int M, int R, int CHT, int MODE, bool XLDS, int XV>
+int launch_xv(const GemvArgs &a, const dim3 grid, const dim3 block, size_t lds, hipStream_t st) {
+    static std::atomic<uint64_t> devices{0};
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w8a16_kernel<M, R, CHT, MODE, XLDS, XV>),
+                                   128 * 1024, devices, "cmi_gemv_w8a16"))
+        return rc;
+    gemv_w8a16_kernel<M, R, CHT, MODE, XLDS, XV><<<grid, block, lds, st>>>(a);
+    return check_launch("cmi_gemv_w8a16");
 }
 
 template <int M, int R, int CHT, int MODE, bool XLDS>
@@ -411,17 +438,17 @@ int launch(GemvArgs &a, hipStream_t st) {
     a.subtrips = (a.unit + CHT - 1) / CHT;
     a.xvecs_rcp = (uint32_t)(((1ull << 32) + (a.K / 8) - 1) / (a.K / 8));
     a.uw = a.units < 4 ? a.units : 4;
+    a.uw_rcp = (65536u + a.uw - 1) / a.uw;
     a.teams = block_waves(M) / a.uw;
     const dim3 grid((a.nblocks + a.teams - 1) / a.teams);
     const dim3 block(64 * a.uw * a.teams);
     const size_t lds = (XLDS ? 16 * (size_t)xlds_vectors(M, a.M, a.K, a.units * a.unit) : 0) +
                        (MODE == 0 ? 0 : sizeof(float) * a.teams * a.units * R * M);
-    static std::atomic<uint64_t> devices{0};
-    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w8a16_kernel<M, R, CHT, MODE, XLDS>),
-                                   128 * 1024, devices, "cmi_gemv_w8a16"))
-        return rc;
-    gemv_w8a16_kernel<M, R, CHT, MODE, XLDS><<<grid, block, lds, st>>>(a);
-    return check_launch("cmi_gemv_w8a16");
+    if constexpr (XLDS && xstage_short(M) < xstage_vectors(M)) {
+        if ((size_t)a.M * (a.K / 8) <= (size_t)xstage_short(M) * block.x)
+            return launch_xv<M, R, CHT, MODE, XLDS, xstage_short(M)>(a, grid, block, lds, st);
+    }
+    return launch_xv<M, R, CHT, MODE, XLDS, xstage_vectors(M)>(a, grid, block, lds, st);
 }
 
 // Whether a workgroup of the M-tile's kernel can carry [rows, K] activations into LDS.
@@ -463,10 +490,8 @@ int dispatch_ch(GemvArgs &a, const Plan &p, hipStream_t st) {
 
 template <int M>
 int dispatch_r(GemvArgs &a, const Plan &p, hipStream_t st) {
-    switch (p.r) {
-        case 1: return dispatch_ch<M, 1>(a, p, st);
-        case 2: return dispatch_ch<M, 2>(a, p, st);
-    }
+    if (p.r == 2) return dispatch_ch<M, 2>(a, p, st);
+    if constexpr (M == 1) if (p.r == 1) return dispatch_ch<M, 1>(a, p, st);
     return fail(CMI_E_UNSUPPORTED, "cmi_gemv_w8a16: no kernel for %d rows per block", p.r);
 }
 
