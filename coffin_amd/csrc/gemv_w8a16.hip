@@ -90,18 +90,25 @@ __device__ __forceinline__ void widen4(uint32_t w, bf16x2_t &lo, bf16x2_t &hi) {
 
 // Wavefronts per workgroup (they share one LDS copy of the activations); wide
 // batches get smaller workgroups so that each wavefront may use more registers.
+// (For one row and K in several units, 9728 -> 2560, that means one team of 3 wavefronts that
+// stages the whole activation row for two weight rows; workgroups of 6, 9 and 12 wavefronts stage
+// less and measured 8.6, 9.3 and 9.7 us against 7.3.)
 constexpr int block_waves(int m) { return m >= 16 ? 16 : m >= 8 ? 8 : 4; }
 
 // Wavefronts per SIMD the register allocation must leave room for.
 constexpr int simd_waves(int m, int cht) { return m >= 8 || (m == 4 && cht == 1) ? 4 : 1; }
 
-// uint4 vectors of the LDS copy of the activations.  Up to 2 rows: [row][K] as in memory plus
-// one zeroed 32-byte slot.  From 4 rows: [segment][row of the M tile][half][lane], 2 KiB per
-// (segment, row) with the tail of the last segment and any dead segments zeroed, so a
-// wavefront's reads are contiguous across lanes, rows differ by a compile-time offset and
-// dead chunks read zeros without a select.
-__host__ __device__ constexpr int xlds_vectors(int mt, int rows, int K, int segs) {
-    return mt >= 4 ? segs * mt * 128 : rows * (K / 8) + 2;
+// uint4 vectors of the LDS copy of the activations.
+//   From 4 rows: [segment][row of the M tile][half][lane], 2 KiB per (segment, row), the tail of
+//     the last segment and any dead segments zeroed: reads are contiguous across lanes, rows
+//     differ by a compile-time offset and dead chunks read zeros without a select.
+//   Up to 2 rows, K one unit: [row][segment][lane][half], i.e. a row as it is in memory, padded
+//     with zeros to whole segments: again no select, a lane's address is its own offset plus
+//     constants.
+//   Up to 2 rows, several units: [row][K] unpadded plus one zeroed 32-byte slot that dead chunks
+//     are pointed at (padding whole dead segments would cost a workgroup per CU at K = 9728).
+__host__ __device__ constexpr int xlds_vectors(int mt, int rows, int K, int segs, bool one_unit) {
+    return mt >= 4 ? mt * segs * 128 : one_unit ? rows * segs * 128 : rows * (K / 8) + 2;
 }
 
 // Activation rows held in registers at a time; wider batches loop over tiles of this many
@@ -144,7 +151,7 @@ gemv_w8a16_kernel(const GemvArgs a) {
     int u = wave - team * a.uw;         // unit in hand; the team's wavefronts stride over units
     const int xvecs = a.K / 8;          // uint4 per activation row
     const int segs = a.units * a.unit;  // segments the unit loop walks (>= nseg)
-    float *unit_total = reinterpret_cast<float *>(smem + (XLDS ? xlds_vectors(M, a.M, a.K, segs) : 0)) +
+    float *unit_total = reinterpret_cast<float *>(smem + (XLDS ? xlds_vectors(M, a.M, a.K, segs, MODE == 0) : 0)) +
                         team * a.units * (R * M);
 
     const int8_t *wrow[R];  // uniform per wavefront
@@ -182,13 +189,17 @@ gemv_w8a16_kernel(const GemvArgs a) {
             for (int m = 0; m < MT; ++m) {
                 const int mrow = mh * MT + m < a.M ? mh * MT + m : a.M - 1;
                 if constexpr (XLDS) {
-                    // dead chunks read the zeroed slot behind the activations: a select
-                    // on the address, so the LDS reads stay unconditional
+                    // dead chunks read zeros: the LDS reads are unconditional
                     if constexpr (M >= 4) {
                         const int at = (seg * M + mh * MT + m) * 128 + lane + xoff;
                         s.x[m][j][0] = smem[at];
                         s.x[m][j][1] = smem[at + 64];
+                    } else if constexpr (MODE == 0) {
+                        const int at = (mrow * segs + seg) * 128 + 2 * lane;
+                        s.x[m][j][0] = smem[at];
+                        s.x[m][j][1] = smem[at + 1];
                     } else {
+                        // a select on the address, so the LDS reads stay unconditional
                         const int at = live ? mrow * xvecs + 2 * chunk : a.M * xvecs;
                         s.x[m][j][0] = smem[at];
                         s.x[m][j][1] = smem[at + 1];
@@ -278,7 +289,10 @@ gemv_w8a16_kernel(const GemvArgs a) {
                 const int seg = v >> 7, half = v & 1, c = (v & 127) >> 1;
                 if (mine) smem[(seg * M + row) * 128 + half * 64 + c] = xstage[j];
             } else {
-                if (mine) smem[idx] = xstage[j];  // little LDS traffic: plain order
+                // little LDS traffic: memory order; the second row starts at its padded offset
+                const int row = idx >= xvecs ? 1 : 0;
+                const int pad = MODE == 0 ? segs * 128 - xvecs : 0;
+                if (mine) smem[idx + row * pad] = xstage[j];
             }
         }
         if constexpr (M >= 4) {
@@ -294,6 +308,12 @@ gemv_w8a16_kernel(const GemvArgs a) {
             const int n_dead = (segs - a.nseg) * M * 128;
             for (int i = threadIdx.x; i < n_dead; i += blockDim.x)
                 smem[a.nseg * M * 128 + i] = make_uint4(0, 0, 0, 0);
+        } else if constexpr (MODE == 0) {
+            const int pad = segs * 128 - xvecs;  // zero vectors behind each row (< 128)
+            for (int i = threadIdx.x; i < a.M * pad; i += blockDim.x) {
+                const int row = i >= pad ? 1 : 0;
+                smem[row * segs * 128 + xvecs + i - row * pad] = make_uint4(0, 0, 0, 0);
+            }
         } else {
             if (threadIdx.x < 2) smem[xtotal + threadIdx.x] = make_uint4(0, 0, 0, 0);
         }
@@ -442,7 +462,7 @@ int launch(GemvArgs &a, hipStream_t st) {
     a.teams = block_waves(M) / a.uw;
     const dim3 grid((a.nblocks + a.teams - 1) / a.teams);
     const dim3 block(64 * a.uw * a.teams);
-    const size_t lds = (XLDS ? 16 * (size_t)xlds_vectors(M, a.M, a.K, a.units * a.unit) : 0) +
+    const size_t lds = (XLDS ? 16 * (size_t)xlds_vectors(M, a.M, a.K, a.units * a.unit, MODE == 0) : 0) +
                        (MODE == 0 ? 0 : sizeof(float) * a.teams * a.units * R * M);
     if constexpr (XLDS && xstage_short(M) < xstage_vectors(M)) {
         if ((size_t)a.M * (a.K / 8) <= (size_t)xstage_short(M) * block.x)
@@ -454,7 +474,7 @@ int launch(GemvArgs &a, hipStream_t st) {
 // Whether a workgroup of the M-tile's kernel can carry [rows, K] activations into LDS.
 bool x_fits_lds(int mt, int rows, int K, int units, int segs) {
     const size_t xbytes = (size_t)rows * K * 2;                              // carried by the threads
-    const size_t ldsbytes = 16 * (size_t)xlds_vectors(mt, rows, K, segs);   // held in LDS
+    const size_t ldsbytes = 16 * (size_t)xlds_vectors(mt, rows, K, segs, units == 1);   // held in LDS
     const int uw = units < 4 ? units : 4;
     const int bw = mt >= 16 ? block_waves(16) : mt >= 8 ? block_waves(8) : block_waves(1);
     const int xv = mt <= 1 ? xstage_vectors(1) : mt <= 2 ? xstage_vectors(2) : mt <= 4 ? xstage_vectors(4)
