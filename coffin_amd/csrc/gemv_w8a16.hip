@@ -93,7 +93,13 @@ __device__ __forceinline__ void widen4(uint32_t w, bf16x2_t &lo, bf16x2_t &hi) {
 // (For one row and K in several units, 9728 -> 2560, that means one team of 3 wavefronts that
 // stages the whole activation row for two weight rows; workgroups of 6, 9 and 12 wavefronts stage
 // less and measured 8.6, 9.3 and 9.7 us against 7.3.)
-constexpr int block_waves(int m) { return m >= 16 ? 16 : m >= 8 ? 8 : 4; }
+// Four rows and more with K in several units (a team is then 3 or 4 wavefronts that share two
+// weight rows): sixteen wavefronts, or every two weight rows would pay for staging the whole
+// activation block (9728 -> 2560 at 4 rows: 19 us with 4 wavefronts, 16 with 8, 9 with 16).
+constexpr int block_waves(int m, int mode = 0, bool multi_unit = false) {
+    return m >= 16 ? 16 : (m >= 4 && multi_unit) ? 16 : m >= 8 ? 8 : (m == 4 && mode == 2) ? 8 : 4;
+}
+constexpr int max_block_waves(int m, int mode) { return (m >= 4 && mode != 0) ? 16 : block_waves(m); }
 
 // Wavefronts per SIMD the register allocation must leave room for.
 constexpr int simd_waves(int m, int cht) { return m >= 8 || (m == 4 && cht == 1) ? 4 : 1; }
@@ -117,9 +123,10 @@ __host__ __device__ constexpr int xlds_vectors(int mt, int rows, int K, int segs
 constexpr int m_tile(int m) { return m < 4 ? m : 4; }
 
 // 16-byte vectors of activations each thread can carry from global memory to LDS, and the
-// short variant compiled for one or two rows of ordinary width (K up to 4096 at four wavefronts).
+// short variant that covers the decode shapes of up to four rows (e.g. K up to 4096 at four
+// wavefronts and one row).
 constexpr int xstage_vectors(int m) { return m <= 1 ? 8 : m <= 2 ? 16 : m <= 4 ? 20 : 8; }
-constexpr int xstage_short(int m) { return m <= 1 ? 2 : m <= 2 ? 4 : xstage_vectors(m); }
+constexpr int xstage_short(int m) { return m <= 1 ? 2 : m <= 2 ? 4 : m <= 4 ? 6 : xstage_vectors(m); }
 
 template <int M, int CHT>
 struct XStage {
@@ -138,7 +145,7 @@ struct WStage {
 //       reads them from global memory (only when they do not fit).
 // XV: 16-byte vectors of activations each thread carries from global memory to LDS.
 template <int M, int R, int CHT, int MODE, bool XLDS, int XV>
-__global__ void __launch_bounds__(64 * block_waves(M), simd_waves(M, CHT))
+__global__ void __launch_bounds__(64 * max_block_waves(M, MODE), simd_waves(M, CHT))
 gemv_w8a16_kernel(const GemvArgs a) {
     extern __shared__ uint4 smem[];  // staged activations (XLDS, see xlds_vectors), then unit totals
     const int lane = threadIdx.x & 63;
@@ -459,7 +466,7 @@ int launch(GemvArgs &a, hipStream_t st) {
     a.xvecs_rcp = (uint32_t)(((1ull << 32) + (a.K / 8) - 1) / (a.K / 8));
     a.uw = a.units < 4 ? a.units : 4;
     a.uw_rcp = (65536u + a.uw - 1) / a.uw;
-    a.teams = block_waves(M) / a.uw;
+    a.teams = block_waves(M, MODE, a.units > 1) / a.uw;
     const dim3 grid((a.nblocks + a.teams - 1) / a.teams);
     const dim3 block(64 * a.uw * a.teams);
     const size_t lds = (XLDS ? 16 * (size_t)xlds_vectors(M, a.M, a.K, a.units * a.unit, MODE == 0) : 0) +
@@ -472,11 +479,11 @@ int launch(GemvArgs &a, hipStream_t st) {
 }
 
 // Whether a workgroup of the M-tile's kernel can carry [rows, K] activations into LDS.
-bool x_fits_lds(int mt, int rows, int K, int units, int segs) {
+bool x_fits_lds(int mt, int rows, int K, int units, int segs, int mode) {
     const size_t xbytes = (size_t)rows * K * 2;                              // carried by the threads
     const size_t ldsbytes = 16 * (size_t)xlds_vectors(mt, rows, K, segs, units == 1);   // held in LDS
     const int uw = units < 4 ? units : 4;
-    const int bw = mt >= 16 ? block_waves(16) : mt >= 8 ? block_waves(8) : block_waves(1);
+    const int bw = block_waves(mt, mode, units > 1);
     const int xv = mt <= 1 ? xstage_vectors(1) : mt <= 2 ? xstage_vectors(2) : mt <= 4 ? xstage_vectors(4)
                                                                              : xstage_vectors(8);
     const size_t threads = 64 * (size_t)uw * (bw / uw);  // as launch() sizes the workgroup
@@ -485,7 +492,7 @@ bool x_fits_lds(int mt, int rows, int K, int units, int segs) {
 
 template <int M, int R, int CHT, int MODE>
 int dispatch_lds(GemvArgs &a, hipStream_t st) {
-    if (x_fits_lds(M, a.M, a.K, a.units, a.units * a.unit)) return launch<M, R, CHT, MODE, true>(a, st);
+    if (x_fits_lds(M, a.M, a.K, a.units, a.units * a.unit, MODE)) return launch<M, R, CHT, MODE, true>(a, st);
     return launch<M, R, CHT, MODE, false>(a, st);
 }
 
@@ -542,7 +549,7 @@ extern "C" int cmi_gemv_w8a16(const int8_t *wq, const float *ws, const void *x, 
                 MAX_UNITS * 4096);
     // Activations too large for LDS: narrower batches fit more often, and rows are
     // independent (same bits whatever the batch), so halve the batch instead.
-    if (M > 1 && !x_fits_lds(p.mt, M, K, a.units, a.units * a.unit)) {
+    if (M > 1 && !x_fits_lds(p.mt, M, K, a.units, a.units * a.unit, p.mode)) {
         const int half = p.mt / 2;
         const int rc = cmi_gemv_w8a16(wq, ws, x, y, half, N, K, stream);
         if (rc != CMI_OK) return rc;
