@@ -36,7 +36,7 @@ METRIC = "decode GEMV HBM GB/s (% of peak) + W8A8 prefill int8 TOPS, Qwen3.5-4B 
 
 #: gemv_w8a16_kernel, default workload (M=1): fetched + written bytes per launch, from the
 #: FETCH_SIZE and WRITE_SIZE runs summarised in profiles/gemv_w8a16_decode_model_M1.md
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28.39e6
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28.42e6
 
 
 def parse_args():
