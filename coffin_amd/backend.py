@@ -67,7 +67,7 @@ W8A8_VERIFY = os.environ.get("COFFIN_AMD_W8A8_VERIFY", "0").strip() == "1"
 #: weight-only arithmetic, last-place differences from fp32 summation order.
 #: ``COFFIN_AMD_BATCH_MFMA=1`` moves *every* int8 weight-only call -- ``linear`` included, one row
 #: included -- to the matrix-pipe GEMV: the contract holds again (one kernel family, a row's bits
-#: independent of its batch), static batches of 4-16 requests run 1.5-3.8 times faster, and
+#: independent of its batch), static batches of 4-16 requests run 1.05-2.8 times faster, and
 #: single-stream decode pays for it (7.9 us instead of 6.3 us for 2560 -> 9728).  A deployment choice.
 BATCH_MFMA = os.environ.get("COFFIN_AMD_BATCH_MFMA", "0").strip() == "1"
 #: Rows from which the matrix-pipe GEMV beats the dot-product one (measured on every layer shape).
@@ -80,6 +80,18 @@ W4_GEMM_MIN_ROWS = 17
 #: win (10.8 us against 12.7 us at 9728 -> 2560).
 W4_FUSED_MAX_ROWS = 1
 W4_FUSED_MAX_ROWS_LONG_K = 2
+
+
+def _w4_fused(rows: int, n: int, k: int) -> bool:
+    """Whether a W4A8 projection of ``rows`` rows takes the one-launch GEMV.
+
+    Rows longer than 4096 run on the matrix-pipe kernel, whose every 16-row workgroup then
+    quantises the whole activation row; with many workgroups that costs more than a quantiser
+    launch (5120 -> 9728: 16.3 us fused, 9.8 + 2.5 us as two launches; 9728 -> 5120 the other way).
+    """
+    if k > 4096 and n >= 8192:
+        return False
+    return rows <= (W4_FUSED_MAX_ROWS_LONG_K if k > 5120 else W4_FUSED_MAX_ROWS)
 
 def _vp(address: int) -> int:
     """Pointer argument: the entry points declare ``void *`` (``argtypes``), so a plain int passes."""
@@ -266,7 +278,7 @@ def _gemm_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> N
 def _rows_w4(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> None:
     n, k, gs = rec.n, rec.k, rec.gs
     lib = _native.load()
-    if rows <= (W4_FUSED_MAX_ROWS_LONG_K if k > 5120 else W4_FUSED_MAX_ROWS):
+    if _w4_fused(rows, n, k):
         # decode: one launch, activations quantised inside the GEMV (same bits)
         rc = lib.cmi_gemv_w4a8_bf16(rec.a, rec.b, act.data_ptr(), out.data_ptr(), 0, 0, 0,
                                     rows, n, k, gs, _stream())

@@ -344,9 +344,19 @@ extern "C" int cmi_gemv_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     CMI_REQUIRE(aligned(w4, 16) && aligned(xq, 16), CMI_E_ARG,
                 "cmi_gemv_w4a8: w4 and xq must be 16-byte aligned");
     if (gs == GS && N >= 1 && M >= 1) {
-        // 1..2 rows: dot-product kernel; 3..16: group sums on the matrix pipe (measured faster from 3 up)
-        const int rc = M <= 2 ? gemv_w4a8_decode(w4, ws, nullptr, xq, xs, y, group_acc, nullptr, nullptr, M, N, K, stream)
-                              : gemv_w4a8_rows16(w4, ws, xq, xs, nullptr, y, group_acc, nullptr, nullptr, M, N, K, stream);
+        // One row: the dot-product kernel while a wavefront can hold its whole rows (K <= 4096) or
+        // the grid is small enough that the wavefronts of a workgroup share rows; with longer rows
+        // it runs 10-20 KiB per wavefront at low occupancy (5120 -> 25600: 40 us against 20).
+        // Two rows: the same kernel only for whole rows of a large weight (2560 -> 151936: 34.5 us
+        // against 42); otherwise, and from three rows, group sums on the matrix pipe.
+        const bool shared_rows = (N + 15) / 16 < 256, whole_rows = K <= 4096;
+        int rc = CMI_E_UNSUPPORTED;
+        if ((M == 1 && (whole_rows || shared_rows)) || (M == 2 && whole_rows && N >= 12288))
+            rc = gemv_w4a8_decode(w4, ws, nullptr, xq, xs, y, group_acc, nullptr, nullptr, M, N, K, stream);
+        if (rc == CMI_E_UNSUPPORTED)
+            rc = gemv_w4a8_rows16(w4, ws, xq, xs, nullptr, y, group_acc, nullptr, nullptr, M, N, K, stream);
+        if (rc == CMI_E_UNSUPPORTED && M <= 2)
+            rc = gemv_w4a8_decode(w4, ws, nullptr, xq, xs, y, group_acc, nullptr, nullptr, M, N, K, stream);
         if (rc != CMI_E_UNSUPPORTED) return rc;
     }
     return run_gemv_w4a8("cmi_gemv_w4a8", w4, ws, xq, xs, nullptr, nullptr, nullptr, y, group_acc, M, N, K, gs,
@@ -366,10 +376,11 @@ extern "C" int cmi_gemv_w4a8_bf16(const uint8_t *w4, const float *ws, const void
     CMI_REQUIRE(gs == GS, CMI_E_UNSUPPORTED, "cmi_gemv_w4a8_bf16: group size %d, kernels are built for %d", gs, GS);
     CMI_REQUIRE(K % GS == 0, CMI_E_UNSUPPORTED, "cmi_gemv_w4a8_bf16: K=%d is not a multiple of %d", K, GS);
     // long rows: the matrix-pipe kernel with the quantiser folded in (the dot-product kernel shares
-    // such rows among wavefronts and its fp32 chain serialises: 10.5 us at 9728 -> 2560); else the
+    // such rows among wavefronts and its fp32 chain serialises: 10.5 us at 9728 -> 2560; or holds
+    // 10-20 KiB per wavefront: 5120 -> 25600 42 us against 26); else the
     // decode kernel (whole rows requested up front) where it applies, else the general one
     int rc = CMI_E_UNSUPPORTED;
-    if (K > 5120)
+    if (K > 4096)
         rc = gemv_w4a8_rows16(w4, ws, nullptr, nullptr, x, y, group_acc, xq_out, xs_out, M, N, K, stream);
     if (rc != CMI_E_UNSUPPORTED) return rc;
     rc = gemv_w4a8_decode(w4, ws, x, nullptr, nullptr, y, group_acc, xq_out, xs_out, M, N, K, stream);

@@ -183,6 +183,21 @@ def test_w4_entries_match_the_oracle_bit_for_bit(orc, rows):
     assert _rel(y.reshape(ref.shape), ref) < 5e-2
 
 
+@pytest.mark.parametrize("n,k", [(8192, 5120), (1024, 5120), (512, 9728)])
+def test_w4_long_rows_take_the_same_bits_on_every_route(orc, n, k):
+    # rows beyond 4096 leave the dot-product kernel: matrix-pipe GEMV, one launch or two
+    # (quantiser + GEMV) depending on the number of workgroups; the bits are the oracle's either way
+    g = synth.generator()
+    w = _w4(n, k, g)
+    for rows in (1, 2, 3):
+        x = synth.activations(rows, k, g).to(G.DEV)
+        xq, xs = orc.quant_act_i8(G.bits(x))
+        _, y_ref = orc.linear_w4a8(xq, xs, w.packed.cpu().numpy(), w.scale.cpu().numpy(), k, 128)
+        for fn in (backend.linear_m, backend.linear_m_verify):
+            assert (G.bits(fn(w, x)) == y_ref).all(), (fn.__name__, rows)
+        assert (G.bits(backend.linear(w, x[0])) == y_ref[0]).all()
+
+
 def test_tied_embedding_on_the_gpu(orc):
     """Row gather on the device gives the oracle's dequantised rows; the projection is the
     native GEMV on the same weight (ops/embed.py:64-104)."""

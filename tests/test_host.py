@@ -171,6 +171,14 @@ def test_gemv_regimes_follow_row_count():
         ("linear_m", (8, 4)), ("linear_prefill", (9, 4))]
 
 
+def test_w4_one_launch_rule():
+    from coffin_amd import backend
+    assert backend._w4_fused(1, 9728, 2560) and not backend._w4_fused(2, 9728, 2560)
+    assert backend._w4_fused(2, 2560, 9728) and not backend._w4_fused(3, 2560, 9728)
+    # long rows and many workgroups: the quantiser gets a launch of its own
+    assert not backend._w4_fused(1, 25600, 5120) and backend._w4_fused(1, 5120, 25600)
+
+
 def test_gemv_group_fuses_and_splits():
     g = synth.generator()
     qa, qb = synth.int8_weight(6, 32, g), synth.int8_weight(10, 32, g)
