@@ -89,7 +89,7 @@ def _w4_fused(rows: int, n: int, k: int) -> bool:
     quantises the whole activation row; with many workgroups that costs more than a quantiser
     launch (5120 -> 9728: 16.3 us fused, 9.8 + 2.5 us as two launches; 9728 -> 5120 the other way).
     """
-    if k > 4096 and n >= 8192:
+    if (k > 4096 and n >= 8192) or k > 10240:  # (beyond 10240 only the two-launch route has a fast kernel)
         return False
     return rows <= (W4_FUSED_MAX_ROWS_LONG_K if k > 5120 else W4_FUSED_MAX_ROWS)
 

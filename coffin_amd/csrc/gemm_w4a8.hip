@@ -308,11 +308,13 @@ extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     // matrix-pipe GEMV reads the weight once per 16 rows at memory speed; same integer sums, same
     // fp32 chain, same bits.  Cost model fitted to measurements on the layer shapes (us).
     const char *force = getenv("CMI_GEMM_TILE");
-    if (M <= 256 && K <= 10240 && !(force && force[0])) {
+    if (M <= 256 && !(force && force[0])) {
         const double steps = K / 128.0;
         const double tiles = (double)a_ceil(M, BM) * a_ceil(N, BN);
         const double t_tiled = 3.0 + steps * 1.17 * ceil(tiles / 512.0);
-        const double t_rows16 = a_ceil(M, 16) * (3.6 + (double)N * K / 2 / 4.2e6 + steps * 0.025);
+        // (rows beyond 10240 run the GEMV in passes: about half the speed)
+        const double t_rows16 = K <= 10240 ? a_ceil(M, 16) * (3.6 + (double)N * K / 2 / 4.2e6 + steps * 0.025)
+                                           : a_ceil(M, 16) * (3.6 + (double)N * K / 2 / 2.1e6);
         if (t_rows16 < t_tiled) {
             const int G = K / BK;
             for (int lo = 0; lo < M; lo += 16) {

@@ -1,5 +1,6 @@
-// W4A8 GEMV for 3..16 activation rows (speculative verify, small batches), from
-// already quantised activations, K <= 10240.
+// W4A8 GEMV for up to 16 activation rows (speculative verify, small batches, long rows), from
+// already quantised activations (K <= 10240 in one pass, longer rows in passes) or, up to 4
+// rows and K <= 10240, from bf16 activations.
 //
 //   sum_g   = sum_{k in group g} xq[m,k] * (code(n,k) - 8)     int32, exact
 //   total   = fma((float)sum_g, ws[n,g], total)                 g = 0,1,.. from 0.f
@@ -289,6 +290,161 @@ int launch(const Args &a, hipStream_t st) {
     return a.group_acc ? launch_one<NLP, WAVES, true, false>(a, st) : launch_one<NLP, WAVES, false, false>(a, st);
 }
 
+
+// Rows longer than MAX_K: the same work in passes of 80 groups (10240 k), the fp32 chain carried
+// from pass to pass in the register of its thread.  The next pass's bytes are requested as soon
+// as this pass's MFMAs have consumed their registers, so memory keeps working while the chain of
+// this pass runs.  Quantised activations only (a caller with bf16 rows quantises first).
+constexpr int LONG_NLP = 3, LONG_WAVES = 8, LONG_GP = 2 * LONG_NLP * LONG_WAVES;  // groups per pass
+constexpr int LONG_THREADS = LONG_WAVES * 64;
+constexpr int LONG_WSN = (ROWS * LONG_GP + LONG_THREADS - 1) / LONG_THREADS;
+
+template <bool DUMP>
+__global__ void __launch_bounds__(LONG_THREADS)
+gemv_w4a8_rows16_long_kernel(const Args a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    int32_t *sums = reinterpret_cast<int32_t *>(lds);                 // [LONG_GP][64 lanes][4]
+    float *ws_lds = reinterpret_cast<float *>(lds + LONG_GP * 1024);  // [16][LONG_GP]
+    uint8_t *patches = lds + LONG_GP * 1024 + ROWS * LONG_GP * 4;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kq = lane >> 4;
+    const int n0 = blockIdx.x * ROWS;
+    const int lines = (a.G + 1) / 2;
+    const int passes = (a.G + LONG_GP - 1) / LONG_GP;
+    const int nrows = min(ROWS, a.N - n0);
+    uint8_t *patch = patches + wave * PATCH_BYTES;
+
+    v4i32 xa[LONG_NLP][2][2], w[LONG_NLP][2];
+    float wsreg[LONG_WSN];
+    // requests of one pass: activations first, then the scales, then every weight byte
+    auto request = [&](int pass) {
+        const int line0 = pass * (LONG_NLP * LONG_WAVES) + wave;
+#pragma unroll
+        for (int i = 0; i < LONG_NLP; ++i) {
+            const int line = line0 + i * LONG_WAVES;
+            if (line >= lines) break;  // uniform per wavefront
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int g = min(2 * line + h, a.G - 1);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    xa[i][h][j] =
+                        *reinterpret_cast<const v4i32 *>(a.xq + tile_src(lane, j, 0, a.M - 1, a.K, g * GS));
+            }
+        }
+        const int gp = min(LONG_GP, a.G - pass * LONG_GP);  // groups of this pass
+#pragma unroll
+        for (int i = 0; i < LONG_WSN; ++i) {
+            const int idx = threadIdx.x + i * LONG_THREADS;
+            const int row = idx / LONG_GP, col = idx - row * LONG_GP;
+            wsreg[i] = (row < nrows && col < gp) ? a.ws[(size_t)(n0 + row) * a.G + pass * LONG_GP + col] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < LONG_NLP; ++i) {
+            const int line = line0 + i * LONG_WAVES;
+            if (line >= lines) break;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                w[i][j] = __builtin_nontemporal_load(reinterpret_cast<const v4i32 *>(
+                    a.w4 + tile_src<true>(lane, j, n0, a.N - 1, a.K / 2, line * 128)));
+        }
+    };
+    request(0);
+
+    const int p = threadIdx.x, l = (p >> 2) & 63, v = p & 3;
+    const int nn = l & 15, m = 4 * (l >> 4) + v, n = n0 + nn;
+    const bool chain = p < 256 && n < a.N && m < a.M;
+    float total = 0.f;
+    const v4i32 minus8 = {(int)0xF8F8F8F8u, (int)0xF8F8F8F8u, (int)0xF8F8F8F8u, (int)0xF8F8F8F8u};
+#pragma unroll 1
+    for (int pass = 0; pass < passes; ++pass) {
+        const int line0 = pass * (LONG_NLP * LONG_WAVES) + wave;
+        // scales of this pass (the previous pass's chain is behind the barrier that ended it)
+#pragma unroll
+        for (int i = 0; i < LONG_WSN; ++i) {
+            const int idx = threadIdx.x + i * LONG_THREADS;
+            if (idx < ROWS * LONG_GP) ws_lds[idx] = wsreg[i];
+        }
+        // activations into the MFMA arrangement: row lane%16, bytes 32*kq .. +31 of each group
+#pragma unroll
+        for (int i = 0; i < LONG_NLP; ++i) {
+            if (line0 + i * LONG_WAVES >= lines) break;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                tile_park(patch, lane, xa[i][h][0], xa[i][h][1]);
+                xa[i][h][0] = tile_take(patch, lane, 2 * kq);
+                xa[i][h][1] = tile_take(patch, lane, 2 * kq + 1);
+            }
+        }
+        // integer group sums: lane holds (n = lane%16, m = 4*kq + v), v = 0..3
+#pragma unroll
+        for (int i = 0; i < LONG_NLP; ++i) {
+            const int line = line0 + i * LONG_WAVES;
+            if (line >= lines) break;
+            tile_park(patch, lane, w[i][0], w[i][1]);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int g = 2 * line + h;
+                if (g >= a.G) break;  // uniform per wavefront
+                const u32x4 ww = __builtin_bit_cast(u32x4, tile_take(patch, lane, 4 * h + kq));
+                const v4i32 x0 = {xa[i][h][0].x, xa[i][h][0].z, xa[i][h][1].x, xa[i][h][1].z};
+                const v4i32 x1 = {xa[i][h][0].y, xa[i][h][0].w, xa[i][h][1].y, xa[i][h][1].w};
+                const u32x4 lo = ww & 0x0F0F0F0Fu, hi = (ww >> 4) & 0x0F0F0F0Fu;
+                v4i32 acc = {0, 0, 0, 0};
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x0, minus8, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x1, minus8, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x0, __builtin_bit_cast(v4i32, lo), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x1, __builtin_bit_cast(v4i32, hi), acc, 0, 0, 0);
+                reinterpret_cast<v4i32 *>(sums)[(g - pass * LONG_GP) * 64 + lane] = acc;
+            }
+        }
+        if (pass + 1 < passes) request(pass + 1);
+        __syncthreads();
+        // fp32 chain over this pass's groups, one thread per (n, m)
+        if (chain) {
+            const int gp = min(LONG_GP, a.G - pass * LONG_GP);
+            const int32_t *sp = sums + p;
+            const float *wsn = ws_lds + nn * LONG_GP;
+            int g = 0;
+            for (; g + 4 <= gp; g += 4) {
+                int sv[4];
+                float wv[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    sv[i] = sp[(g + i) * 256];
+                    wv[i] = wsn[g + i];
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if constexpr (DUMP) a.group_acc[((size_t)m * a.G + pass * LONG_GP + g + i) * a.N + n] = sv[i];
+                    total = fmaf((float)sv[i], wv[i], total);
+                }
+            }
+            for (; g < gp; ++g) {
+                const int sg = sp[g * 256];
+                if constexpr (DUMP) a.group_acc[((size_t)m * a.G + pass * LONG_GP + g) * a.N + n] = sg;
+                total = fmaf((float)sg, wsn[g], total);
+            }
+        }
+        __syncthreads();  // sums and scales are overwritten by the next pass
+    }
+    if (chain) a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * a.xs[m]);
+}
+
+template <bool DUMP>
+int launch_long(const Args &a, hipStream_t st) {
+    constexpr int LDS_BYTES = LONG_GP * 1024 + ROWS * LONG_GP * 4 + LONG_WAVES * PATCH_BYTES;
+    static std::atomic<uint64_t> devices{0};
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w4a8_rows16_long_kernel<DUMP>), LDS_BYTES,
+                                   devices, "cmi_gemv_w4a8"))
+        return rc;
+    const dim3 grid((a.N + ROWS - 1) / ROWS);
+    gemv_w4a8_rows16_long_kernel<DUMP><<<grid, dim3(LONG_THREADS), LDS_BYTES, st>>>(a);
+    return check_launch("cmi_gemv_w4a8");
+}
+
 }  // namespace
 
 namespace cmi {
@@ -300,8 +456,8 @@ namespace cmi {
 int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs, const void *x,
                      void *y, int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
                      void *stream) {
-    if (M < 1 || M > (x ? FUSED_ROWS : ROWS) || K < GS || K > MAX_K || K % GS != 0 || N < 1)
-        return CMI_E_UNSUPPORTED;
+    if (M < 1 || M > (x ? FUSED_ROWS : ROWS) || K < GS || K % GS != 0 || N < 1) return CMI_E_UNSUPPORTED;
+    if (K > MAX_K && (x || (size_t)K * M > ((size_t)1 << 31))) return CMI_E_UNSUPPORTED;
     Args a;
     a.w4 = w4;
     a.ws = ws;
@@ -317,6 +473,7 @@ int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const
     a.K = K;
     a.G = K / GS;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (K > MAX_K) return group_acc ? launch_long<true>(a, st) : launch_long<false>(a, st);
     const int lines = (a.G + 1) / 2;
     // Eight wavefronts per workgroup beyond 20 lines, and up to ~640 workgroups (2.5 per compute
     // unit) where a wavefront's chain of dependent steps is what is left to shorten (0.6-0.9 us

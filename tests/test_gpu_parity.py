@@ -345,7 +345,9 @@ def _w4_case(orc, m, n, k, g):
                                    # 3..16 rows: every lines-per-wavefront variant, ragged N, odd group counts
                                    (5, 9728, 2560), (16, 9728, 2560), (7, 37, 128), (9, 100, 384),
                                    (16, 530, 1152), (12, 2560, 4096), (6, 300, 5120), (16, 256, 6656),
-                                   (13, 200, 8192), (16, 333, 10240), (5, 64, 10368), (16, 64, 12288)])
+                                   (13, 200, 8192), (16, 333, 10240), (5, 64, 10368), (16, 64, 12288),
+                                   # rows beyond 10240: passes of 80 groups, the chain carried across them
+                                   (16, 100, 20480), (2, 33, 25728), (16, 1024, 25600)])
 def test_gemv_w4a8_bit_exact(orc, m, n, k):
     w4, ws, xq, xs, gacc_ref, y_ref = _w4_case(orc, m, n, k, seeded())
     gacc, y = G.w4a8(w4, ws, xq, xs, k, gemm=False)

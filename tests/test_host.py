@@ -176,7 +176,8 @@ def test_w4_one_launch_rule():
     assert backend._w4_fused(1, 9728, 2560) and not backend._w4_fused(2, 9728, 2560)
     assert backend._w4_fused(2, 2560, 9728) and not backend._w4_fused(3, 2560, 9728)
     # long rows and many workgroups: the quantiser gets a launch of its own
-    assert not backend._w4_fused(1, 25600, 5120) and backend._w4_fused(1, 5120, 25600)
+    assert not backend._w4_fused(1, 25600, 5120) and not backend._w4_fused(1, 5120, 25600)
+    assert backend._w4_fused(1, 5120, 9728)
 
 
 def test_gemv_group_fuses_and_splits():
