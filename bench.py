@@ -386,6 +386,38 @@ def main() -> int:
         extra["w4a8_prefill_gemm_M1024_N25600_K5120"] = {
             "us": round(t * 1e6, 2), "tops": round(tops, 1), "frac_of_int8_peak": round(tops / INT8_PEAK_TOPS, 4)}
 
+        # W4A8 larger dense shape, both directions, M = 1 / 64 / 1024 (quantiser + GEMV or GEMM, as
+        # the adapter issues them); a few distinct weights per shape so that no call finds its
+        # weight in a cache
+        sweep = {}
+        for n_, k_ in ((25600, 5120), (5120, 25600)):
+            ws_ = []
+            for _ in range(4):
+                w = synth.int4_weight(n_, k_, gen)
+                d4 = torch.empty((n_, k_ // 2), dtype=torch.uint8, device=dev)
+                ds = torch.empty((n_, k_ // 128), dtype=torch.float32, device=dev)
+                lib.cmi_w4_repack(ptr(w.packed), ptr(w.scale), ptr(d4), ptr(ds), n_, k_, 128, cur_stream())
+                ws_.append((d4, ds))
+            torch.cuda.synchronize()
+            for m in (1, 64, 1024):
+                x = synth.activations(m, k_, gen)
+                xq = torch.empty((m, k_), dtype=torch.int8, device=dev)
+                xs = torch.empty(m, dtype=torch.float32, device=dev)
+                y = torch.empty((m, n_), dtype=torch.bfloat16, device=dev)
+                fn = lib.cmi_gemv_w4a8 if m <= 16 else lib.cmi_gemm_w4a8
+                def both(m=m, x=x, xq=xq, xs=xs, y=y, ws_=ws_, n_=n_, k_=k_, fn=fn):
+                    st = cur_stream()
+                    for d4, ds in ws_:
+                        lib.cmi_quant_act_i8(ptr(x), ptr(xq), ptr(xs), m, k_, st)
+                        fn(ptr(d4), ptr(ds), ptr(xq), ptr(xs), ptr(y), vp(0), m, n_, k_, 128, st)
+                t = timed(both, 5) / len(ws_)
+                sweep[f"{k_}->{n_}_M{m}"] = {
+                    "us": round(t * 1e6, 2), "GBps": round(synth.w4_gemv_bytes(m, n_, k_) / t / 1e9, 1),
+                    "tops": round(synth.gemm_ops(m, n_, k_) / t / 1e12, 1)}
+            del ws_
+        extra["w4a8_large_shape_quant_plus_linear"] = sweep
+        torch.cuda.empty_cache()
+
         # quantiser alone at prefill size
         m, k_ = 8192, 2560
         x = synth.activations(m, k_, gen)
