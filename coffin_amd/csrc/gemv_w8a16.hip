@@ -446,6 +446,10 @@ Plan make_plan(int M, int N, int K) {
     // when a wavefront's last bytes arrive (4096 -> 2560: 4.4 -> 4.1 us); from ~20 MB on the
     // launch is throughput-bound and the shared fragments win.
     p.r = (M == 1 && p.mode == 0 && (size_t)N * K <= ((size_t)20 << 20)) ? 1 : 2;
+    // Eight rows against a very tall weight (lm_head): four weight rows per wavefront halve the LDS
+    // reads of the activation fragments (154 -> 133 us at 2560 -> 151936); on the layer shapes, and
+    // at 16 rows (registers), two rows stay faster.
+    if (p.mt == 8 && N >= 65536) p.r = 4;
     return p;
 }
 
@@ -519,6 +523,7 @@ template <int M>
 int dispatch_r(GemvArgs &a, const Plan &p, hipStream_t st) {
     if (p.r == 2) return dispatch_ch<M, 2>(a, p, st);
     if constexpr (M == 1) if (p.r == 1) return dispatch_ch<M, 1>(a, p, st);
+    if constexpr (M == 8) if (p.r == 4) return dispatch_ch<M, 4>(a, p, st);
     return fail(CMI_E_UNSUPPORTED, "cmi_gemv_w8a16: no kernel for %d rows per block", p.r);
 }
 
