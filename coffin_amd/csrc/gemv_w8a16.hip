@@ -491,7 +491,10 @@ bool x_fits_lds(int mt, int rows, int K, int units, int segs, int mode) {
     const int xv = mt <= 1 ? xstage_vectors(1) : mt <= 2 ? xstage_vectors(2) : mt <= 4 ? xstage_vectors(4)
                                                                              : xstage_vectors(8);
     const size_t threads = 64 * (size_t)uw * (bw / uw);  // as launch() sizes the workgroup
-    return ldsbytes <= XLDS_MAX_BYTES && xbytes <= 16 * (size_t)xv * threads;
+    // the unit totals share the allocation: one float per (team, unit, weight row, activation row),
+    // at most four weight rows per wavefront
+    const size_t totals = units > 1 ? sizeof(float) * (bw / uw) * units * 4 * mt : 0;
+    return ldsbytes + totals <= XLDS_MAX_BYTES && xbytes <= 16 * (size_t)xv * threads;
 }
 
 template <int M, int R, int CHT, int MODE>

@@ -116,7 +116,9 @@ def _assert_weight_only_tolerance(orc, wq, ws, x, y):
                                    (5, 333, 2560), (11, 77, 1040), (1, 640, 25600), (8, 512, 5120),
                                    (16, 300, 7168), (4, 96, 9728), (12, 640, 3088), (16, 9728, 2560),
                                    (7, 37, 128), (9, 100, 384), (16, 64, 10368), (6, 530, 1152),
-                                   (16, 200, 12800), (5, 2560, 9728)])
+                                   (16, 200, 12800), (5, 2560, 9728),
+                                   # the activations just fit LDS / do not (batch split), many K units
+                                   (4, 200, 16384), (16, 100, 16384), (2, 64, 65536), (8, 48, 32768)])
 def test_gemv_w8a16_within_tolerance(orc, m, n, k):
     wq, ws, x, y = _w8a16_case(orc, m, n, k, seeded())
     _assert_weight_only_tolerance(orc, wq, ws, x, y)
@@ -142,7 +144,7 @@ def test_gemv_w8a16_golden(golden):
 
 
 @pytest.mark.parametrize("n,k", [(4096, 2560), (2560, 9728), (1000, 4112), (512, 5120), (300, 7168),
-                                 (777, 10368), (64, 128)])
+                                 (777, 10368), (64, 128), (100, 16384), (70000, 2560)])
 def test_gemv_w8a16_batched_row_equals_single_row(n, k):
     """The contract of static-batch decode (models/qwen35/batch.py:19-22): row r of a batched
     call carries the bits of the single-row call on x[r], whatever the batch."""
