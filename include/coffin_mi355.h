@@ -106,7 +106,8 @@ int cmi_gemv_w4a8_bf16(const uint8_t *w4, const float *ws, const void *x, void *
 
 /* W8A8 GEMM with fused epilogue:
  *   acc[m,n] = sum_k xq[m,k]*wq[n,k]  (int32) ; y[m,n] = bf16((float)acc*xs[m]*ws[n])
- * xq int8 [M,K], wq int8 [N,K], y bf16 with row stride ldy >= N.  K % 64 == 0.
+ * xq int8 [M,K], wq int8 [N,K], y bf16 with row stride ldy >= N.  K % 16 == 0
+ * (K % 128 == 0 for the pipelined kernels; other K take a generic one).
  * acc_out (nullable) receives the int32 accumulators as [M,N].
  * Up to 16 rows (K % 128 == 0, K <= 10240) the weight is read once, GEMV style:
  * the place of w8a8_dp4a_nk on the verify path (backends/corex/__init__.py:450-494).
