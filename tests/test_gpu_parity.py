@@ -134,6 +134,19 @@ def test_gemv_w8a16_mfma_within_tolerance(orc, m, n, k):
     _assert_weight_only_tolerance(orc, wq, ws, x, y)
 
 
+@pytest.mark.parametrize("n,k", [(9728, 2560), (300, 5120), (70, 1024), (33000, 2560), (2560, 4096)])
+def test_gemv_w8a16_mfma_wide_batches_carry_the_16_row_bits(n, k):
+    """17..64 rows in one launch (K <= 5120): every row has the bits of a 16-row call."""
+    g = seeded()
+    q = synth.int8_weight(n, k, g)
+    wq, ws = q.wq.to(G.DEV), q.scale.to(G.DEV)
+    x = synth.activations(64, k, g).to(G.DEV)
+    ref = torch.cat([G.gemv_w8a16(wq, ws, x[lo:lo + 16].contiguous(), mfma=True) for lo in range(0, 64, 16)])
+    for m in (17, 31, 32, 49, 64):
+        y = G.gemv_w8a16(wq, ws, x[:m].contiguous(), mfma=True)
+        assert (y.view(torch.int16) == ref[:m].view(torch.int16)).all(), m
+
+
 def test_gemv_w8a16_golden(golden):
     g = golden("linear_w8a16")
     y = G.gemv_w8a16(G.dev(g["wq"]), G.dev(g["scale"]), G.bf16_dev(g["x_bits"]))
