@@ -730,16 +730,18 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
         if (rc != CMI_E_UNSUPPORTED) return rc;
     }
     if (M > 16 && M <= 256 && K % 128 == 0 && K <= 10240 && !(force && force[0])) {
-        // Few rows: the tile pipeline is latency-bound (K/128 dependent steps of ~0.5 us with three
-        // LDS stages, ~0.9 us with two, whatever M is), the read-once kernel runs at memory speed per
-        // 16 rows; same bits.  Cost model fitted to measurements on the layer shapes (us).
-        const double steps = K / 128.0;
+        // Few rows: the tile pipeline is latency-bound (K/128 dependent steps of 0.45-1.4 us, growing
+        // with the number of tiles that share the chip, whatever M is); the read-once kernel asks
+        // for the weight once per 128 rows and pays per 16-row chunk only the chunk's trip through
+        // the matrix pipe; same bits.  Cost models fitted to measurements on the layer shapes with
+        // cold weights (us).
+        const double steps = K / 128.0, wbytes = (double)N * K;
         const double tiles = (double)((M + 127) / 128) * ((N + 127) / 128);
-        const double t_tiled = 2.5 + steps * (tiles <= 256 ? 0.5 : 0.9 * ceil(tiles / 512.0));
-        const double t_rows16 = ((M + 15) / 16) * (3.2 + (double)N * K / 6.0e6);
-        if (t_rows16 < t_tiled) {
-            for (int lo = 0; lo < M; lo += 16) {
-                const int m = M - lo < 16 ? M - lo : 16;
+        const double t_tiled = 2.5 + steps * (tiles <= 512 ? 0.42 + 0.0033 * tiles : 2.1 * ceil(tiles / 512.0));
+        const double t_rows = ((M + 127) / 128) * (3.2 + wbytes / 6.0e6) + ((M + 15) / 16) * (0.5 + wbytes / 2.0e7);
+        if (t_rows < t_tiled) {
+            for (int lo = 0; lo < M; lo += 128) {
+                const int m = M - lo < 128 ? M - lo : 128;
                 const int rc = gemm_w8a8_rows16(xq + (size_t)lo * K, wq, xs + lo, ws,
                                                 static_cast<uint16_t *>(y) + (size_t)lo * ldy,
                                                 acc_out ? acc_out + (size_t)lo * N : nullptr, m, N, K, ldy, stream);

@@ -1,4 +1,4 @@
-// W8A8 projection for 1..16 activation rows (speculative verify): the weight is
+// W8A8 projection for 1..16 (and, weight kept in registers, up to 128) activation rows: the weight is
 // read once, straight into registers, and the kernel is HBM-bound like a GEMV.
 //
 //   acc[m,n] = sum_k xq[m,k] * wq[n,k]                  int32, exact
@@ -108,6 +108,90 @@ int launch(const Args &a, hipStream_t st) {
     return check_launch("cmi_gemm_w8a8");
 }
 
+
+// 17..128 activation rows: the workgroup's 16 weight rows are asked for once and stay in
+// registers in the MFMA arrangement; the activation rows go through in chunks of 16.  Integer
+// sums are exact in any order, so the wavefronts add their partial tiles into one LDS tile per
+// chunk with ds_add and the bits are those of the 16-row kernel by construction.
+constexpr int MAX_CHUNKS = 8;
+
+template <int NLP, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
+gemm_w8a8_rows128_kernel(const Args a) {
+    __shared__ __align__(16) int32_t sums[MAX_CHUNKS][64][4];
+    __shared__ __align__(16) uint8_t patches[WAVES][PATCH_BYTES];
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kq = lane >> 4;
+    const int n0 = blockIdx.x * ROWS;
+    const int lines = a.K / LINE;
+    const int chunks = (a.M + ROWS - 1) / ROWS;
+    uint8_t *patch = patches[wave];
+    auto line_of = [&](int i) { return min(wave + i * WAVES, lines - 1); };  // surplus slots repeat the last line
+
+    v4i32 xr[NLP][2], wr[NLP][2];
+    auto request_x = [&](int c, int i) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)  // rows past M repeat the last one; their sums are dropped
+            xr[i][h] = *reinterpret_cast<const v4i32 *>(
+                a.xq + tile_src(lane, h, c * ROWS, a.M - 1, a.K, line_of(i) * LINE));
+    };
+#pragma unroll
+    for (int i = 0; i < NLP; ++i) request_x(0, i);
+#pragma unroll
+    for (int i = 0; i < NLP; ++i)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            wr[i][h] = __builtin_nontemporal_load(
+                reinterpret_cast<const v4i32 *>(a.wq + tile_src(lane, h, n0, a.N - 1, a.K, line_of(i) * LINE)));
+    for (int o = threadIdx.x; o < chunks * 256; o += WAVES * 64) (&sums[0][0][0])[o] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NLP; ++i) {
+        tile_park(patch, lane, wr[i][0], wr[i][1]);
+        wr[i][0] = tile_take(patch, lane, kq);
+        wr[i][1] = tile_take(patch, lane, 4 + kq);
+    }
+#pragma unroll 1
+    for (int c = 0; c < chunks; ++c) {
+        v4i32 acc = {0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < NLP; ++i) {
+            tile_park(patch, lane, xr[i][0], xr[i][1]);
+            const v4i32 x0 = tile_take(patch, lane, kq), x1 = tile_take(patch, lane, 4 + kq);
+            if (wave + i * WAVES < lines) {  // uniform per wavefront
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x0, wr[i][0], acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x1, wr[i][1], acc, 0, 0, 0);
+            }
+            if (c + 1 < chunks) request_x(c + 1, i);
+        }
+        int32_t *dst = &sums[c][lane][0];
+        atomicAdd(dst + 0, acc.x);
+        atomicAdd(dst + 1, acc.y);
+        atomicAdd(dst + 2, acc.z);
+        atomicAdd(dst + 3, acc.w);
+    }
+    __syncthreads();
+
+    for (int o = threadIdx.x; o < chunks * 256; o += WAVES * 64) {
+        const int c = o >> 8, l = (o >> 2) & 63, v = o & 3;
+        const int n = n0 + (l & 15), m = c * ROWS + 4 * (l >> 4) + v;
+        if (n < a.N && m < a.M) {
+            const int sm = sums[c][l][v];
+            if (a.acc_out) a.acc_out[(size_t)m * a.N + n] = sm;
+            a.y[(size_t)m * a.ldy + n] = (uint16_t)f32_to_bf16_bits(((float)sm * a.xs[m]) * a.ws[n]);
+        }
+    }
+}
+
+template <int NLP, int WAVES>
+int launch128(const Args &a, hipStream_t st) {
+    const dim3 grid((a.N + ROWS - 1) / ROWS);
+    gemm_w8a8_rows128_kernel<NLP, WAVES><<<grid, dim3(WAVES * 64), 0, st>>>(a);
+    return check_launch("cmi_gemm_w8a8");
+}
+
 }  // namespace
 
 namespace cmi {
@@ -116,7 +200,8 @@ namespace cmi {
 // outside this kernel's range (the caller then uses a tiled kernel).
 int gemm_w8a8_rows16(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws, void *y,
                      int32_t *acc_out, int M, int N, int K, int ldy, void *stream) {
-    if (M < 1 || M > ROWS || N < 1 || K < LINE || K % LINE != 0 || K > 80 * LINE) return CMI_E_UNSUPPORTED;
+    if (M < 1 || M > MAX_CHUNKS * ROWS || N < 1 || K < LINE || K % LINE != 0 || K > 80 * LINE)
+        return CMI_E_UNSUPPORTED;
     if (!aligned(xq, 16) || !aligned(wq, 16)) return CMI_E_UNSUPPORTED;
     Args a;
     a.xq = xq;
@@ -134,6 +219,13 @@ int gemm_w8a8_rows16(const int8_t *xq, const int8_t *wq, const float *xs, const 
     // eight wavefronts (shorter chains of dependent steps) measured 0.3-0.7 us faster up to
     // N = 19456; no difference at N = 151936
     const bool eight = (N + ROWS - 1) / ROWS <= 2048;
+    if (M > ROWS) {
+        if (lines <= 8) return launch128<2, 4>(a, st);
+        if (lines <= 24 && eight) return launch128<3, 8>(a, st);
+        if (lines <= 20) return launch128<5, 4>(a, st);
+        if (lines <= 40) return launch128<5, 8>(a, st);
+        return launch128<10, 8>(a, st);
+    }
     if (lines <= 8) return launch<2, 4>(a, st);
     if (lines <= 24 && eight) return launch<3, 8>(a, st);
     if (lines <= 20) return launch<5, 4>(a, st);

@@ -111,7 +111,8 @@ int cmi_gemv_w4a8_bf16(const uint8_t *w4, const float *ws, const void *x, void *
  * xq int8 [M,K], wq int8 [N,K], y bf16 with row stride ldy >= N.  K % 16 == 0
  * (K % 128 == 0 for the pipelined kernels; other K take a generic one).
  * acc_out (nullable) receives the int32 accumulators as [M,N].
- * Up to 16 rows (K % 128 == 0, K <= 10240) the weight is read once, GEMV style:
+ * Up to 16 rows (K % 128 == 0, K <= 10240) the weight is read once, GEMV style
+ * (and once per 128 rows for batches up to 256 rows where that is cheaper than the tile pipeline):
  * the place of w8a8_dp4a_nk on the verify path (backends/corex/__init__.py:450-494).
  * Replaces w8a8_gemm + w8a8_epilogue (backends/corex/kernels/w8a8.cu:195-211,
  * 289-336) and w8a8_gemm_tcu (backends/corex/kernels/w8a8_tcu.cu:276-384),

@@ -288,9 +288,13 @@ def test_gemm_w8a8_bit_exact(orc, gemm_tile, m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(16, 9728, 2560), (16, 2560, 9728), (1, 37, 128), (5, 530, 1152),
                                    (9, 100, 384), (12, 2560, 4096), (16, 256, 10240), (7, 300, 5120),
-                                   (2, 6144, 2560), (16, 64, 6656)])
+                                   (2, 6144, 2560), (16, 64, 6656),
+                                   # 17..128 rows per launch with the weight kept in registers (and two
+                                   # such launches): every lines-per-wavefront variant, ragged N and M
+                                   (17, 100, 9728), (48, 2560, 2560), (128, 333, 4096), (100, 77, 1024),
+                                   (33, 40, 10240), (200, 64, 9728), (64, 1200, 5120)])
 def test_gemm_w8a8_verify_batches_bit_exact(orc, monkeypatch, m, n, k):
-    """Up to 16 rows take the read-the-weight-once kernel: exact against the oracle, and the
+    """Few rows take the read-the-weight-once kernels: exact against the oracle, and the
     same bits as the tiled kernel gives for the same rows (also with a row stride)."""
     monkeypatch.delenv("CMI_GEMM_TILE", raising=False)
     g = seeded()
