@@ -309,16 +309,20 @@ extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     // fp32 chain, same bits.  Cost model fitted to measurements on the layer shapes (us).
     const char *force = getenv("CMI_GEMM_TILE");
     if (M <= 256 && !(force && force[0])) {
-        const double steps = K / 128.0;
+        const double steps = K / 128.0, wn = (double)N * K;
         const double tiles = (double)a_ceil(M, BM) * a_ceil(N, BN);
-        const double t_tiled = 3.0 + steps * 1.17 * ceil(tiles / 512.0);
-        // (rows beyond 10240 run the GEMV in passes: about half the speed)
-        const double t_rows16 = K <= 10240 ? a_ceil(M, 16) * (3.6 + (double)N * K / 2 / 4.2e6 + steps * 0.025)
-                                           : a_ceil(M, 16) * (3.6 + (double)N * K / 2 / 2.1e6);
+        const double t_tiled = 3.0 + steps * (tiles <= 512 ? 1.15 + 0.0013 * tiles : 1.8 * ceil(tiles / 512.0));
+        // up to 10240 elements per row the GEMV keeps the weight in registers for 128 rows per launch
+        // and pays per 16-row chunk only the chunk's sums and chain; longer rows run it in passes,
+        // 16 rows per launch, at about half the speed
+        const double t_rows16 =
+            K <= 10240 ? a_ceil(M, 128) * (2.0 + wn / 2 / 4.2e6) + a_ceil(M, 16) * (0.6 + wn / 1.3e7 + steps * 0.012)
+                       : a_ceil(M, 16) * (3.6 + wn / 2 / 2.1e6);
         if (t_rows16 < t_tiled) {
             const int G = K / BK;
-            for (int lo = 0; lo < M; lo += 16) {
-                const int m = M - lo < 16 ? M - lo : 16;
+            const int step = K <= 10240 ? 128 : 16;
+            for (int lo = 0; lo < M; lo += step) {
+                const int m = M - lo < step ? M - lo : step;
                 const int rc = gemv_w4a8_rows16(w4, ws, xq + (size_t)lo * K, xs + lo, nullptr,
                                                 static_cast<uint16_t *>(y) + (size_t)lo * N,
                                                 group_acc ? group_acc + (size_t)lo * G * N : nullptr, nullptr,

@@ -445,6 +445,165 @@ int launch_long(const Args &a, hipStream_t st) {
     return check_launch("cmi_gemv_w4a8");
 }
 
+
+// 17..128 quantised activation rows, K <= 10240: the workgroup's 16 weight rows are asked for once
+// and stay in registers as the MFMA pieces; the activation rows go through in chunks of 16, each
+// with the group sums, the barrier and the fp32 chain of the 16-row kernel (so the bits are the
+// same), the next chunk's activations requested as soon as this chunk's MFMAs have consumed their
+// registers.
+constexpr int MAX_CHUNKS = 8;
+
+template <int NLP, int WAVES, bool DUMP>
+__global__ void __launch_bounds__(WAVES * 64)
+gemv_w4a8_rows128_kernel(const Args a) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    int32_t *sums = reinterpret_cast<int32_t *>(lds);             // [G][64 lanes][4]
+    float *ws_lds = reinterpret_cast<float *>(lds + a.G * 1024);  // [16][G]
+    uint8_t *patches = lds + a.G * 1024 + ROWS * a.G * 4;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kq = lane >> 4;
+    const int n0 = blockIdx.x * ROWS;
+    const int lines = (a.G + 1) / 2;
+    const int chunks = (a.M + ROWS - 1) / ROWS;
+    uint8_t *patch = patches + wave * PATCH_BYTES;
+
+    v4i32 xa[NLP][2][2], w[NLP][2];
+    auto request_x = [&](int c) {
+#pragma unroll
+        for (int i = 0; i < NLP; ++i) {
+            const int line = wave + i * WAVES;
+            if (line >= lines) break;  // uniform per wavefront
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int g = min(2 * line + h, a.G - 1);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    xa[i][h][j] = *reinterpret_cast<const v4i32 *>(
+                        a.xq + tile_src(lane, j, c * ROWS, a.M - 1, a.K, g * GS));
+            }
+        }
+    };
+    request_x(0);
+    const int ws_total = min(ROWS, a.N - n0) * a.G;
+    constexpr int WSN = (ROWS * (MAX_K / GS) + WAVES * 64 - 1) / (WAVES * 64);
+    float wsreg[WSN];
+    {
+        const float *src = a.ws + (size_t)n0 * a.G;
+#pragma unroll
+        for (int i = 0; i < WSN; ++i) {
+            const int idx = threadIdx.x + i * (WAVES * 64);
+            wsreg[i] = idx < ws_total ? src[idx] : 0.f;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NLP; ++i) {
+        const int line = wave + i * WAVES;
+        if (line >= lines) break;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            w[i][j] = __builtin_nontemporal_load(reinterpret_cast<const v4i32 *>(
+                a.w4 + tile_src<true>(lane, j, n0, a.N - 1, a.K / 2, line * 128)));
+    }
+#pragma unroll
+    for (int i = 0; i < WSN; ++i) {
+        const int idx = threadIdx.x + i * (WAVES * 64);
+        if (idx < ws_total) ws_lds[idx] = wsreg[i];
+    }
+    // weights into the MFMA pieces, once: piece 4*h + kq of the line for group 2*line + h
+#pragma unroll
+    for (int i = 0; i < NLP; ++i) {
+        if (wave + i * WAVES >= lines) break;
+        tile_park(patch, lane, w[i][0], w[i][1]);
+        w[i][0] = tile_take(patch, lane, kq);
+        w[i][1] = tile_take(patch, lane, 4 + kq);
+    }
+
+    const int p = threadIdx.x, l = (p >> 2) & 63, v = p & 3;
+    const int nn = l & 15, n = n0 + nn;
+    const v4i32 minus8 = {(int)0xF8F8F8F8u, (int)0xF8F8F8F8u, (int)0xF8F8F8F8u, (int)0xF8F8F8F8u};
+#pragma unroll 1
+    for (int c = 0; c < chunks; ++c) {
+#pragma unroll
+        for (int i = 0; i < NLP; ++i) {
+            if (wave + i * WAVES >= lines) break;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                tile_park(patch, lane, xa[i][h][0], xa[i][h][1]);
+                xa[i][h][0] = tile_take(patch, lane, 2 * kq);
+                xa[i][h][1] = tile_take(patch, lane, 2 * kq + 1);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NLP; ++i) {
+            const int line = wave + i * WAVES;
+            if (line >= lines) break;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int g = 2 * line + h;
+                if (g >= a.G) break;  // uniform per wavefront
+                const u32x4 ww = __builtin_bit_cast(u32x4, w[i][h]);
+                const v4i32 x0 = {xa[i][h][0].x, xa[i][h][0].z, xa[i][h][1].x, xa[i][h][1].z};
+                const v4i32 x1 = {xa[i][h][0].y, xa[i][h][0].w, xa[i][h][1].y, xa[i][h][1].w};
+                const u32x4 lo = ww & 0x0F0F0F0Fu, hi = (ww >> 4) & 0x0F0F0F0Fu;
+                v4i32 acc = {0, 0, 0, 0};
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x0, minus8, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x1, minus8, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x0, __builtin_bit_cast(v4i32, lo), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(x1, __builtin_bit_cast(v4i32, hi), acc, 0, 0, 0);
+                reinterpret_cast<v4i32 *>(sums)[g * 64 + lane] = acc;
+            }
+        }
+        if (c + 1 < chunks) request_x(c + 1);
+        __syncthreads();
+        const int m = c * ROWS + 4 * (l >> 4) + v;
+        if (p < 256 && n < a.N && m < a.M) {
+            const int32_t *sp = sums + p;
+            const float *wsn = ws_lds + nn * a.G;
+            float total = 0.f;
+            int g = 0;
+            for (; g + 4 <= a.G; g += 4) {
+                int sv[4];
+                float wv[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    sv[i] = sp[(g + i) * 256];
+                    wv[i] = wsn[g + i];
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    if constexpr (DUMP) a.group_acc[((size_t)m * a.G + g + i) * a.N + n] = sv[i];
+                    total = fmaf((float)sv[i], wv[i], total);
+                }
+            }
+            for (; g < a.G; ++g) {
+                const int sg = sp[g * 256];
+                if constexpr (DUMP) a.group_acc[((size_t)m * a.G + g) * a.N + n] = sg;
+                total = fmaf((float)sg, wsn[g], total);
+            }
+            a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * a.xs[m]);
+        }
+        __syncthreads();  // the next chunk overwrites the sums
+    }
+}
+
+template <int NLP, int WAVES>
+int launch128(const Args &a, hipStream_t st) {
+    static std::atomic<uint64_t> devices{0};
+    const void *fn = a.group_acc ? reinterpret_cast<const void *>(gemv_w4a8_rows128_kernel<NLP, WAVES, true>)
+                                 : reinterpret_cast<const void *>(gemv_w4a8_rows128_kernel<NLP, WAVES, false>);
+    static std::atomic<uint64_t> devices_dump{0};
+    if (const int rc = reserve_lds(fn, lds_bytes(MAX_K / GS, WAVES), a.group_acc ? devices_dump : devices, "cmi_gemv_w4a8"))
+        return rc;
+    const dim3 grid((a.N + ROWS - 1) / ROWS);
+    if (a.group_acc)
+        gemv_w4a8_rows128_kernel<NLP, WAVES, true><<<grid, dim3(WAVES * 64), lds_bytes(a.G, WAVES), st>>>(a);
+    else
+        gemv_w4a8_rows128_kernel<NLP, WAVES, false><<<grid, dim3(WAVES * 64), lds_bytes(a.G, WAVES), st>>>(a);
+    return check_launch("cmi_gemv_w4a8");
+}
+
 }  // namespace
 
 namespace cmi {
@@ -456,8 +615,8 @@ namespace cmi {
 int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs, const void *x,
                      void *y, int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
                      void *stream) {
-    if (M < 1 || M > (x ? FUSED_ROWS : ROWS) || K < GS || K % GS != 0 || N < 1) return CMI_E_UNSUPPORTED;
-    if (K > MAX_K && (x || (size_t)K * M > ((size_t)1 << 31))) return CMI_E_UNSUPPORTED;
+    if (M < 1 || M > (x ? FUSED_ROWS : MAX_CHUNKS * ROWS) || K < GS || K % GS != 0 || N < 1) return CMI_E_UNSUPPORTED;
+    if (K > MAX_K && (x || M > ROWS)) return CMI_E_UNSUPPORTED;
     Args a;
     a.w4 = w4;
     a.ws = ws;
@@ -480,6 +639,24 @@ int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const
     // faster at N = 2560..9728); four on larger grids (7 % faster at N = 151936).
     const int grid = (N + ROWS - 1) / ROWS;
     const bool eight = lines > 20 || (grid <= 640 && lines >= 8);
+    if (M > ROWS) {
+        if (!eight) {
+            switch ((lines + 3) / 4) {
+                case 1: return launch128<1, 4>(a, st);
+                case 2: return launch128<2, 4>(a, st);
+                case 3: return launch128<3, 4>(a, st);
+                case 4: return launch128<4, 4>(a, st);
+                default: return launch128<5, 4>(a, st);
+            }
+        }
+        switch ((lines + 7) / 8) {
+            case 1: return launch128<1, 8>(a, st);
+            case 2: return launch128<2, 8>(a, st);
+            case 3: return launch128<3, 8>(a, st);
+            case 4: return launch128<4, 8>(a, st);
+            default: return launch128<5, 8>(a, st);
+        }
+    }
     if (!eight) {
         switch ((lines + 3) / 4) {
             case 1: return launch<1, 4>(a, st);

@@ -84,7 +84,7 @@ int cmi_gemv_w8a16_mfma(const int8_t *wq, const float *ws, const void *x, void *
 int cmi_w4_repack(const uint8_t *packed, const float *scale, uint8_t *w4, float *ws,
                   int N, int K, int gs, void *stream);
 
-/* W4A8 GEMV, 1 <= M <= 16, on the re-laid-out weight:
+/* W4A8 GEMV, 1 <= M <= 16 (up to 128 when K <= 10240), on the re-laid-out weight:
  *   sum_g = sum_{k in g} xq[m,k]*(code-8)           (int32, exact)
  *   total = fma((float)sum_g, ws[n,g], total)        (g ascending, from 0)
  *   y[m,n] = bf16(total * xs[m])

@@ -406,7 +406,11 @@ def test_gemv_w4a8_bf16_refuses_wide_batches():
 
 @pytest.mark.parametrize("m,n,k", [(128, 128, 128), (64, 256, 256), (512, 2560, 2560),
                                    (256, 1280, 5120), (100, 200, 384), (1, 1024, 2560),
-                                   (16, 300, 2560)])
+                                   (16, 300, 2560),
+                                   # 17..128 rows per launch of the matrix-pipe GEMV (weight kept in
+                                   # registers, 16-row chunks), and two such launches
+                                   (48, 2560, 2560), (128, 300, 9728), (100, 77, 1024), (33, 40, 10240),
+                                   (200, 64, 4096), (17, 1000, 6656)])
 def test_gemm_w4a8_bit_exact(orc, m, n, k):
     w4, ws, xq, xs, gacc_ref, y_ref = _w4_case(orc, m, n, k, seeded())
     gacc, y = G.w4a8(w4, ws, xq, xs, k, gemm=True)
