@@ -345,6 +345,24 @@ def test_gemm_w8a8_full_size_sampled_and_blockwise(orc, gemm_tile, m, n):
     assert float(acc.double().sum()) == float(total)
 
 
+@pytest.mark.parametrize("n,k", [(9728, 2560), (2560, 9728), (6144, 2560)])
+def test_gemm_w8a8_full_size_mid_batches_equal_the_tile_pipeline(n, k, monkeypatch):
+    """17..256 rows at the layer shapes: whatever route the entry picks (weight kept in
+    registers for up to 128 rows per launch, or tiles) gives the bits of the tile pipeline,
+    and a row does not depend on the batch it came in."""
+    g = synth.generator(1234, G.DEV)
+    q = synth.int8_weight(n, k, g)
+    x = synth.activations(256, k, g, outliers=True)
+    xq, xs = G.quant(x)
+    monkeypatch.setenv("CMI_GEMM_TILE", "128")
+    acc_t, y_t = G.gemm_w8a8(xq, q.wq, xs, q.scale)
+    monkeypatch.delenv("CMI_GEMM_TILE")
+    for m in (17, 48, 128, 129, 200, 256):
+        acc, y = G.gemm_w8a8(xq[:m].contiguous(), q.wq, xs[:m].contiguous(), q.scale)
+        assert (acc == acc_t[:m]).all(), m
+        assert (y.view(torch.int16) == y_t[:m].view(torch.int16)).all(), m
+
+
 # ------------------------------------------------------------ W4A8 GEMV / GEMM
 
 def _w4_case(orc, m, n, k, g):
@@ -449,7 +467,7 @@ def test_w4_repack_is_a_permutation_of_the_codes():
 
 
 @pytest.mark.parametrize("n,k", [(9728, 2560), (2560, 9728), (5120, 25600)])
-def test_w4a8_full_size_gemv_equals_gemm_rows(n, k):
+def test_w4a8_full_size_gemv_equals_gemm_rows(n, k, monkeypatch):
     """At benchmark sizes the GEMV and the MFMA GEMM must agree bit for bit (the
     arithmetic is the same by definition), and a batched GEMV row must equal the
     single-row call."""
@@ -458,7 +476,13 @@ def test_w4a8_full_size_gemv_equals_gemm_rows(n, k):
     w4, ws = G.w4_repack(w.packed, w.scale, k)
     x = synth.activations(64, k, g)
     xq, xs = G.quant(x)
+    # the tile pipeline itself (at 64 rows the entry would otherwise pick the read-once kernel),
+    # then the entry's own choice: same bits
+    monkeypatch.setenv("CMI_GEMM_TILE", "128")
     ga_mm, y_mm = G.w4a8(w4, ws, xq, xs, k, gemm=True)
+    monkeypatch.delenv("CMI_GEMM_TILE")
+    ga_auto, y_auto = G.w4a8(w4, ws, xq, xs, k, gemm=True)
+    assert (ga_auto == ga_mm).all() and (y_auto.view(torch.int16) == y_mm.view(torch.int16)).all()
     ga_mv, y_mv = G.w4a8(w4, ws, xq[:16].contiguous(), xs[:16].contiguous(), k, gemm=False)
     assert (ga_mv == ga_mm[:16]).all()
     assert (y_mv.view(torch.int16) == y_mm[:16].view(torch.int16)).all()
