@@ -386,7 +386,7 @@ def main() -> int:
             xq = torch.empty((m, k_), dtype=torch.int8, device=dev)
             xs = torch.empty(m, dtype=torch.float32, device=dev)
             y = torch.empty((m, n_), dtype=torch.bfloat16, device=dev)
-            rows_per_call = 64 if k_ <= 5120 else 16
+            rows_per_call = 64
             def weight_only():
                 st = cur_stream()
                 for q in w8:

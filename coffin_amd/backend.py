@@ -45,10 +45,9 @@ from coffin_amd import _native
 
 #: Widest batch the GEMV kernels take in one launch.
 GEMV_MAX_ROWS = 16
-#: The matrix-pipe weight-only GEMV takes this many when K <= 5120 (the weight is read once, the
-#: activation rows go through in chunks of 16 inside the kernel: same bits as 16-row calls).
+#: The matrix-pipe weight-only GEMV takes this many (the weight is read once, the activation rows
+#: go through in chunks of 16 inside the kernel: same bits as 16-row calls).
 GEMV_MFMA_MAX_ROWS = 64
-GEMV_MFMA_WIDE_MAX_K = 5120
 #: From this many rows ``linear_prefill`` quantizes activations and runs the
 #: int8 MFMA GEMM (the reference's corex backend draws the same line at 64,
 #: backends/corex/__init__.py:633,1655-1659).
@@ -260,7 +259,7 @@ def _gemv_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor, mfma
             if mfma and (BATCH_MFMA or rows >= MFMA_MIN_ROWS) and k % 128 == 0 and k <= 10240 else None)
     stream = _stream()
     x0, y0 = act.data_ptr(), out.data_ptr()
-    step = GEMV_MFMA_MAX_ROWS if fast is not None and k <= GEMV_MFMA_WIDE_MAX_K else GEMV_MAX_ROWS
+    step = GEMV_MFMA_MAX_ROWS if fast is not None else GEMV_MAX_ROWS
     for lo in range(0, rows, step):
         m = min(step, rows - lo)
         # every chunk of a fast call takes the fast kernel, also a short last one: a row's bits

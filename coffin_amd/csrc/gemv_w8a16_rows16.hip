@@ -180,14 +180,16 @@ int launch(const Args &a, hipStream_t st) {
 }
 
 
-// 17..64 activation rows, K up to 128*NLP*WAVES (one round): the workgroup still asks for its
-// 16 weight rows once and keeps them in registers in the MFMA arrangement; the activation rows
-// go through in chunks of 16, each with the arithmetic of the kernel above -- so a row's bits are
+// 17..64 activation rows: the workgroup still asks for its 16 weight rows once and keeps them in
+// registers in the MFMA arrangement (NLP*ROUNDS lines per wavefront); the activation rows go
+// through in chunks of 16, each with the arithmetic of the kernel above -- so a row's bits are
 // the same as in a 16-row call -- and only the activations (L2 resident) and the widening are
-// paid again per chunk.  The partial tiles of all chunks meet in LDS behind one barrier.
+// paid again per chunk.  The activation registers hold NLP lines: with two rounds a chunk is two
+// such batches, and the batch after the one in hand is requested line by line as its registers
+// free up.  The partial tiles of all chunks meet in LDS behind one barrier.
 constexpr int MAX_CHUNKS = 4;
 
-template <int NLP, int WAVES>
+template <int NLP, int WAVES, int ROUNDS>
 __global__ void __launch_bounds__(WAVES * 64)
 gemv_w8a16_rows64_kernel(const Args a) {
     extern __shared__ __align__(16) uint8_t lds[];
@@ -202,29 +204,31 @@ gemv_w8a16_rows64_kernel(const Args a) {
     const int lines = a.K / LINE;
     uint8_t *wpatch = patches + wave * (PATCH_BYTES + XPATCH_BYTES), *xpatch = wpatch + PATCH_BYTES;
     const uint8_t *xbytes = reinterpret_cast<const uint8_t *>(a.x);
-    auto line_of = [&](int i) { return i * WAVES + wave; };
+    auto line_of = [&](int r, int i) { return (r * NLP + i) * WAVES + wave; };
 
-    v4i32 xr[NLP][4], wr[NLP][2];
-    auto request_x = [&](int c, int i) {
-        const int line = min(line_of(i), lines - 1);  // a slot past the last line is not used
+    v4i32 xr[NLP][4], wr[ROUNDS * NLP][2];
+    auto request_x = [&](int c, int r, int i) {
+        const int line = min(line_of(r, i), lines - 1);  // a slot past the last line is not used
 #pragma unroll
         for (int q = 0; q < 4; ++q)
             xr[i][q] = *reinterpret_cast<const v4i32 *>(
                 xbytes + tile_src(lane, q & 1, c * ROWS, a.M - 1, (size_t)a.K * 2, line * 256 + (q >> 1) * 128));
     };
 #pragma unroll
-    for (int i = 0; i < NLP; ++i) request_x(0, i);
+    for (int i = 0; i < NLP; ++i) request_x(0, 0, i);
 #pragma unroll
-    for (int i = 0; i < NLP; ++i) {
-        const int line = min(line_of(i), lines - 1);
+    for (int r = 0; r < ROUNDS; ++r)
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
-            wr[i][h] = __builtin_nontemporal_load(
-                reinterpret_cast<const v4i32 *>(a.wq + tile_src(lane, h, n0, a.N - 1, a.K, line * LINE)));
-    }
+        for (int i = 0; i < NLP; ++i) {
+            const int line = min(line_of(r, i), lines - 1);
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                wr[r * NLP + i][h] = __builtin_nontemporal_load(
+                    reinterpret_cast<const v4i32 *>(a.wq + tile_src(lane, h, n0, a.N - 1, a.K, line * LINE)));
+        }
     // weights into the MFMA arrangement, once
 #pragma unroll
-    for (int i = 0; i < NLP; ++i) {
+    for (int i = 0; i < ROUNDS * NLP; ++i) {
         tile_park(wpatch, lane, wr[i][0], wr[i][1]);
         wr[i][0] = tile_take(wpatch, lane, 2 * kq);
         wr[i][1] = tile_take(wpatch, lane, 2 * kq + 1);
@@ -232,36 +236,43 @@ gemv_w8a16_rows64_kernel(const Args a) {
 
 #pragma unroll 1
     for (int c = 0; c < chunks; ++c) {
-        // activations of this chunk into the MFMA arrangement: row lane%16, bytes 64*kq .. +63
-#pragma unroll
-        for (int i = 0; i < NLP; ++i) {
-            uint8_t *p = xpatch + (lane >> 3) * XPITCH + (lane & 7) * 16;
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                *reinterpret_cast<v4i32 *>(p + (q & 1) * 8 * XPITCH + (q >> 1) * 128) = xr[i][q];
-            const uint8_t *t = xpatch + (lane & 15) * XPITCH + kq * 64;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) xr[i][q] = *reinterpret_cast<const v4i32 *>(t + q * 16);
-        }
         v4f32 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int i = 0; i < NLP; ++i) {
-            if (line_of(i) < lines) {  // uniform per wavefront
-                const uint32_t d[8] = {(uint32_t)wr[i][0].x, (uint32_t)wr[i][0].y, (uint32_t)wr[i][0].z,
-                                       (uint32_t)wr[i][0].w, (uint32_t)wr[i][1].x, (uint32_t)wr[i][1].y,
-                                       (uint32_t)wr[i][1].z, (uint32_t)wr[i][1].w};
+        for (int r = 0; r < ROUNDS; ++r) {
+            // this batch of activation lines into the MFMA arrangement: row lane%16, bytes 64*kq .. +63
 #pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    uint32_t b[4];
-                    widen4(d[2 * s], b[0], b[1]);
-                    widen4(d[2 * s + 1], b[2], b[3]);
-                    const v4i32 bw = {(int)b[0], (int)b[1], (int)b[2], (int)b[3]};
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xr[i][s]),
-                                                                  __builtin_bit_cast(bf16x8, bw), acc, 0, 0, 0);
-                }
+            for (int i = 0; i < NLP; ++i) {
+                uint8_t *p = xpatch + (lane >> 3) * XPITCH + (lane & 7) * 16;
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    *reinterpret_cast<v4i32 *>(p + (q & 1) * 8 * XPITCH + (q >> 1) * 128) = xr[i][q];
+                const uint8_t *t = xpatch + (lane & 15) * XPITCH + kq * 64;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) xr[i][q] = *reinterpret_cast<const v4i32 *>(t + q * 16);
             }
-            // this line's activation registers are free: ask for the next chunk's
-            if (c + 1 < chunks) request_x(c + 1, i);
+#pragma unroll
+            for (int i = 0; i < NLP; ++i) {
+                if (line_of(r, i) < lines) {  // uniform per wavefront
+                    v4i32 w0 = wr[r * NLP + i][0], w1 = wr[r * NLP + i][1];
+                    // with two rounds of weight registers the widened copies must not be kept
+                    // across chunks (the compiler would hoist them out of the loop and spill)
+                    if (ROUNDS > 1) asm volatile("" : "+v"(w0), "+v"(w1));
+                    const uint32_t d[8] = {(uint32_t)w0.x, (uint32_t)w0.y, (uint32_t)w0.z, (uint32_t)w0.w,
+                                           (uint32_t)w1.x, (uint32_t)w1.y, (uint32_t)w1.z, (uint32_t)w1.w};
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) {
+                        uint32_t b[4];
+                        widen4(d[2 * s], b[0], b[1]);
+                        widen4(d[2 * s + 1], b[2], b[3]);
+                        const v4i32 bw = {(int)b[0], (int)b[1], (int)b[2], (int)b[3]};
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xr[i][s]),
+                                                                      __builtin_bit_cast(bf16x8, bw), acc, 0, 0, 0);
+                    }
+                }
+                // this line's activation registers are free: ask for the same slot of the next batch
+                if (r + 1 < ROUNDS) request_x(c, r + 1, i);
+                else if (c + 1 < chunks) request_x(c + 1, 0, i);
+            }
         }
         *reinterpret_cast<v4f32 *>(&partial[c * WAVES + wave][lane][0]) = acc;
     }
@@ -279,17 +290,17 @@ gemv_w8a16_rows64_kernel(const Args a) {
     }
 }
 
-template <int NLP, int WAVES>
+template <int NLP, int WAVES, int ROUNDS = 1>
 int launch64(const Args &a, hipStream_t st) {
     constexpr int LDS_MAX = MAX_CHUNKS * WAVES * 1024 + WAVES * (PATCH_BYTES + XPATCH_BYTES);
     static std::atomic<uint64_t> devices{0};
-    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w8a16_rows64_kernel<NLP, WAVES>), LDS_MAX,
-                                   devices, "cmi_gemv_w8a16_mfma"))
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w8a16_rows64_kernel<NLP, WAVES, ROUNDS>),
+                                   LDS_MAX, devices, "cmi_gemv_w8a16_mfma"))
         return rc;
     const int chunks = (a.M + ROWS - 1) / ROWS;
     const int lds_bytes = chunks * WAVES * 1024 + WAVES * (PATCH_BYTES + XPATCH_BYTES);
     const dim3 grid((a.N + ROWS - 1) / ROWS);
-    gemv_w8a16_rows64_kernel<NLP, WAVES><<<grid, dim3(WAVES * 64), lds_bytes, st>>>(a);
+    gemv_w8a16_rows64_kernel<NLP, WAVES, ROUNDS><<<grid, dim3(WAVES * 64), lds_bytes, st>>>(a);
     return check_launch("cmi_gemv_w8a16_mfma");
 }
 
@@ -299,8 +310,6 @@ extern "C" int cmi_gemv_w8a16_mfma(const int8_t *wq, const float *ws, const void
                                    int K, void *stream) {
     CMI_REQUIRE(wq && ws && x && y, CMI_E_ARG, "cmi_gemv_w8a16_mfma: null pointer");
     CMI_REQUIRE(M >= 1 && M <= MAX_CHUNKS * ROWS, CMI_E_UNSUPPORTED, "cmi_gemv_w8a16_mfma: M=%d outside 1..64", M);
-    CMI_REQUIRE(M <= ROWS || K <= 40 * LINE, CMI_E_UNSUPPORTED,
-                "cmi_gemv_w8a16_mfma: M=%d rows need K <= 5120 (K=%d): call with 16 rows at a time", M, K);
     CMI_REQUIRE(N >= 1 && K >= 1, CMI_E_ARG, "cmi_gemv_w8a16_mfma: bad shape N=%d K=%d", N, K);
     CMI_REQUIRE(K % LINE == 0 && K <= 80 * LINE, CMI_E_UNSUPPORTED,
                 "cmi_gemv_w8a16_mfma: K=%d is not a multiple of 128 up to 10240 (use cmi_gemv_w8a16)", K);
@@ -320,7 +329,8 @@ extern "C" int cmi_gemv_w8a16_mfma(const int8_t *wq, const float *ws, const void
         if (lines <= 8) return launch64<2, 4>(a, st);
         if (lines <= 20 && (N + ROWS - 1) / ROWS > 2048) return launch64<5, 4>(a, st);
         if (lines <= 24) return launch64<3, 8>(a, st);
-        return launch64<5, 8>(a, st);
+        if (lines <= 40) return launch64<5, 8>(a, st);
+        return launch64<5, 8, 2>(a, st);
     }
     // eight wavefronts (shorter chains of dependent steps) up to 2048 workgroups, four beyond
     // (2560 -> 151936: 72 us against 84)

@@ -58,9 +58,9 @@ int cmi_gemv_w8a16(const int8_t *wq, const float *ws, const void *x, void *y,
 
 /* The same product for a batch with the sums on the matrix pipe
  * (v_mfma_f32_16x16x32_bf16; int8 -> bf16 is exact), 1 <= M <= 16,
- * K % 128 == 0, K <= 10240 (else CMI_E_UNSUPPORTED: use cmi_gemv_w8a16); up
- * to 64 rows when K <= 5120 (the weight is still read once, the rows go
- * through in chunks of 16 with the 16-row arithmetic).
+ * K % 128 == 0, K <= 10240 (else CMI_E_UNSUPPORTED: use cmi_gemv_w8a16); also
+ * up to 64 rows (the weight is still read once, the rows go through in chunks
+ * of 16 with the 16-row arithmetic).
  * 2-3 times faster than cmi_gemv_w8a16 at 8-16 rows.  A row's bits depend on K
  * only, not on the rows it travels with, but differ from cmi_gemv_w8a16's in
  * the last place (fp32 summation order): for callers without the

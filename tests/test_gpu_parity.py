@@ -134,9 +134,10 @@ def test_gemv_w8a16_mfma_within_tolerance(orc, m, n, k):
     _assert_weight_only_tolerance(orc, wq, ws, x, y)
 
 
-@pytest.mark.parametrize("n,k", [(9728, 2560), (300, 5120), (70, 1024), (33000, 2560), (2560, 4096)])
+@pytest.mark.parametrize("n,k", [(9728, 2560), (300, 5120), (70, 1024), (33000, 2560), (2560, 4096),
+                                 (2560, 9728), (100, 10240), (77, 6656)])
 def test_gemv_w8a16_mfma_wide_batches_carry_the_16_row_bits(n, k):
-    """17..64 rows in one launch (K <= 5120): every row has the bits of a 16-row call."""
+    """17..64 rows in one launch: every row has the bits of a 16-row call."""
     g = seeded()
     q = synth.int8_weight(n, k, g)
     wq, ws = q.wq.to(G.DEV), q.scale.to(G.DEV)
