@@ -66,7 +66,7 @@ W8A8_VERIFY = os.environ.get("COFFIN_AMD_W8A8_VERIFY", "0").strip() == "1"
 #: numbers), so ``linear`` and ``linear_m`` on int8 weights stay on the dot-product GEMV, whose
 #: summation order depends on K only.  ``linear_m_verify`` (which may use a path of its own,
 #: backends/protocol.py:152-155) and short ``linear_prefill`` chunks do not carry that obligation
-#: and take the matrix-pipe GEMV from three rows up: 3-4 times faster at 8-16 rows, same
+#: and take the matrix-pipe GEMV from three rows up: 1.5-2.8 times faster at 8-16 rows, same
 #: weight-only arithmetic, last-place differences from fp32 summation order.
 #: ``COFFIN_AMD_BATCH_MFMA=1`` moves *every* int8 weight-only call -- ``linear`` included, one row
 #: included -- to the matrix-pipe GEMV: the contract holds again (one kernel family, a row's bits
