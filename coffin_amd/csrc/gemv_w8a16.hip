@@ -37,9 +37,12 @@
 // weights in flight.  When K spans several units the wavefronts of a team each take units
 // of the same rows and the unit totals meet in LDS (summed in unit order by one
 // lane per output); otherwise lane 63, which holds the tree result, scales and
-// stores.
+// stores.  A single activation row against a K of two or three units takes
+// gemv_w8a16_wholerow_kernel instead: one wavefront per weight row, all units.
 
 #include "common.hpp"
+
+#include <cstdlib>
 
 namespace {
 
@@ -417,6 +420,105 @@ gemv_w8a16_kernel(const GemvArgs a) {
     }
 }
 
+// One activation row, K in two or three units of one sub-trip each: a wavefront owns a whole
+// weight row -- all units, every byte requested up front -- and adds its unit totals in lane
+// 63 in the canonical order, so there is no exchange through LDS and no second barrier, and a
+// workgroup of W wavefronts stages the activation row once for W weight rows (the team
+// arrangement of the general kernel stages it once per two rows).  Same bits.
+template <int CHT, int NU, int XV>
+__global__ void __launch_bounds__(256)
+gemv_w8a16_wholerow_kernel(const GemvArgs a) {
+    extern __shared__ uint4 smem[];  // the activation row, then one zeroed 32-byte slot
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int waves = blockDim.x >> 6;
+    const int n_raw = blockIdx.x * waves + wave;
+    const int n = n_raw < a.N ? n_raw : a.N - 1;
+    const int8_t *wrow = a.wq + (size_t)n * a.K;
+    const int xvecs = a.K / 8;
+
+    uint4 xstage[XV];
+    const uint4 *xg = reinterpret_cast<const uint4 *>(a.x);
+#pragma unroll
+    for (int j = 0; j < XV; ++j) {
+        const int idx = threadIdx.x + j * blockDim.x;
+        xstage[j] = idx < xvecs ? xg[idx] : make_uint4(0, 0, 0, 0);
+    }
+    u32x4 w[NU][CHT];
+#pragma unroll
+    for (int u = 0; u < NU; ++u)
+#pragma unroll
+        for (int j = 0; j < CHT; ++j) {
+            const int chunk = ((u * CHT + j) * 64 + lane);
+            w[u][j] = __builtin_nontemporal_load(
+                reinterpret_cast<const u32x4 *>(wrow + (uint32_t)min(chunk, a.nchunks - 1) * 16u));
+        }
+    int vzero = 0;
+    asm volatile("" : "+v"(vzero));
+    const float scale = a.ws[n + vzero];
+#pragma unroll
+    for (int j = 0; j < XV; ++j) {
+        const int idx = threadIdx.x + j * blockDim.x;
+        if (idx < xvecs) smem[idx] = xstage[j];
+    }
+    if (threadIdx.x < 2) smem[xvecs + threadIdx.x] = make_uint4(0, 0, 0, 0);
+    __syncthreads();
+
+    float total = 0.f;
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+        const int seg_end = min((u + 1) * CHT, a.nseg);
+        float v = 0.f;
+#pragma unroll
+        for (int j = 0; j < CHT; ++j) {
+            const int seg = u * CHT + j;
+            const int chunk = seg * 64 + lane;
+            const bool live = seg < seg_end && chunk < a.nchunks;
+            const int at = live ? 2 * chunk : xvecs;
+            const uint4 x0 = smem[at], x1 = smem[at + 1];
+            bf16x2_t wb[8];
+            widen4(w[u][j].x, wb[0], wb[1]);
+            widen4(w[u][j].y, wb[2], wb[3]);
+            widen4(w[u][j].z, wb[4], wb[5]);
+            widen4(w[u][j].w, wb[6], wb[7]);
+            const uint32_t xv[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                v = __builtin_amdgcn_fdot2_f32_bf16(wb[i], __builtin_bit_cast(bf16x2_t, xv[i]), v, false);
+        }
+        v = wave_sum_to_lane63(v);
+        total = u == 0 ? v : total + v;
+    }
+    if (lane == 63 && n_raw < a.N) a.y[n] = (uint16_t)f32_to_bf16_bits(scale * total);
+}
+
+//: Wavefronts per workgroup of the whole-row kernel (2, 3, 5, 6 and 8 measured slower:
+//: 9728 -> 2560 takes 7.2, 7.5, 7.3, 7.7 and 8.0 us against 6.7).
+constexpr int WHOLEROW_WAVES = 4;
+//: 16-byte vectors of the activation row per thread: K <= 12288, which three units cannot exceed.
+constexpr int WHOLEROW_XV = 6;
+
+template <int CHT, int NU>
+int launch_wholerow(const GemvArgs &a, hipStream_t st) {
+    const size_t lds = 16 * (size_t)(a.K / 8 + 2);
+    const dim3 grid((a.N + WHOLEROW_WAVES - 1) / WHOLEROW_WAVES), block(64 * WHOLEROW_WAVES);
+    gemv_w8a16_wholerow_kernel<CHT, NU, WHOLEROW_XV><<<grid, block, lds, st>>>(a);
+    return check_launch("cmi_gemv_w8a16");
+}
+
+// CMI_E_UNSUPPORTED (no error text) when the shape is not one this kernel takes.
+int dispatch_wholerow(const GemvArgs &a, hipStream_t st) {
+    if (a.K / 8 > WHOLEROW_XV * 64 * WHOLEROW_WAVES) return CMI_E_UNSUPPORTED;
+    if (a.units == 2) {
+        if (a.unit == 4) return launch_wholerow<4, 2>(a, st);
+        if (a.unit == 3) return launch_wholerow<3, 2>(a, st);
+    } else if (a.units == 3) {
+        if (a.unit == 4) return launch_wholerow<4, 3>(a, st);
+        if (a.unit == 3) return launch_wholerow<3, 3>(a, st);
+    }
+    return CMI_E_UNSUPPORTED;
+}
+
 struct Plan {
     int mt, r, cht, mode;
 };
@@ -564,6 +666,15 @@ extern "C" int cmi_gemv_w8a16(const int8_t *wq, const float *ws, const void *x, 
         return cmi_gemv_w8a16(wq, ws, a.x + (size_t)half * K, a.y + (size_t)half * N, M - half, N, K, stream);
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
+    // One row of a long K (two or three units): a wavefront per weight row.  CMI_GEMV_WHOLEROW=0
+    // keeps the team kernel (the tests compare the two bit for bit).
+    if (M == 1 && p.mode == 1) {
+        const char *e = getenv("CMI_GEMV_WHOLEROW");
+        if (!(e && e[0] == '0')) {
+            const int rc = dispatch_wholerow(a, st);
+            if (rc != CMI_E_UNSUPPORTED) return rc;
+        }
+    }
     switch (p.mt) {
         case 1: return dispatch_r<1>(a, p, st);
         case 2: return dispatch_r<2>(a, p, st);

@@ -124,6 +124,25 @@ def test_gemv_w8a16_within_tolerance(orc, m, n, k):
     _assert_weight_only_tolerance(orc, wq, ws, x, y)
 
 
+@pytest.mark.parametrize("n,k", [(2560, 9728), (2560, 9216), (333, 4112), (1001, 6160), (50, 7168),
+                                 (2, 12288), (5120, 8192), (77, 5120), (640, 11280)])
+def test_gemv_w8a16_whole_row_kernel_gives_the_team_kernels_bits(orc, monkeypatch, n, k):
+    """One row against a K of two or three units runs a wavefront per weight row; with
+    CMI_GEMV_WHOLEROW=0 the library keeps the team kernel.  Both follow the canonical
+    summation order, so their outputs agree bit for bit (ragged N, K with dead chunks and
+    dead segments, both unit widths), and the result is within the oracle's tolerance."""
+    g = seeded()
+    q = synth.int8_weight(n, k, g)
+    x = synth.activations(1, k, g)
+    args = (q.wq.to(G.DEV), q.scale.to(G.DEV), x.to(G.DEV))
+    monkeypatch.delenv("CMI_GEMV_WHOLEROW", raising=False)
+    y = G.gemv_w8a16(*args)
+    monkeypatch.setenv("CMI_GEMV_WHOLEROW", "0")
+    y_team = G.gemv_w8a16(*args)
+    assert (y.view(torch.int16) == y_team.view(torch.int16)).all()
+    _assert_weight_only_tolerance(orc, q.wq.numpy(), q.scale.numpy(), x, y)
+
+
 @pytest.mark.parametrize("m,n,k", [(16, 9728, 2560), (5, 2560, 9728), (7, 37, 128), (9, 100, 384),
                                    (16, 64, 10240), (6, 530, 1152), (1, 333, 2560), (3, 2560, 4096),
                                    (16, 1024, 5120), (12, 640, 3072), (2, 96, 8192), (16, 300, 6656)])
