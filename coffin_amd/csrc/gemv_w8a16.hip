@@ -37,8 +37,9 @@
 // weights in flight.  When K spans several units the wavefronts of a team each take units
 // of the same rows and the unit totals meet in LDS (summed in unit order by one
 // lane per output); otherwise lane 63, which holds the tree result, scales and
-// stores.  A single activation row against a K of two or three units takes
-// gemv_w8a16_wholerow_kernel instead: one wavefront per weight row, all units.
+// stores.  A single activation row against a K of two or three units (and against a
+// mid-sized weight with K in one unit) takes gemv_w8a16_wholerow_kernel instead: one
+// wavefront per weight row, all units.
 
 #include "common.hpp"
 
@@ -420,7 +421,7 @@ gemv_w8a16_kernel(const GemvArgs a) {
     }
 }
 
-// One activation row, K in two or three units of one sub-trip each: a wavefront owns a whole
+// One activation row, K in up to three units of one sub-trip each: a wavefront owns a whole
 // weight row -- all units, every byte requested up front -- and adds its unit totals in lane
 // 63 in the canonical order, so there is no exchange through LDS and no second barrier, and a
 // workgroup of W wavefronts stages the activation row once for W weight rows (the team
@@ -509,6 +510,18 @@ int launch_wholerow(const GemvArgs &a, hipStream_t st) {
 // CMI_E_UNSUPPORTED (no error text) when the shape is not one this kernel takes.
 int dispatch_wholerow(const GemvArgs &a, hipStream_t st) {
     if (a.K / 8 > WHOLEROW_XV * 64 * WHOLEROW_WAVES) return CMI_E_UNSUPPORTED;
+    if (a.units == 1) {
+        // K in one unit: the general kernel is as good or better for small launches (one weight row per
+        // wavefront there too, padded activation copy without selects: 4096 -> 2560 3.85 against 3.91 us)
+        // and for very tall weights; in between this kernel is 2-4 % faster (2560 -> 19456 9.7 -> 9.4 us,
+        // 2560 -> 9728 6.03 -> 5.81 us; two weight rows per wavefront here measured slower again).
+        const size_t wbytes = (size_t)a.N * a.K;
+        if (wbytes <= ((size_t)20 << 20) || wbytes > ((size_t)128 << 20)) return CMI_E_UNSUPPORTED;
+        if (a.unit == 4) return launch_wholerow<4, 1>(a, st);
+        if (a.unit == 3) return launch_wholerow<3, 1>(a, st);
+        if (a.unit == 2) return launch_wholerow<2, 1>(a, st);
+        return CMI_E_UNSUPPORTED;
+    }
     if (a.units == 2) {
         if (a.unit == 4) return launch_wholerow<4, 2>(a, st);
         if (a.unit == 3) return launch_wholerow<3, 2>(a, st);
@@ -666,9 +679,10 @@ extern "C" int cmi_gemv_w8a16(const int8_t *wq, const float *ws, const void *x, 
         return cmi_gemv_w8a16(wq, ws, a.x + (size_t)half * K, a.y + (size_t)half * N, M - half, N, K, stream);
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
-    // One row of a long K (two or three units): a wavefront per weight row.  CMI_GEMV_WHOLEROW=0
-    // keeps the team kernel (the tests compare the two bit for bit).
-    if (M == 1 && p.mode == 1) {
+    // One row of a long K (two or three units), or of a mid-sized weight with K in one unit: a
+    // wavefront per weight row.  CMI_GEMV_WHOLEROW=0 keeps the general kernel (the tests compare
+    // the two bit for bit).
+    if (M == 1 && p.mode != 2) {
         const char *e = getenv("CMI_GEMV_WHOLEROW");
         if (!(e && e[0] == '0')) {
             const int rc = dispatch_wholerow(a, st);

@@ -125,12 +125,15 @@ def test_gemv_w8a16_within_tolerance(orc, m, n, k):
 
 
 @pytest.mark.parametrize("n,k", [(2560, 9728), (2560, 9216), (333, 4112), (1001, 6160), (50, 7168),
-                                 (2, 12288), (5120, 8192), (77, 5120), (640, 11280)])
-def test_gemv_w8a16_whole_row_kernel_gives_the_team_kernels_bits(orc, monkeypatch, n, k):
-    """One row against a K of two or three units runs a wavefront per weight row; with
-    CMI_GEMV_WHOLEROW=0 the library keeps the team kernel.  Both follow the canonical
-    summation order, so their outputs agree bit for bit (ragged N, K with dead chunks and
-    dead segments, both unit widths), and the result is within the oracle's tolerance."""
+                                 (2, 12288), (5120, 8192), (77, 5120), (640, 11280),
+                                 # K in one unit, weights of 20..128 MB (units of 2, 3 and 4 segments)
+                                 (9728, 2560), (19456, 2560), (6001, 4096), (10300, 2064), (11000, 2048)])
+def test_gemv_w8a16_whole_row_kernel_gives_the_general_kernels_bits(orc, monkeypatch, n, k):
+    """One row against a K of two or three units, or against a mid-sized weight with K in one
+    unit, runs a wavefront per weight row; with CMI_GEMV_WHOLEROW=0 the library keeps the
+    general kernel.  Both follow the canonical summation order, so their outputs agree bit for
+    bit (ragged N, K with dead chunks and dead segments, every unit width), and the result is
+    within the oracle's tolerance."""
     g = seeded()
     q = synth.int8_weight(n, k, g)
     x = synth.activations(1, k, g)
