@@ -34,9 +34,10 @@ LAYERS = 32
 METRIC = "decode GEMV HBM GB/s (% of peak) + W8A8 prefill int8 TOPS, Qwen3.5-4B shapes"
 
 
-#: gemv_w8a16_kernel, default workload (M=1): fetched + written bytes per launch, from the
+#: gemv_w8a16_kernel and gemv_w8a16_wholerow_kernel (the two instantiation families the 129 launches
+#: of the default workload, M=1, use): fetched + written bytes per launch, from the
 #: FETCH_SIZE and WRITE_SIZE runs summarised in profiles/gemv_w8a16_decode_model_M1.md
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28.42e6
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28.51e6
 
 
 def parse_args():
@@ -248,7 +249,7 @@ def main() -> int:
             # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this same
             # command (summary under profiles/); it only describes the default workload
             "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if (M == 1 and not args.no_graph) else None,
-            "kernel": "gemv_w8a16_rows16_kernel" if args.mfma else "gemv_w8a16_kernel",
+            "kernel": "gemv_w8a16_rows16_kernel" if args.mfma else ("gemv_w8a16_kernel + gemv_w8a16_wholerow_kernel" if M == 1 else "gemv_w8a16_kernel"),
             "avg_launch_us": round(step_s / n_launch * 1e6, 3),
             "algorithmic_bytes_per_launch": round(bytes_per_step / n_launch),
         },
