@@ -380,10 +380,17 @@ extern "C" int cmi_gemv_w4a8_bf16(const uint8_t *w4, const float *ws, const void
     // 10-20 KiB per wavefront: 5120 -> 25600 42 us against 26); else the
     // decode kernel (whole rows requested up front) where it applies, else the general one
     int rc = CMI_E_UNSUPPORTED;
-    if (K > 4096)
+    // (one row of a weight whose grid is small enough that the wavefronts of a workgroup share
+    // rows is the exception since that kernel's walk over the groups was made branch-free:
+    // 9728 -> 2560 8.6 -> 8.25 us, 6144 -> 1024 5.9 -> 4.6 us)
+    const bool one_shared_row = M == 1 && (N + 15) / 16 < 256;
+    if (K > 4096 && !one_shared_row)
         rc = gemv_w4a8_rows16(w4, ws, nullptr, nullptr, x, y, group_acc, xq_out, xs_out, M, N, K, stream);
     if (rc != CMI_E_UNSUPPORTED) return rc;
     rc = gemv_w4a8_decode(w4, ws, x, nullptr, nullptr, y, group_acc, xq_out, xs_out, M, N, K, stream);
+    if (rc != CMI_E_UNSUPPORTED) return rc;
+    if (K > 4096 && one_shared_row)  // beyond the decode kernel's K
+        rc = gemv_w4a8_rows16(w4, ws, nullptr, nullptr, x, y, group_acc, xq_out, xs_out, M, N, K, stream);
     if (rc != CMI_E_UNSUPPORTED) return rc;
     return run_gemv_w4a8("cmi_gemv_w4a8_bf16", w4, ws, nullptr, nullptr, x, xq_out, xs_out, y, group_acc, M, N, K,
                          gs, stream);

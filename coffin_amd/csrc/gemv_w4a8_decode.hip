@@ -56,7 +56,7 @@ __host__ __device__ inline Lds lds_layout(int mt, int K, bool ksplit) {
     l.xsum = l.xq + mt * K;                           // int8 [mt][K]
     l.wsc = l.xsum + mt * (K / 32) * 4;               // int32 [mt][K/32]
     l.sums = l.wsc + ((rows * G * 4 + 15) & ~15);     // float [rows][G]
-    l.xs = l.sums + ((rows * G * mt * 4 + 15) & ~15); // int32 [rows/4][G][4][mt]
+    l.xs = l.sums + rows * ((G + 3) & ~3) * mt * 4;   // int32 [rows][mt][G padded to 4]
     l.part = l.xs + 16 * 4;                           // float [mt] (padded to 16)
     l.total = l.part + 16 * 4 * 4;                    // float [mt][4]
     return l;
@@ -191,7 +191,9 @@ gemv_w4a8_decode_kernel(const Args a) {
     __syncthreads();
 
     // 5. integer group sums
-    int32_t *wsums = sums + (KSPLIT ? 0 : wave * (a.G * ROWS_PER_WAVE * M));
+    // [row of the wavefront][m][group]: the lane that walks a row's groups reads them 16 bytes at a time
+    const int Gpad = (a.G + 3) & ~3;
+    int32_t *wsums = sums + (KSPLIT ? 0 : wave * (Gpad * ROWS_PER_WAVE * M));
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
         if ((KSPLIT ? j * 4 + wave : j) * 16 >= nchunks) break;  // uniform per wavefront
@@ -215,7 +217,7 @@ gemv_w4a8_decode_kernel(const Args a) {
             for (int i = 0; i < 8; ++i) acc = __builtin_amdgcn_sdot4((int)op[i], (int)xv[i], acc, false);
             acc += dpp_i32<0xB1, 0xf>(acc);
             acc += dpp_i32<0x4E, 0xf>(acc);
-            if ((lane & 3) == 0 && live) wsums[((c >> 2) * ROWS_PER_WAVE + r) * M + m] = acc;
+            if ((lane & 3) == 0 && live) wsums[(r * M + m) * Gpad + (c >> 2)] = acc;
         }
     }
     if constexpr (KSPLIT) {
@@ -227,35 +229,58 @@ gemv_w4a8_decode_kernel(const Args a) {
         __builtin_amdgcn_wave_barrier();
     }
 
-    // 6. fp32 chain over the groups, one lane per (row, m)
+    // 6. fp32 chain over the groups, one lane per (row, m).  The integer sums go out first, all
+    // lanes sharing the work, so that the chain itself is free of branches and stores.
+    if (a.group_acc) {
+        const int n_out = ROWS_PER_WAVE * M * a.G;
+        for (int i = lane; i < n_out; i += 64) {
+            const int rm = i / a.G, g = i - rm * a.G;
+            const int rr = rm / M, m = rm - rr * M;
+            const int n = n0 + (KSPLIT ? 0 : wave * ROWS_PER_WAVE) + rr;
+            if (n < a.N && m < a.M) a.group_acc[((size_t)m * a.G + g) * a.N + n] = wsums[rm * Gpad + g];
+        }
+    }
     if (lane < ROWS_PER_WAVE * M) {
         const int rr = lane / M, m = lane - rr * M;
         const int brow = (KSPLIT ? 0 : wave * ROWS_PER_WAVE) + rr;  // row within the workgroup
         const int n = n0 + brow;
         if (n < a.N && m < a.M) {
             const float *wsn = ws_lds + brow * a.G;
+            const int32_t *sn = wsums + (rr * M + m) * Gpad;
             float total = 0.f;
-            // four groups at a time: the eight LDS reads go out together, the fmas stay in order
             int g = 0;
-            for (; g + 4 <= a.G; g += 4) {
-                int sv[4];
-                float wv[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    sv[i] = wsums[((g + i) * ROWS_PER_WAVE + rr) * M + m];
-                    wv[i] = wsn[g + i];
+            if ((a.G & 3) == 0) {
+                // Eight groups per trip, read as 16-byte vectors with the next trip's reads in
+                // flight during this trip's chain (one convert and one fma per group, each fma
+                // waiting for the last).
+                const v4i32 *sv = reinterpret_cast<const v4i32 *>(sn);
+                const float4 *wv = reinterpret_cast<const float4 *>(wsn);
+                auto chain4 = [&](const v4i32 &sq, const float4 &wq) {
+                    total = fmaf((float)sq[0], wq.x, total);
+                    total = fmaf((float)sq[1], wq.y, total);
+                    total = fmaf((float)sq[2], wq.z, total);
+                    total = fmaf((float)sq[3], wq.w, total);
+                };
+                const int quads = a.G >> 2;
+                int q = 0;
+                if (quads >= 2) {
+                    v4i32 s0 = sv[0], s1 = sv[1];
+                    float4 w0 = wv[0], w1 = wv[1];
+                    for (; q + 4 <= quads; q += 2) {
+                        const v4i32 t0 = sv[q + 2], t1 = sv[q + 3];
+                        const float4 u0 = wv[q + 2], u1 = wv[q + 3];
+                        chain4(s0, w0);
+                        chain4(s1, w1);
+                        s0 = t0, s1 = t1, w0 = u0, w1 = u1;
+                    }
+                    chain4(s0, w0);
+                    chain4(s1, w1);
+                    q += 2;
                 }
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    if (a.group_acc) a.group_acc[((size_t)m * a.G + g + i) * a.N + n] = sv[i];
-                    total = fmaf((float)sv[i], wv[i], total);
-                }
+                if (q < quads) chain4(sv[q], wv[q]);
+                g = a.G;
             }
-            for (; g < a.G; ++g) {
-                const int sg = wsums[(g * ROWS_PER_WAVE + rr) * M + m];
-                if (a.group_acc) a.group_acc[((size_t)m * a.G + g) * a.N + n] = sg;
-                total = fmaf((float)sg, wsn[g], total);
-            }
+            for (; g < a.G; ++g) total = fmaf((float)sn[g], wsn[g], total);
             a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * xs_lds[m]);
         }
     }
