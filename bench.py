@@ -326,7 +326,7 @@ def main() -> int:
 
         # W8A8 prefill GEMM (GEMM kernel alone, and quantiser + GEMM)
         mm = {}
-        for m, n_ in ((2048, 9728), (2048, 4096), (512, 9728), (8192, 9728)):
+        for m, n_ in ((2048, 9728), (2048, 4096), (512, 9728), (512, 4096), (8192, 9728), (8192, 4096)):
             k_ = 2560
             q = synth.int8_weight(n_, k_, gen)
             x = synth.activations(m, k_, gen, outliers=True)
