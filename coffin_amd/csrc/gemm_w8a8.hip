@@ -765,9 +765,9 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
     hipStream_t st = static_cast<hipStream_t>(stream);
     // Tile choice: how full the last round of workgroups is (256 CUs; one large workgroup or
     // two 128 x 128 workgroups per CU) and how much of the tiles' area is real output, times
-    // the steady-state advantage of the larger tiles.  CMI_GEMM_TILE=128|256|320 overrides
+    // the steady-state advantage of the larger tiles.  CMI_GEMM_TILE=64|128|256|320 overrides
     // (tests, tuning).
-    int pick;  // 128, 256 or 320: block tile along n
+    int pick;  // 64, 128, 256 or 320: block tile along n
     if (force && force[0]) {
         pick = atoi(force);
     } else {
@@ -783,12 +783,21 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
         pick = e128 >= e256 && e128 >= e320 ? 128 : e256 >= e320 ? 256 : 320;
     }
     if (pick == 320) return launch_wide(a, st);
+    // 128 x 128 tiles that would leave half of the CUs idle: 128(m) x 64(n) tiles of the same kernel
+    // instead, twice as many workgroups with half the MFMAs per dependent step each (512 x 4096 x 2560
+    // 16.8 -> 12.7 us, 512 x 2560 x 9728 47 -> 34 us; with more tiles than that it measured 10-30 % slower).
+    const int tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+    if (pick == 128 && !(force && force[0]) && tiles128 <= 128 && N > 64) pick = 64;
+    if (pick == 64) {
+        const int tiles64 = ((M + 127) / 128) * ((N + 63) / 64);
+        if (tiles64 <= 256) return launch<1, 2, 3>(a, st);
+        return launch<1, 2, 2>(a, st);
+    }
     const bool use_big = pick == 256;
     if (use_big) return launch_big(a, st);
     // Up to one 128 x 128 workgroup per CU the launch is a chain of K/128 dependent steps: a third
     // LDS stage (96 KiB, one workgroup per CU anyway) puts two steps of loads in flight (-20 % at
     // K = 2560, -33 % at K = 9728); with two workgroups per CU it measured slower.
-    const int tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
     if (tiles128 <= 256) return launch<2, 2, 3>(a, st);
     return launch<2, 2, 2>(a, st);
 }

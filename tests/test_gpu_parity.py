@@ -282,9 +282,9 @@ def test_sixteen_row_kernels_at_lm_head_size_sampled_columns(orc):
 
 # ------------------------------------------------------------------ W8A8 GEMM
 
-@pytest.fixture(params=["auto", "128", "256", "320"])
+@pytest.fixture(params=["auto", "64", "128", "256", "320"])
 def gemm_tile(request, monkeypatch):
-    """Force the 128 x 128, 256 x 256 or 256 x 320 block-tile kernel (the library reads
+    """Force the 128 x 64, 128 x 128, 256 x 256 or 256 x 320 block-tile kernel (the library reads
     CMI_GEMM_TILE on every call), or leave the choice to the library."""
     if request.param != "auto":
         monkeypatch.setenv("CMI_GEMM_TILE", request.param)
