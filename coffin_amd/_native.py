@@ -14,14 +14,15 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libcoffin_mi355.so"
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 OK, E_ARG, E_UNSUPPORTED, E_HIP = 0, 1, 2, 3
 
-_vp, _ci = ctypes.c_void_p, ctypes.c_int
+_vp, _ci, _cs = ctypes.c_void_p, ctypes.c_int, ctypes.c_char_p
 
 #: name -> argtypes, exactly the declarations of include/coffin_mi355.h.
 SIGNATURES: dict[str, list] = {
+    "cmi_set_option": [_cs, _ci],
     "cmi_quant_act_i8": [_vp, _vp, _vp, _ci, _ci, _vp],
     "cmi_gemv_w8a16": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp],
     "cmi_gemv_w8a16_mfma": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp],

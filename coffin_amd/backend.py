@@ -34,9 +34,9 @@ re-layout is a private copy made once per weight).
 
 from __future__ import annotations
 
-import ctypes
 import os
 import weakref
+from collections import OrderedDict
 
 import torch
 import torch.nn.functional as F
@@ -140,7 +140,7 @@ def _on_gpu(t: torch.Tensor) -> bool:
 
 #: (rows, k, device) -> (xq int8 [rows,k], xs fp32 [rows]); single-threaded caller
 #: by contract (backends/corex/__init__.py:654-690 keeps the same kind of pool).
-_SCRATCH: dict = {}
+_SCRATCH: OrderedDict = OrderedDict()
 _SCRATCH_MAX = 32
 
 
@@ -148,11 +148,13 @@ def _scratch(rows: int, k: int, device: torch.device):
     key = (rows, k, device)
     hit = _SCRATCH.get(key)
     if hit is None:
-        if len(_SCRATCH) >= _SCRATCH_MAX:
-            _SCRATCH.clear()
+        while len(_SCRATCH) >= _SCRATCH_MAX:
+            _SCRATCH.popitem(last=False)          # least recently used shape goes first
         hit = (torch.empty((rows, k), dtype=torch.int8, device=device),
                torch.empty(rows, dtype=torch.float32, device=device))
         _SCRATCH[key] = hit
+    else:
+        _SCRATCH.move_to_end(key)
     return hit
 
 
@@ -186,9 +188,48 @@ def _q8_operands(w):
     return wq, scale
 
 
+def _w4_check(w) -> None:
+    """Refuse a W4A8Weight-like whose buffers are not what the re-layout kernel reads.
+
+    The adapter accepts any object with ``packed`` / ``scale`` / ``k`` / ``n`` / ``group_size``;
+    the kernel reads ``K/2 * N`` bytes and ``K/gs * N`` floats from raw addresses, so dtype,
+    contiguity, device and shape are checked here (the reference's own class checks the same in
+    its constructor, w4a8_weights.py:35-44).
+    """
+    n, k, gs = int(w.n), int(w.k), int(w.group_size)
+    packed, scale = w.packed, w.scale
+    if packed.dtype != torch.uint8 or packed.dim() != 2 or not packed.is_contiguous():
+        raise ValueError(f"int4 weight: packed must be contiguous 2-D uint8, got "
+                         f"{tuple(packed.shape)} {packed.dtype}")
+    if packed.shape[1] != n or packed.shape[0] * 2 < k:
+        raise ValueError(f"int4 weight: packed {tuple(packed.shape)} does not hold K={k} x N={n} codes")
+    if scale.dtype != torch.float32 or scale.dim() != 2 or not scale.is_contiguous():
+        raise ValueError(f"int4 weight: scale must be contiguous 2-D fp32, got "
+                         f"{tuple(scale.shape)} {scale.dtype}")
+    if tuple(scale.shape) != (-(-k // gs), n):
+        raise ValueError(f"int4 weight: scale {tuple(scale.shape)} does not match "
+                         f"[{-(-k // gs)}, {n}] (K={k}, group size {gs})")
+    if packed.device.type != "cuda" or scale.device != packed.device:
+        raise ValueError(f"int4 weight: packed on {packed.device} and scale on {scale.device} "
+                         f"must share a GPU")
+
+
+def _kernels_take(w) -> bool:
+    """Whether the native kernels are built for this quantized weight's shape.
+
+    int4: group size 128 and K a multiple of 128; int8: K a multiple of 16.  Other shapes are
+    answered by the torch statement of the op (the reference's corex adapter likewise falls back
+    for group sizes its GEMM does not take, backends/corex/__init__.py:633).
+    """
+    if _is_w4(w):
+        return int(w.group_size) == 128 and int(w.k) % 128 == 0
+    return int(w.wq.shape[-1]) % 16 == 0
+
+
 def _w4_operands(w):
     """Device layout ``(w4 uint8 [N,K/2], ws fp32 [N,G])`` of a W4A8Weight-like, built once."""
     def make():
+        _w4_check(w)
         n, k, gs = int(w.n), int(w.k), int(w.group_size)
         w4 = torch.empty((n, k // 2), dtype=torch.uint8, device=w.packed.device)
         ws = torch.empty((n, k // gs), dtype=torch.float32, device=w.packed.device)
@@ -217,17 +258,19 @@ class _Record:
 
 #: id(weight object) -> _Record; an entry is trusted only while the tensors it was
 #: built from are still the ones the weight object holds.
-_RECORDS: dict = {}
+_RECORDS: OrderedDict = OrderedDict()
 _RECORDS_MAX = 8192
 
 
 def _lookup(w) -> _Record | None:
-    rec = _RECORDS.get(id(w))
+    key = id(w)
+    rec = _RECORDS.get(key)
     if rec is None:
         return None
     try:
         first = w.wq if rec.kind == 8 else w.packed
         if rec.src() is first and rec.src2() is w.scale:
+            _RECORDS.move_to_end(key)
             return rec
     except AttributeError:
         pass
@@ -245,8 +288,9 @@ def _make_record(w) -> _Record:
         rec.kind, rec.src, rec.a, rec.b = 8, weakref.ref(w.wq), wq.data_ptr(), scale.data_ptr()
         rec.n, rec.k, rec.gs, rec.dev = int(wq.shape[0]), int(wq.shape[1]), 0, w.wq.device
     rec.src2 = weakref.ref(w.scale)
-    if len(_RECORDS) >= _RECORDS_MAX:
-        _RECORDS.clear()
+    _RECORDS.pop(id(w), None)                     # a stale entry under a reused id
+    while len(_RECORDS) >= _RECORDS_MAX:
+        _RECORDS.popitem(last=False)              # least recently used weight goes first
     _RECORDS[id(w)] = rec
     return rec
 
@@ -327,7 +371,7 @@ def _project(w, x: torch.Tensor, prefill: bool, min_rows: int = PREFILL_MIN_ROWS
         # path for quantized weights: refuse instead of answering slowly.
         raise ValueError("coffin_amd: quantized weights need activations on the GPU, "
                          f"got {x.device}")
-    if x.dtype != torch.bfloat16:
+    if x.dtype != torch.bfloat16 or (rec is None and not _kernels_take(w)):
         return _dense(w, x)
     k = rec.k if rec is not None else int(w.k)
     nd = x.dim()

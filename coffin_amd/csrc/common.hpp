@@ -18,6 +18,10 @@ int check_launch(const char *what);
 // (`devices`: one bit per device ordinal, owned by the call site).  CMI_OK or CMI_E_HIP.
 int reserve_lds(const void *kernel, int bytes, std::atomic<uint64_t> &devices, const char *who);
 
+// Kernel-selection overrides (cmi_set_option / CMI_GEMM_TILE, CMI_GEMV_WHOLEROW read once).
+int option_gemm_tile();      // 0 = the library chooses, else 64 / 128 / 256 / 320
+int option_gemv_wholerow();  // -1 = the library chooses, 0 = never, 1 = where it can
+
 #define CMI_REQUIRE(cond, code, ...)                 \
     do {                                             \
         if (!(cond)) return cmi::fail(code, __VA_ARGS__); \

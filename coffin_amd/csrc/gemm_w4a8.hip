@@ -307,8 +307,7 @@ extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     // Few rows: the tile pipeline is latency-bound (K/128 steps of ~1.2 us whatever M is), while the
     // matrix-pipe GEMV reads the weight once per 16 rows at memory speed; same integer sums, same
     // fp32 chain, same bits.  Cost model fitted to measurements on the layer shapes (us).
-    const char *force = getenv("CMI_GEMM_TILE");
-    if (M <= 256 && !(force && force[0])) {
+    if (M <= 256 && !option_gemm_tile()) {
         const double steps = K / 128.0, wn = (double)N * K;
         const double tiles = (double)a_ceil(M, BM) * a_ceil(N, BN);
         const double t_tiled = 3.0 + steps * (tiles <= 512 ? 1.15 + 0.0013 * tiles : 1.8 * ceil(tiles / 512.0));

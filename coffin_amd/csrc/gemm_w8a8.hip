@@ -723,13 +723,13 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
     CMI_REQUIRE(K % 16 == 0, CMI_E_UNSUPPORTED, "cmi_gemm_w8a8: K=%d is not a multiple of 16", K);
     CMI_REQUIRE(aligned(xq, 16) && aligned(wq, 16), CMI_E_ARG,
                 "cmi_gemm_w8a8: xq and wq must be 16-byte aligned");
-    const char *force = getenv("CMI_GEMM_TILE");
-    if (M <= 16 && !(force && force[0])) {
+    const int force = option_gemm_tile();
+    if (M <= 16 && !force) {
         // a verify-sized batch: read the weight once, GEMV style
         const int rc = gemm_w8a8_rows16(xq, wq, xs, ws, y, acc_out, M, N, K, ldy, stream);
         if (rc != CMI_E_UNSUPPORTED) return rc;
     }
-    if (M > 16 && M <= 256 && K % 128 == 0 && K <= 10240 && !(force && force[0])) {
+    if (M > 16 && M <= 256 && K % 128 == 0 && K <= 10240 && !force) {
         // Few rows: the tile pipeline is latency-bound (K/128 dependent steps of 0.45-1.4 us, growing
         // with the number of tiles that share the chip, whatever M is); the read-once kernel asks
         // for the weight once per 128 rows and pays per 16-row chunk only the chunk's trip through
@@ -768,8 +768,8 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
     // the steady-state advantage of the larger tiles.  CMI_GEMM_TILE=64|128|256|320 overrides
     // (tests, tuning).
     int pick;  // 64, 128, 256 or 320: block tile along n
-    if (force && force[0]) {
-        pick = atoi(force);
+    if (force) {
+        pick = force;
     } else {
         auto fill = [](double tiles, double slots) { return tiles / (ceil(tiles / slots) * slots); };
         const double t128 = (double)((M + 127) / 128) * ((N + 127) / 128);
@@ -787,7 +787,7 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
     // instead, twice as many workgroups with half the MFMAs per dependent step each (512 x 4096 x 2560
     // 16.8 -> 12.7 us, 512 x 2560 x 9728 47 -> 34 us; with more tiles than that it measured 10-30 % slower).
     const int tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
-    if (pick == 128 && !(force && force[0]) && tiles128 <= 128 && N > 64) pick = 64;
+    if (pick == 128 && !force && tiles128 <= 128 && N > 64) pick = 64;
     if (pick == 64) {
         const int tiles64 = ((M + 127) / 128) * ((N + 63) / 64);
         if (tiles64 <= 256) return launch<1, 2, 3>(a, st);

@@ -683,8 +683,7 @@ extern "C" int cmi_gemv_w8a16(const int8_t *wq, const float *ws, const void *x, 
     // wavefront per weight row.  CMI_GEMV_WHOLEROW=0 keeps the general kernel (the tests compare
     // the two bit for bit).
     if (M == 1 && p.mode != 2) {
-        const char *e = getenv("CMI_GEMV_WHOLEROW");
-        if (!(e && e[0] == '0')) {
+        if (option_gemv_wholerow() != 0) {
             const int rc = dispatch_wholerow(a, st);
             if (rc != CMI_E_UNSUPPORTED) return rc;
         }

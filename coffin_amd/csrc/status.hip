@@ -3,6 +3,8 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
+#include <cstring>
 
 namespace {
 thread_local char g_error[512] = "";
@@ -42,8 +44,69 @@ int reserve_lds(const void *kernel, int bytes, std::atomic<uint64_t> &devices, c
     return CMI_OK;
 }
 
+// ------------------------------------------------------------------ options
+// Kernel-selection overrides for tests and tuning.  Each is read from its environment variable
+// once, when first asked for, and validated there; afterwards only cmi_set_option changes it, so
+// the hot path costs one relaxed atomic load per call and never calls getenv.
+namespace {
+constexpr int UNREAD = INT32_MIN;
+std::atomic<int> g_gemm_tile{UNREAD};      // 0 = the library chooses
+std::atomic<int> g_gemv_wholerow{UNREAD};  // -1 = the library chooses, 0 = never, 1 = where it can
+
+bool valid_gemm_tile(int v) { return v == 0 || v == 64 || v == 128 || v == 256 || v == 320; }
+bool valid_wholerow(int v) { return v >= -1 && v <= 1; }
+
+int from_env(const char *name, int fallback, bool (*valid)(int)) {
+    const char *e = getenv(name);
+    if (!e || !e[0]) return fallback;
+    char *end = nullptr;
+    const long v = strtol(e, &end, 10);
+    if (end == e || *end != '\0' || !valid((int)v)) {
+        fprintf(stderr, "coffin_mi355: ignoring %s=%s (not a value this library knows)\n", name, e);
+        return fallback;
+    }
+    return (int)v;
+}
+}  // namespace
+
+int option_gemm_tile() {
+    int v = g_gemm_tile.load(std::memory_order_relaxed);
+    if (v == UNREAD) {
+        v = from_env("CMI_GEMM_TILE", 0, valid_gemm_tile);
+        g_gemm_tile.store(v, std::memory_order_relaxed);
+    }
+    return v;
+}
+
+int option_gemv_wholerow() {
+    int v = g_gemv_wholerow.load(std::memory_order_relaxed);
+    if (v == UNREAD) {
+        v = from_env("CMI_GEMV_WHOLEROW", -1, valid_wholerow);
+        g_gemv_wholerow.store(v, std::memory_order_relaxed);
+    }
+    return v;
+}
+
 }  // namespace cmi
 
-extern "C" int cmi_abi_version(void) { return 1; }
+extern "C" int cmi_set_option(const char *name, int value) {
+    using namespace cmi;
+    CMI_REQUIRE(name, CMI_E_ARG, "cmi_set_option: null name");
+    if (!strcmp(name, "gemm_tile")) {
+        CMI_REQUIRE(valid_gemm_tile(value), CMI_E_ARG,
+                    "cmi_set_option: gemm_tile=%d, expected 0 (library's choice), 64, 128, 256 or 320", value);
+        g_gemm_tile.store(value, std::memory_order_relaxed);
+        return CMI_OK;
+    }
+    if (!strcmp(name, "gemv_wholerow")) {
+        CMI_REQUIRE(valid_wholerow(value), CMI_E_ARG,
+                    "cmi_set_option: gemv_wholerow=%d, expected -1 (library's choice), 0 or 1", value);
+        g_gemv_wholerow.store(value, std::memory_order_relaxed);
+        return CMI_OK;
+    }
+    return fail(CMI_E_ARG, "cmi_set_option: unknown option '%s'", name);
+}
+
+extern "C" int cmi_abi_version(void) { return 2; }
 
 extern "C" const char *cmi_last_error(void) { return g_error; }

@@ -51,10 +51,12 @@ SPEC = VendorSpec(
     name="mi355x",
     detection=Detection(
         namespace="cuda",
-        # Boards report "AMD Instinct MI355X"; hosts without the amdgpu id table
-        # report the generic "AMD Radeon Graphics", which build_ops() narrows
-        # down to gfx950 by the ISA name before handing out any kernel.
-        name_markers=("mi355", "mi350", "amd radeon graphics"),
+        # Boards report "AMD Instinct MI355X".  A host without the amdgpu id table
+        # reports the generic "AMD Radeon Graphics" for every AMD part; claiming
+        # that name would take non-gfx950 devices away from the backend written
+        # for them, so such hosts select this backend by name
+        # (COFFIN_BACKEND=mi355x).  build_ops() checks the ISA either way.
+        name_markers=("mi355", "mi350"),
         hip=True,
     ),
     act_dtype=torch.bfloat16,

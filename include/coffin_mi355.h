@@ -35,6 +35,16 @@ extern "C" {
 /* ABI version; bumped when a signature changes. */
 int cmi_abi_version(void);
 
+/* Kernel-selection override for tests and tuning; no counterpart in the reference.
+ *   "gemm_tile"     0 (the library chooses) | 64 | 128 | 256 | 320: block tile of cmi_gemm_w8a8 /
+ *                   cmi_gemm_w4a8 (non-zero also bypasses their few-row routes);
+ *   "gemv_wholerow" -1 (the library chooses) | 0 (never) | 1: the one-wavefront-per-weight-row
+ *                   kernel of cmi_gemv_w8a16.
+ * The environment variables CMI_GEMM_TILE and CMI_GEMV_WHOLEROW give the initial values; they are
+ * read once, at the first call that needs them.  Unknown names or values: CMI_E_ARG.  Every choice
+ * gives the same bits. */
+int cmi_set_option(const char *name, int value);
+
 /* Message for the last non-zero status returned on this thread ("" if none). */
 const char *cmi_last_error(void);
 

@@ -29,6 +29,17 @@ def pytest_collection_modifyitems(config, items):
             item.add_marker(skip)
 
 
+@pytest.fixture(autouse=True)
+def _library_options_back_to_default(request):
+    """Tests force kernels through cmi_set_option; none of that may leak into the next test."""
+    yield
+    if "gpu" in request.keywords:
+        from coffin_amd import _native
+        lib = _native.load()
+        lib.cmi_set_option(b"gemm_tile", 0)
+        lib.cmi_set_option(b"gemv_wholerow", -1)
+
+
 @pytest.fixture(scope="session")
 def golden():
     def load(name: str):

@@ -20,6 +20,11 @@ def stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
+def set_option(name: str, value: int) -> None:
+    """Kernel-selection override of the library (cmi_set_option): gemm_tile, gemv_wholerow."""
+    _native.check(_native.load().cmi_set_option(name.encode(), int(value)), "set_option")
+
+
 def dev(a: np.ndarray) -> torch.Tensor:
     return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
 

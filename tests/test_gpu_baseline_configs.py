@@ -27,11 +27,11 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.fixture(params=["auto", "64", "128", "256", "320"])
-def gemm_tile(request, monkeypatch):
+def gemm_tile(request):
     if request.param != "auto":
-        monkeypatch.setenv("CMI_GEMM_TILE", request.param)
+        G.set_option("gemm_tile", int(request.param))
     else:
-        monkeypatch.delenv("CMI_GEMM_TILE", raising=False)
+        G.set_option("gemm_tile", 0)
     return request.param
 
 

@@ -128,9 +128,9 @@ def test_gemv_w8a16_within_tolerance(orc, m, n, k):
                                  (2, 12288), (5120, 8192), (77, 5120), (640, 11280),
                                  # K in one unit, weights of 20..128 MB (units of 2, 3 and 4 segments)
                                  (9728, 2560), (19456, 2560), (6001, 4096), (10300, 2064), (11000, 2048)])
-def test_gemv_w8a16_whole_row_kernel_gives_the_general_kernels_bits(orc, monkeypatch, n, k):
+def test_gemv_w8a16_whole_row_kernel_gives_the_general_kernels_bits(orc, n, k):
     """One row against a K of two or three units, or against a mid-sized weight with K in one
-    unit, runs a wavefront per weight row; with CMI_GEMV_WHOLEROW=0 the library keeps the
+    unit, runs a wavefront per weight row; with the option gemv_wholerow = 0 the library keeps the
     general kernel.  Both follow the canonical summation order, so their outputs agree bit for
     bit (ragged N, K with dead chunks and dead segments, every unit width), and the result is
     within the oracle's tolerance."""
@@ -138,9 +138,9 @@ def test_gemv_w8a16_whole_row_kernel_gives_the_general_kernels_bits(orc, monkeyp
     q = synth.int8_weight(n, k, g)
     x = synth.activations(1, k, g)
     args = (q.wq.to(G.DEV), q.scale.to(G.DEV), x.to(G.DEV))
-    monkeypatch.delenv("CMI_GEMV_WHOLEROW", raising=False)
+    G.set_option("gemv_wholerow", -1)
     y = G.gemv_w8a16(*args)
-    monkeypatch.setenv("CMI_GEMV_WHOLEROW", "0")
+    G.set_option("gemv_wholerow", 0)
     y_team = G.gemv_w8a16(*args)
     assert (y.view(torch.int16) == y_team.view(torch.int16)).all()
     _assert_weight_only_tolerance(orc, q.wq.numpy(), q.scale.numpy(), x, y)
@@ -283,13 +283,13 @@ def test_sixteen_row_kernels_at_lm_head_size_sampled_columns(orc):
 # ------------------------------------------------------------------ W8A8 GEMM
 
 @pytest.fixture(params=["auto", "64", "128", "256", "320"])
-def gemm_tile(request, monkeypatch):
-    """Force the 128 x 64, 128 x 128, 256 x 256 or 256 x 320 block-tile kernel (the library reads
-    CMI_GEMM_TILE on every call), or leave the choice to the library."""
+def gemm_tile(request):
+    """Force the 128 x 64, 128 x 128, 256 x 256 or 256 x 320 block-tile kernel through
+    cmi_set_option, or leave the choice to the library (conftest resets it after each test)."""
     if request.param != "auto":
-        monkeypatch.setenv("CMI_GEMM_TILE", request.param)
+        G.set_option("gemm_tile", int(request.param))
     else:
-        monkeypatch.delenv("CMI_GEMM_TILE", raising=False)
+        G.set_option("gemm_tile", 0)
     return request.param
 
 
@@ -316,10 +316,10 @@ def test_gemm_w8a8_bit_exact(orc, gemm_tile, m, n, k):
                                    # such launches): every lines-per-wavefront variant, ragged N and M
                                    (17, 100, 9728), (48, 2560, 2560), (128, 333, 4096), (100, 77, 1024),
                                    (33, 40, 10240), (200, 64, 9728), (64, 1200, 5120)])
-def test_gemm_w8a8_verify_batches_bit_exact(orc, monkeypatch, m, n, k):
+def test_gemm_w8a8_verify_batches_bit_exact(orc, m, n, k):
     """Few rows take the read-the-weight-once kernels: exact against the oracle, and the
     same bits as the tiled kernel gives for the same rows (also with a row stride)."""
-    monkeypatch.delenv("CMI_GEMM_TILE", raising=False)
+    G.set_option("gemm_tile", 0)
     g = seeded()
     q = synth.int8_weight(n, k, g)
     x = synth.activations(m, k, g, outliers=True)
@@ -331,7 +331,7 @@ def test_gemm_w8a8_verify_batches_bit_exact(orc, monkeypatch, m, n, k):
     assert (G.bits(y) == y_ref).all()
     _, wide = G.gemm_w8a8(*args, want_acc=False, ldy=n + 8)
     assert (G.bits(wide[:, :n]) == y_ref).all() and (wide[:, n:].float() == 0).all()
-    monkeypatch.setenv("CMI_GEMM_TILE", "128")
+    G.set_option("gemm_tile", 128)
     _, tiled = G.gemm_w8a8(*args, want_acc=False)
     assert (tiled.view(torch.int16) == y.view(torch.int16)).all()
 
@@ -369,7 +369,7 @@ def test_gemm_w8a8_full_size_sampled_and_blockwise(orc, gemm_tile, m, n):
 
 
 @pytest.mark.parametrize("n,k", [(9728, 2560), (2560, 9728), (6144, 2560)])
-def test_gemm_w8a8_full_size_mid_batches_equal_the_tile_pipeline(n, k, monkeypatch):
+def test_gemm_w8a8_full_size_mid_batches_equal_the_tile_pipeline(n, k):
     """17..256 rows at the layer shapes: whatever route the entry picks (weight kept in
     registers for up to 128 rows per launch, or tiles) gives the bits of the tile pipeline,
     and a row does not depend on the batch it came in."""
@@ -377,9 +377,9 @@ def test_gemm_w8a8_full_size_mid_batches_equal_the_tile_pipeline(n, k, monkeypat
     q = synth.int8_weight(n, k, g)
     x = synth.activations(256, k, g, outliers=True)
     xq, xs = G.quant(x)
-    monkeypatch.setenv("CMI_GEMM_TILE", "128")
+    G.set_option("gemm_tile", 128)
     acc_t, y_t = G.gemm_w8a8(xq, q.wq, xs, q.scale)
-    monkeypatch.delenv("CMI_GEMM_TILE")
+    G.set_option("gemm_tile", 0)
     for m in (17, 48, 128, 129, 200, 256):
         acc, y = G.gemm_w8a8(xq[:m].contiguous(), q.wq, xs[:m].contiguous(), q.scale)
         assert (acc == acc_t[:m]).all(), m
@@ -490,7 +490,7 @@ def test_w4_repack_is_a_permutation_of_the_codes():
 
 
 @pytest.mark.parametrize("n,k", [(9728, 2560), (2560, 9728), (5120, 25600)])
-def test_w4a8_full_size_gemv_equals_gemm_rows(n, k, monkeypatch):
+def test_w4a8_full_size_gemv_equals_gemm_rows(n, k):
     """At benchmark sizes the GEMV and the MFMA GEMM must agree bit for bit (the
     arithmetic is the same by definition), and a batched GEMV row must equal the
     single-row call."""
@@ -501,9 +501,9 @@ def test_w4a8_full_size_gemv_equals_gemm_rows(n, k, monkeypatch):
     xq, xs = G.quant(x)
     # the tile pipeline itself (at 64 rows the entry would otherwise pick the read-once kernel),
     # then the entry's own choice: same bits
-    monkeypatch.setenv("CMI_GEMM_TILE", "128")
+    G.set_option("gemm_tile", 128)
     ga_mm, y_mm = G.w4a8(w4, ws, xq, xs, k, gemm=True)
-    monkeypatch.delenv("CMI_GEMM_TILE")
+    G.set_option("gemm_tile", 0)
     ga_auto, y_auto = G.w4a8(w4, ws, xq, xs, k, gemm=True)
     assert (ga_auto == ga_mm).all() and (y_auto.view(torch.int16) == y_mm.view(torch.int16)).all()
     ga_mv, y_mv = G.w4a8(w4, ws, xq[:16].contiguous(), xs[:16].contiguous(), k, gemm=False)

@@ -71,8 +71,8 @@ def test_gemv_w8a16_vocabulary_rows_sampled(orc):
 
 @pytest.mark.parametrize("m,n,k", [(16, 12352, 2560), (96, 2560, 9216), (16, 2560, 9216), (384, 1544, 9216),
                                    (300, 12352, 512)])
-def test_gemm_w8a8_reference_shapes_bit_exact(orc, monkeypatch, m, n, k):
-    monkeypatch.delenv("CMI_GEMM_TILE", raising=False)
+def test_gemm_w8a8_reference_shapes_bit_exact(orc, m, n, k):
+    G.set_option("gemm_tile", 0)
     g = seeded()
     q = synth.int8_weight(n, k, g)
     x = synth.activations(m, k, g, outliers=True)

@@ -250,6 +250,55 @@ def test_adapter_answers_dense_and_refuses_cpu_quantized():
     assert set(backend.native_table()) == set(contract.Ops.NAMES)
 
 
+def test_w4_operands_are_checked_before_any_address_reaches_a_kernel():
+    """A duck-typed int4 weight hands raw addresses to the re-layout kernel; dtype, contiguity
+    and shape must be refused on the host (the device check comes last and fails here too)."""
+    from types import SimpleNamespace as NS
+    k, n, gs = 256, 8, 128
+    good = dict(packed=torch.zeros((k // 2, n), dtype=torch.uint8), scale=torch.ones((k // gs, n)),
+                k=k, n=n, group_size=gs)
+    for patch, match in (
+            (dict(packed=torch.zeros((k // 2, n), dtype=torch.int8)), "uint8"),
+            (dict(packed=torch.zeros((n, k // 2), dtype=torch.uint8).t()), "contiguous"),
+            (dict(packed=torch.zeros((k // 2 - 1, n), dtype=torch.uint8)), "does not hold"),
+            (dict(packed=torch.zeros((k // 2, n + 1), dtype=torch.uint8)), "does not hold"),
+            (dict(scale=torch.ones((k // gs, n), dtype=torch.float16)), "fp32"),
+            (dict(scale=torch.ones((n, k // gs)).t()), "contiguous"),
+            (dict(scale=torch.ones((k // gs + 1, n))), "does not match"),
+            (dict(), "GPU")):
+        with pytest.raises(ValueError, match=match):
+            backend._w4_check(NS(**{**good, **patch}))
+    # shapes the kernels are not built for are answered by the torch statement of the op
+    assert backend._kernels_take(NS(**good))
+    assert not backend._kernels_take(NS(**{**good, "group_size": 64}))
+    assert not backend._kernels_take(NS(**{**good, "k": 192}))
+    assert backend._kernels_take(NS(wq=torch.zeros((4, 32), dtype=torch.int8), scale=torch.ones(4)))
+    assert not backend._kernels_take(NS(wq=torch.zeros((4, 24), dtype=torch.int8), scale=torch.ones(4)))
+
+
+def test_scratch_and_record_pools_evict_the_least_recently_used_entry(monkeypatch):
+    monkeypatch.setattr(backend, "_SCRATCH_MAX", 3)
+    backend._SCRATCH.clear()
+    cpu = torch.device("cpu")
+    a = backend._scratch(1, 16, cpu)
+    backend._scratch(2, 16, cpu)
+    backend._scratch(3, 16, cpu)
+    assert backend._scratch(1, 16, cpu) is a               # refreshed: now the most recent
+    backend._scratch(4, 16, cpu)                           # evicts (2, 16), the oldest
+    assert list(k[0] for k in backend._SCRATCH) == [3, 1, 4]
+    backend._SCRATCH.clear()
+    monkeypatch.setattr(backend, "_RECORDS_MAX", 2)
+    backend._RECORDS.clear()
+    g = synth.generator()
+    ws = [synth.int8_weight(4, 32, g) for _ in range(3)]
+    backend._make_record(ws[0])
+    backend._make_record(ws[1])
+    assert backend._lookup(ws[0]) is not None              # refreshed
+    backend._make_record(ws[2])                            # evicts ws[1]
+    assert backend._lookup(ws[1]) is None and backend._lookup(ws[0]) is not None
+    backend._RECORDS.clear()
+
+
 def test_weight_records_are_cached_weakly_and_revalidated():
     """The adapters resolve a weight's operand addresses once; the cached record must stop
     being trusted when the weight object swaps a tensor, and must not keep weights alive."""
@@ -293,11 +342,24 @@ def _declared_symbols() -> list[str]:
 def test_library_exports_every_declared_symbol():
     lib = _native.load()
     names = _declared_symbols()
-    assert len(names) == 10
     for name in names:
         assert getattr(lib, name) is not None
     assert set(_native.SIGNATURES) | {"cmi_abi_version", "cmi_last_error"} == set(names)
     assert lib.cmi_abi_version() == _native.ABI_VERSION
+
+
+def test_set_option_validates_names_and_values():
+    lib = _native.load()
+    for name, good, bad in ((b"gemm_tile", (64, 128, 256, 320, 0), (1, 100, -1)),
+                            (b"gemv_wholerow", (0, 1, -1), (2, -2))):
+        for v in bad:
+            assert lib.cmi_set_option(name, v) == _native.E_ARG
+            assert "expected" in _native.last_error()
+        for v in good:
+            assert lib.cmi_set_option(name, v) == _native.OK
+    assert lib.cmi_set_option(b"no_such_option", 0) == _native.E_ARG
+    assert "unknown option" in _native.last_error()
+    assert lib.cmi_set_option(None, 0) == _native.E_ARG
 
 
 def test_entry_points_reject_bad_arguments_before_touching_the_device():
