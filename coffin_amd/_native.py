@@ -19,6 +19,7 @@ ABI_VERSION = 2
 OK, E_ARG, E_UNSUPPORTED, E_HIP = 0, 1, 2, 3
 
 _vp, _ci, _cs = ctypes.c_void_p, ctypes.c_int, ctypes.c_char_p
+_i64, _sz, _f32 = ctypes.c_int64, ctypes.c_size_t, ctypes.c_float
 
 #: name -> argtypes, exactly the declarations of include/coffin_mi355.h.
 SIGNATURES: dict[str, list] = {
@@ -31,7 +32,17 @@ SIGNATURES: dict[str, list] = {
     "cmi_gemv_w4a8_bf16": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cmi_gemm_w8a8": [_vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cmi_gemm_w4a8": [_vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
+    "cmi_linear_w8a8_bf16": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp, _sz, _vp],
+    "cmi_linear_w4a8_bf16": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp, _sz, _vp],
+    "cmi_silu_mul_quant": [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _i64, _i64, _i64, _vp],
+    "cmi_rms_norm_i8": [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _i64, _i64, _f32, _vp],
+    "cmi_add_rms_norm_i8": [_vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _i64, _i64, _i64, _f32, _vp],
+    "cmi_embed_rows_i8": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp],
+    "cmi_embed_rows_w4": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
 }
+
+#: Entry points that do not return a status.
+OTHER_RESTYPES = {"cmi_linear_workspace_bytes": ([_ci, _ci], _sz)}
 
 
 class NativeError(RuntimeError):
@@ -71,6 +82,10 @@ def load() -> ctypes.CDLL:
             fn = getattr(lib, name)
             fn.argtypes = argtypes
             fn.restype = _ci
+        for name, (argtypes, restype) in OTHER_RESTYPES.items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = restype
     except (OSError, AttributeError) as exc:
         # Memoised: a failed load is reported the same way on every call instead
         # of being retried on the decode path.

@@ -75,27 +75,6 @@ W8A8_VERIFY = os.environ.get("COFFIN_AMD_W8A8_VERIFY", "0").strip() == "1"
 BATCH_MFMA = os.environ.get("COFFIN_AMD_BATCH_MFMA", "0").strip() == "1"
 #: Rows from which the matrix-pipe GEMV beats the dot-product one (measured on every layer shape).
 MFMA_MIN_ROWS = 3
-#: W4A8 switches from the GEMV to the MFMA GEMM above this many rows.
-W4_GEMM_MIN_ROWS = 17
-#: Up to this many rows the W4A8 GEMV quantises its activations itself (one launch); the
-#: kernel takes up to 4, but from 2 rows on every workgroup redoing the quantisation costs more
-#: than the separate quantiser launch -- except on long rows (K > 5120), where two rows still
-#: win (10.8 us against 12.7 us at 9728 -> 2560).
-W4_FUSED_MAX_ROWS = 1
-W4_FUSED_MAX_ROWS_LONG_K = 2
-
-
-def _w4_fused(rows: int, n: int, k: int) -> bool:
-    """Whether a W4A8 projection of ``rows`` rows takes the one-launch GEMV.
-
-    Rows longer than 4096 run on the matrix-pipe kernel, whose every 16-row workgroup then
-    quantises the whole activation row; with many workgroups that costs more than a quantiser
-    launch (5120 -> 9728: 16.3 us fused, 9.8 + 2.5 us as two launches; 9728 -> 5120 the other way).
-    """
-    if (k > 4096 and n >= 8192) or k > 10240:  # (beyond 10240 only the two-launch route has a fast kernel)
-        return False
-    return rows <= (W4_FUSED_MAX_ROWS_LONG_K if k > 5120 else W4_FUSED_MAX_ROWS)
-
 def _vp(address: int) -> int:
     """Pointer argument: the entry points declare ``void *`` (``argtypes``), so a plain int passes."""
     return address
@@ -138,20 +117,21 @@ def _on_gpu(t: torch.Tensor) -> bool:
 
 # --------------------------------------------------------------- private state
 
-#: (rows, k, device) -> (xq int8 [rows,k], xs fp32 [rows]); single-threaded caller
-#: by contract (backends/corex/__init__.py:654-690 keeps the same kind of pool).
+#: (rows, k, device) -> uint8 workspace of cmi_linear_workspace_bytes(rows, k) bytes (the
+#: quantised rows and their scales of one projection); single-threaded caller by contract
+#: (backends/corex/__init__.py:654-690 keeps the same kind of pool).
 _SCRATCH: OrderedDict = OrderedDict()
 _SCRATCH_MAX = 32
 
 
-def _scratch(rows: int, k: int, device: torch.device):
+def _scratch(rows: int, k: int, device: torch.device) -> torch.Tensor:
     key = (rows, k, device)
     hit = _SCRATCH.get(key)
     if hit is None:
         while len(_SCRATCH) >= _SCRATCH_MAX:
             _SCRATCH.popitem(last=False)          # least recently used shape goes first
-        hit = (torch.empty((rows, k), dtype=torch.int8, device=device),
-               torch.empty(rows, dtype=torch.float32, device=device))
+        nbytes = int(_native.load().cmi_linear_workspace_bytes(rows, k))
+        hit = torch.empty(nbytes, dtype=torch.uint8, device=device)
         _SCRATCH[key] = hit
     else:
         _SCRATCH.move_to_end(key)
@@ -316,30 +296,22 @@ def _gemv_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor, mfma
 
 def _gemm_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> None:
     n, k = rec.n, rec.k
-    xq, xs = _scratch(rows, k, act.device)
-    _quantize_rows(act, xq, xs, rows, k)
-    _native.check(_native.load().cmi_gemm_w8a8(_ptr(xq), rec.a, _ptr(xs), rec.b,
-                                               _ptr(out), 0, rows, n, k, n, _stream()),
-                  "gemm_w8a8")
+    work = _scratch(rows, k, act.device)
+    rc = _native.load().cmi_linear_w8a8_bf16(act.data_ptr(), rec.a, rec.b, out.data_ptr(), rows, n, k, n,
+                                             work.data_ptr(), work.numel(), _stream())
+    if rc:
+        _native.check(rc, "linear_w8a8_bf16")
 
 
 def _rows_w4(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> None:
-    n, k, gs = rec.n, rec.k, rec.gs
-    lib = _native.load()
-    if _w4_fused(rows, n, k):
-        # decode: one launch, activations quantised inside the GEMV (same bits)
-        rc = lib.cmi_gemv_w4a8_bf16(rec.a, rec.b, act.data_ptr(), out.data_ptr(), 0, 0, 0,
-                                    rows, n, k, gs, _stream())
-        if rc == 0:
-            return
-        if rc != _native.E_UNSUPPORTED:
-            _native.check(rc, "gemv_w4a8_bf16")
-    xq, xs = _scratch(rows, k, act.device)
-    _quantize_rows(act, xq, xs, rows, k)
-    fn, what = ((lib.cmi_gemm_w4a8, "gemm_w4a8") if rows >= W4_GEMM_MIN_ROWS
-                else (lib.cmi_gemv_w4a8, "gemv_w4a8"))
-    _native.check(fn(rec.a, rec.b, _ptr(xq), _ptr(xs), out.data_ptr(), 0, rows, n, k, gs,
-                     _stream()), what)
+    """Quantiser + W4A8 GEMV or GEMM in one native call; the library picks the route (one launch
+    with the quantiser folded into the GEMV for one or two rows, else two launches)."""
+    n, k = rec.n, rec.k
+    work = _scratch(rows, k, act.device)
+    rc = _native.load().cmi_linear_w4a8_bf16(rec.a, rec.b, act.data_ptr(), out.data_ptr(), rows, n, k, rec.gs,
+                                             work.data_ptr(), work.numel(), _stream())
+    if rc:
+        _native.check(rc, "linear_w4a8_bf16")
 
 
 # ------------------------------------------------------------------ dispatch
@@ -457,8 +429,143 @@ def kv_quant(x: torch.Tensor, out_q: torch.Tensor, out_s: torch.Tensor) -> torch
     return out_q
 
 
+def _rows_view(t: torch.Tensor, what: str):
+    """``(rows, width, row pitch)`` of a 1-D row or a 2-D block whose innermost stride is 1."""
+    if t.dim() == 1:
+        return 1, t.shape[0], t.shape[0]
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise ValueError(f"{what} must be [K] or [rows, K] with a unit innermost stride, "
+                         f"got shape {tuple(t.shape)} strides {t.stride()}")
+    return t.shape[0], t.shape[1], (t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1]))
+
+
+def _silu_mul_native(gate, up, out, out_q, out_s) -> bool:
+    """Run the fused kernel when every tensor is one it takes; False leaves the call to torch."""
+    tensors = [t for t in (gate, up, out, out_q, out_s) if t is not None]
+    if not all(_on_gpu(t) and t.device == gate.device for t in tensors):
+        return False
+    if not (gate.dtype == up.dtype == out.dtype == torch.bfloat16):
+        return False
+    if out_q is not None and not (out_q.dtype == torch.int8 and out_q.is_contiguous()
+                                  and out_s.dtype == torch.float32 and out_s.is_contiguous()):
+        return False
+    rows, k, ldg = _rows_view(gate, "gate")
+    _, _, ldu = _rows_view(up, "up")
+    _, _, ldo = _rows_view(out, "out")
+    with torch.cuda.device(gate.device):
+        rc = _native.load().cmi_silu_mul_quant(gate.data_ptr(), up.data_ptr(), out.data_ptr(), _ptr(out_q),
+                                               _ptr(out_s), rows, k, ldg, ldu, ldo, _stream())
+    if rc:
+        _native.check(rc, "silu_mul_quant")
+    return True
+
+
+def silu_mul(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``silu_mul(gate, up, out) -> out``: ``out = silu(gate) * up`` into a caller-owned buffer
+    that may alias ``up`` (backends/protocol.py:265-273, backends/reference/__init__.py:253-268).
+    Registered together with :func:`silu_mul_quant` so that the two share one arithmetic."""
+    if gate.shape != up.shape or out.shape != gate.shape:
+        raise ValueError("silu_mul needs gate, up and out of one shape")
+    if not _silu_mul_native(gate, up, out, None, None):
+        out.copy_(F.silu(gate) * up)
+    return out
+
+
+def silu_mul_quant(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor, out_q: torch.Tensor,
+                   out_s: torch.Tensor) -> torch.Tensor:
+    """``silu_mul_quant(gate, up, out, out_q, out_s) -> out``: the SwiGLU product written as bf16
+    and, in the same pass, quantised per row to int8 (``out_q`` + ``out_s``) -- bit for bit what
+    ``silu_mul`` followed by ``kv_quant`` gives, because the absmax is taken over the stored bf16
+    values (backends/protocol.py:274-278, backends/corex/__init__.py:1038-1071)."""
+    if gate.shape != up.shape or gate.dim() != 2:
+        raise ValueError("silu_mul_quant needs two same-shaped [rows, K] inputs")
+    if tuple(out.shape) != tuple(gate.shape) or tuple(out_q.shape) != tuple(gate.shape) \
+            or out_s.numel() != gate.shape[0]:
+        raise ValueError("silu_mul_quant expects out [rows, K], out_q [rows, K], out_s [rows]")
+    if not _silu_mul_native(gate, up, out, out_q, out_s):
+        out.copy_(F.silu(gate) * up)
+        kv_quant(out if out.is_contiguous() else out.contiguous(), out_q, out_s)
+    return out
+
+
+def rms_norm_i8(x: torch.Tensor, w: torch.Tensor, out_q: torch.Tensor, out_s: torch.Tensor,
+                eps: float = 1e-6, add: torch.Tensor | None = None,
+                out: torch.Tensor | None = None) -> torch.Tensor:
+    """RMSNorm (after ``x += add`` when ``add`` is given) quantised per row in the same pass.
+
+    Not a table entry of the contract: the reference binds ``rms_norm_i8`` / ``add_rms_norm_i8``
+    in its kernel extension only (backends/corex/kernels/norm.cu:257-350).  Same bits as
+    ``rms_norm`` / ``add_rms_norm`` written as bf16 and then quantised by ``kv_quant``
+    (backends/reference/__init__.py:169-198,224-250).  bf16 rows on the GPU only.
+    ``out`` (optional) also receives the bf16 normalised rows.  Returns ``out_q``.
+    """
+    if x.dim() != 2 or not _on_gpu(x) or x.dtype != torch.bfloat16 or x.stride(1) != 1:
+        raise ValueError("rms_norm_i8 expects bf16 [M, N] rows on the GPU with a unit innermost stride")
+    m, n = x.shape
+    gain = w if (w.dtype == torch.bfloat16 and w.is_contiguous()) else _memo(w, lambda: w.to(torch.bfloat16).contiguous())
+    if gain.numel() != n or tuple(out_q.shape) != (m, n) or out_s.numel() != m:
+        raise ValueError("rms_norm_i8 expects w [N], out_q [M, N], out_s [M]")
+    if not (out_q.dtype == torch.int8 and out_q.is_contiguous() and out_s.dtype == torch.float32
+            and out_s.is_contiguous() and out_q.device == x.device and gain.device == x.device):
+        raise ValueError("rms_norm_i8: out_q must be contiguous int8 and out_s contiguous fp32 on x's device")
+    ldx = x.stride(0) if m > 1 else max(x.stride(0), n)
+    lib = _native.load()
+    y_ptr, ldy = 0, n
+    if out is not None:
+        if tuple(out.shape) != (m, n) or out.dtype != torch.bfloat16 or out.stride(1) != 1 or out.device != x.device:
+            raise ValueError("rms_norm_i8: out must be bf16 [M, N] on x's device")
+        y_ptr, ldy = out.data_ptr(), (out.stride(0) if m > 1 else max(out.stride(0), n))
+    with torch.cuda.device(x.device):
+        if add is None:
+            rc = lib.cmi_rms_norm_i8(x.data_ptr(), gain.data_ptr(), y_ptr, out_q.data_ptr(), out_s.data_ptr(),
+                                     m, n, ldx, ldy, float(eps), _stream())
+        else:
+            if tuple(add.shape) != (m, n) or add.dtype != torch.bfloat16 or add.stride(1) != 1 \
+                    or add.device != x.device:
+                raise ValueError("rms_norm_i8: add must be bf16 [M, N] on x's device")
+            lda = add.stride(0) if m > 1 else max(add.stride(0), n)
+            rc = lib.cmi_add_rms_norm_i8(x.data_ptr(), add.data_ptr(), gain.data_ptr(), y_ptr, out_q.data_ptr(),
+                                         out_s.data_ptr(), m, n, ldx, lda, ldy, float(eps), _stream())
+    if rc:
+        _native.check(rc, "rms_norm_i8")
+    return out_q
+
+
+def embed_rows(w, ids: torch.Tensor) -> torch.Tensor:
+    """Rows ``ids`` of a quantized embedding matrix as bf16 ``[T, K]``: only the gathered rows are
+    dequantised (ops/embed.py:64-81; ``QWeight.rows`` int8_weights.py:361-372,
+    ``W4A8Weight.rows`` w4a8_weights.py:84-94).  Ids outside the vocabulary give NaN rows."""
+    rec = _lookup(w)
+    if rec is None:
+        if not (_is_w4(w) or _is_q8(w)):
+            raise ValueError("embed_rows expects a QWeight or W4A8Weight")
+        if _is_w4(w) and not _kernels_take(w):
+            raise ValueError("embed_rows: int4 rows are gathered for group size 128 and K % 128 == 0")
+        rec = _make_record(w)
+    if rec.dev.type != "cuda":
+        raise ValueError(f"coffin_amd: a quantized embedding is gathered on the GPU, weight is on {rec.dev}")
+    if ids.device != rec.dev:
+        raise ValueError(f"weight on {rec.dev} and ids on {ids.device} must share a device")
+    flat = ids.reshape(-1)
+    if flat.dtype != torch.int64 or not flat.is_contiguous():
+        flat = flat.to(torch.int64).contiguous()
+    t = flat.numel()
+    out = torch.empty((t, rec.k), dtype=torch.bfloat16, device=rec.dev)
+    lib = _native.load()
+    with torch.cuda.device(rec.dev):
+        if rec.kind == 4:
+            rc = lib.cmi_embed_rows_w4(rec.a, rec.b, flat.data_ptr(), out.data_ptr(), t, rec.n, rec.k, rec.gs,
+                                       _stream())
+        else:
+            rc = lib.cmi_embed_rows_i8(rec.a, rec.b, flat.data_ptr(), out.data_ptr(), t, rec.n, rec.k, _stream())
+    if rc:
+        _native.check(rc, "embed_rows")
+    return out
+
+
 #: Contract names this module answers natively.
-NATIVE_NAMES = ("linear", "linear_m", "linear_m_verify", "linear_prefill", "kv_quant")
+NATIVE_NAMES = ("linear", "linear_m", "linear_m_verify", "linear_prefill", "kv_quant",
+                "silu_mul", "silu_mul_quant")
 
 
 def native_table() -> dict:

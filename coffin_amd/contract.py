@@ -3,7 +3,7 @@
 When this package runs inside a coffin checkout the vendor file binds to coffin's
 own ``backends.protocol`` / ``backends.vendor`` classes; everywhere else (this
 repository's tests, the benchmark, a GPU box without the reference tree) these
-stand-ins carry the same names, fields and error behaviour for the five table
+stand-ins carry the same names, fields and error behaviour for the seven table
 entries on the path:
 
 * ``Ops`` -- backends/protocol.py:130-541: a frozen table keyed by op name,
@@ -35,6 +35,8 @@ class Ops:
     linear_m_verify: OpFn | None = None  # same shape, verify batches          (protocol.py:155)
     linear_prefill: OpFn | None = None   # linear_prefill(w, x[C,K]) -> [C,N]  (protocol.py:159)
     kv_quant: OpFn | None = None         # kv_quant(x, out_q, out_s) -> out_q  (protocol.py:258)
+    silu_mul: OpFn | None = None         # silu_mul(gate, up, out) -> out      (protocol.py:273)
+    silu_mul_quant: OpFn | None = None   # (gate, up, out, out_q, out_s) -> out (protocol.py:278)
 
     NAMES: ClassVar[tuple[str, ...]]
 

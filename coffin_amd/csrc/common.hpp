@@ -45,6 +45,10 @@ int gemv_w4a8_decode(const uint8_t *w4, const float *ws, const void *x, const in
 int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs, const void *x,
                      void *y, int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
                      void *stream);
+// linear_bf16.hip: quantiser + W4A8 GEMV / GEMM (or the GEMV that quantises by itself where that
+// is faster) on bf16 rows, with xq int8 [M,K] / xs fp32 [M] as staging; arguments already checked.
+int linear_w4a8_rows(const uint8_t *w4, const float *ws, const void *x, void *y, int M, int N, int K, int gs,
+                     int8_t *xq, float *xs, void *stream);
 static inline bool aligned(const void *p, uintptr_t a) {
     return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
 }

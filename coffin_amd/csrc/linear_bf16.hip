@@ -1,0 +1,82 @@
+// Whole projections from bf16 activations for the integer paths: per-token quantiser + W8A8
+// GEMM, and quantiser + W4A8 GEMV / GEMM (or the GEMV with the quantiser folded in where that
+// is the faster route).  One call per projection instead of two keeps the host side of a decode
+// step short, and puts the choice of route next to the kernels it chooses between.
+//
+// The quantised rows (xq int8 [M,K]) and their scales (xs fp32 [M]) live in a workspace that the
+// caller brings.
+#include "common.hpp"
+
+namespace {
+
+using namespace cmi;
+
+constexpr size_t ALIGN = 256;
+constexpr size_t round_up(size_t v) { return (v + ALIGN - 1) / ALIGN * ALIGN; }
+
+// Whether `rows` bf16 rows go through the W4A8 GEMV that quantises them itself (one launch).
+// That kernel lets every workgroup redo the quantisation: it wins for one row (two on long
+// rows), and loses where many workgroups each quantise a long row (K > 4096 with N >= 8192:
+// 5120 -> 9728 takes 16.3 us fused against 9.8 + 2.5 us as two launches); beyond K = 10240
+// only the two-launch route has a fast kernel.
+bool w4_fused_route(int rows, int N, int K) {
+    if ((K > 4096 && N >= 8192) || K > 10240) return false;
+    return rows <= (K > 5120 ? 2 : 1);
+}
+
+}  // namespace
+
+int cmi::linear_w4a8_rows(const uint8_t *w4, const float *ws, const void *x, void *y, int M, int N, int K,
+                          int gs, int8_t *xq, float *xs, void *stream) {
+    if (w4_fused_route(M, N, K)) {
+        const int rc = cmi_gemv_w4a8_bf16(w4, ws, x, y, nullptr, nullptr, nullptr, M, N, K, gs, stream);
+        if (rc != CMI_E_UNSUPPORTED) return rc;
+    }
+    if (const int rc = cmi_quant_act_i8(x, xq, xs, M, K, stream)) return rc;
+    // up to 16 rows the GEMV entry; beyond, the GEMM entry (which itself goes through the
+    // read-once kernels while they are cheaper than the tile pipeline)
+    if (M <= 16) return cmi_gemv_w4a8(w4, ws, xq, xs, y, nullptr, M, N, K, gs, stream);
+    return cmi_gemm_w4a8(w4, ws, xq, xs, y, nullptr, M, N, K, gs, stream);
+}
+
+namespace {
+
+int split_workspace(const char *who, void *workspace, size_t bytes, int M, int K, int8_t **xq, float **xs) {
+    CMI_REQUIRE(workspace, CMI_E_ARG, "%s: null workspace", who);
+    CMI_REQUIRE(aligned(workspace, 16), CMI_E_ARG, "%s: workspace must be 16-byte aligned", who);
+    const size_t need = cmi_linear_workspace_bytes(M, K);
+    CMI_REQUIRE(bytes >= need, CMI_E_ARG, "%s: workspace of %zu bytes, %zu needed for M=%d K=%d", who, bytes, need, M, K);
+    *xq = static_cast<int8_t *>(workspace);
+    *xs = reinterpret_cast<float *>(static_cast<unsigned char *>(workspace) + round_up((size_t)M * K));
+    return CMI_OK;
+}
+
+}  // namespace
+
+extern "C" size_t cmi_linear_workspace_bytes(int M, int K) {
+    if (M <= 0 || K <= 0) return 0;
+    return round_up((size_t)M * K) + round_up(sizeof(float) * (size_t)M);
+}
+
+extern "C" int cmi_linear_w8a8_bf16(const void *x, const int8_t *wq, const float *ws, void *y, int M, int N, int K,
+                                    int ldy, void *workspace, size_t workspace_bytes, void *stream) {
+    CMI_REQUIRE(M >= 0 && N >= 1 && K >= 16, CMI_E_ARG, "cmi_linear_w8a8_bf16: bad shape M=%d N=%d K=%d", M, N, K);
+    if (M == 0) return CMI_OK;
+    CMI_REQUIRE(x && wq && ws && y, CMI_E_ARG, "cmi_linear_w8a8_bf16: null pointer");
+    int8_t *xq;
+    float *xs;
+    if (const int rc = split_workspace("cmi_linear_w8a8_bf16", workspace, workspace_bytes, M, K, &xq, &xs)) return rc;
+    if (const int rc = cmi_quant_act_i8(x, xq, xs, M, K, stream)) return rc;
+    return cmi_gemm_w8a8(xq, wq, xs, ws, y, nullptr, M, N, K, ldy, stream);
+}
+
+extern "C" int cmi_linear_w4a8_bf16(const uint8_t *w4, const float *ws, const void *x, void *y, int M, int N, int K,
+                                    int gs, void *workspace, size_t workspace_bytes, void *stream) {
+    CMI_REQUIRE(M >= 0 && N >= 1 && K >= 128, CMI_E_ARG, "cmi_linear_w4a8_bf16: bad shape M=%d N=%d K=%d", M, N, K);
+    if (M == 0) return CMI_OK;
+    CMI_REQUIRE(w4 && ws && x && y, CMI_E_ARG, "cmi_linear_w4a8_bf16: null pointer");
+    int8_t *xq;
+    float *xs;
+    if (const int rc = split_workspace("cmi_linear_w4a8_bf16", workspace, workspace_bytes, M, K, &xq, &xs)) return rc;
+    return linear_w4a8_rows(w4, ws, x, y, M, N, K, gs, xq, xs, stream);
+}

@@ -21,6 +21,7 @@
 #ifndef COFFIN_MI355_H
 #define COFFIN_MI355_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -136,6 +137,63 @@ int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs, const flo
  * backends/corex/__init__.py:647). group_acc as in cmi_gemv_w4a8. */
 int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs,
                   void *y, int32_t *group_acc, int M, int N, int K, int gs, void *stream);
+
+/* Whole projections from bf16 activations, one call each: the per-token quantiser into a
+ * caller's workspace, then the integer kernels on the quantised rows; same bits as the separate
+ * calls.  `workspace` is device memory, 16-byte aligned, of at least
+ * cmi_linear_workspace_bytes(M, K) bytes (xq int8 [M,K], then xs fp32 [M], each rounded up to
+ * 256 bytes); its contents after the call are the quantised rows and scales the kernels used.
+ *   cmi_linear_w8a8_bf16: cmi_quant_act_i8 + cmi_gemm_w8a8 -- what _w8a8_rows issues
+ *     (backends/corex/__init__.py:1557-1609: quant_act_i8 into private scratch, then the GEMM).
+ *   cmi_linear_w4a8_bf16: what _w4_rows issues (backends/corex/__init__.py:576-651: quant_act_i8
+ *     into private scratch, then w4a8_gemv or w4a8_gemm_tcu by row count); the GEMV that
+ *     quantises by itself (cmi_gemv_w4a8_bf16) is taken where it is the faster route, the GEMV
+ *     entry up to 16 rows, the GEMM entry beyond. */
+size_t cmi_linear_workspace_bytes(int M, int K);
+int cmi_linear_w8a8_bf16(const void *x, const int8_t *wq, const float *ws, void *y, int M, int N,
+                         int K, int ldy, void *workspace, size_t workspace_bytes, void *stream);
+int cmi_linear_w4a8_bf16(const uint8_t *w4, const float *ws, const void *x, void *y, int M, int N,
+                         int K, int gs, void *workspace, size_t workspace_bytes, void *stream);
+
+/* silu_mul and silu_mul_quant (backends/protocol.py:265-278; native form
+ * backends/corex/kernels/attn.cu:594-641, adapter backends/corex/__init__.py:1038-1071):
+ *   out[m,k] = bf16( float(bf16(silu(gate[m,k]))) * float(up[m,k]) ),  silu(g) = g / (1 + exp(-g)) in fp32
+ *   out_q, out_s = cmi_quant_act_i8(out)      (absmax over the stored bf16 values: same bits as
+ *                                              silu_mul followed by the quantiser)
+ * gate, up: bf16 [M,K] with row pitches ld_gate, ld_up (elements; the two halves of a fused
+ * gate_up projection have pitch 2K); out: bf16 with row pitch ld_out, may alias `up`, nullable
+ * when only the quantised row is wanted; out_q int8 [M,K] dense and out_s fp32 [M], nullable
+ * together (then this is silu_mul). */
+int cmi_silu_mul_quant(const void *gate, const void *up, void *out, int8_t *out_q, float *out_s,
+                       int M, int K, int64_t ld_gate, int64_t ld_up, int64_t ld_out, void *stream);
+
+/* RMSNorm with the gain applied, optionally written as bf16 (y, pitch ld_y, nullable) and / or
+ * quantised per row (out_q int8 [M,N] dense + out_s fp32 [M], nullable together); the
+ * quantised row equals cmi_quant_act_i8 of the bf16 row bit for bit.  Arithmetic of
+ * backends/reference/__init__.py:169-198:
+ *   scale = 1 / sqrt(mean_k x^2 + eps)   (the mean correctly rounded to fp32)
+ *   y = bf16( float(bf16(x * scale)) * float(w) )          x bf16 [M,N] pitch ld_x, w bf16 [N]
+ * Stands where rms_norm_i8 is bound (backends/corex/kernels/norm.cu:310-350). */
+int cmi_rms_norm_i8(const void *x, const void *w, void *y, int8_t *out_q, float *out_s, int M,
+                    int N, int64_t ld_x, int64_t ld_y, float eps, void *stream);
+
+/* The same after the residual add of backends/reference/__init__.py:224-250:
+ * x = bf16(x + add) is written back to x (the residual stream), then normalised as above.
+ * Stands where add_rms_norm_i8 is bound (backends/corex/kernels/norm.cu:257-308). */
+int cmi_add_rms_norm_i8(void *x, const void *add, const void *w, void *y, int8_t *out_q,
+                        float *out_s, int M, int N, int64_t ld_x, int64_t ld_add, int64_t ld_y,
+                        float eps, void *stream);
+
+/* Embedding lookup on a quantized weight: rows `ids` (int64 [T]) dequantised to bf16 [T,K].
+ *   int8: out[t,k] = bf16(float(wq[id,k]) * ws[id])         (ops/embed.py:64-81, int8_weights.py:359)
+ *   int4: out[t,k] = bf16(float(code-8) * ws[id,k/gs])      (w4a8_weights.py:84-94), on the
+ *         re-laid-out weight of cmi_w4_repack (gs == 128, K % 128 == 0)
+ * An id outside [0, N) gives a row of bf16 NaN (a device-side range error cannot be returned
+ * without synchronising). */
+int cmi_embed_rows_i8(const int8_t *wq, const float *ws, const int64_t *ids, void *out, int T,
+                      int N, int K, void *stream);
+int cmi_embed_rows_w4(const uint8_t *w4, const float *ws, const int64_t *ids, void *out, int T,
+                      int N, int K, int gs, void *stream);
 
 #ifdef __cplusplus
 }

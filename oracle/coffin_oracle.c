@@ -351,3 +351,77 @@ void orc_linear_w4a8(const int8_t *xq, const float *xs, const uint8_t *packed,
         free(col);
     }
 }
+
+/* ------------------------------ fused producers of quantised activations */
+
+/* exp(x) rounded once to fp32.  The reference evaluates silu in fp32 with its
+ * library's expf (torch's vectorised routine, accurate to about one unit in the
+ * last place, so the reference's own bits depend on the library); this oracle
+ * fixes the ideal that routine approximates: the double-precision exp narrowed
+ * once. */
+static inline float expf_rounded_once(float x) { return (float)exp((double)x); }
+
+/* silu(g) narrowed to bf16: g / (1 + exp(-g)), every operation in fp32.
+ * backends/reference/__init__.py:253-268 (F.silu on a bf16 tensor computes in
+ * fp32 and narrows); backends/corex/kernels/attn.cu:612-614. */
+static inline uint16_t silu_bf16(uint16_t g_bits) {
+    const float g = bf16_to_f32(g_bits);
+    return f32_to_bf16(g / (1.f + expf_rounded_once(-g)));
+}
+
+void orc_silu_bf16(const uint16_t *g, uint16_t *out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = silu_bf16(g[i]);
+}
+
+/* Ops.silu_mul followed by Ops.kv_quant on its output, which is what
+ * Ops.silu_mul_quant must equal bit for bit (backends/protocol.py:274-278,
+ * backends/corex/kernels/attn.cu:594-641):
+ *   s   = bf16(silu(gate))                    (first narrowing)
+ *   out = bf16(float(s) * float(up))          (second narrowing; F.silu(gate) * up on bf16)
+ *   q, sc = quant_act_i8(out)                 (absmax of the STORED bf16 values)
+ * gate, up: bf16 [M,K] with row pitches ldg, ldu (elements); out bf16 [M,K] dense;
+ * q int8 [M,K]; sc fp32 [M]. */
+void orc_silu_mul_quant(const uint16_t *gate, const uint16_t *up, int64_t M, int64_t K,
+                        int64_t ldg, int64_t ldu, uint16_t *out, int8_t *q, float *sc) {
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t k = 0; k < K; ++k) {
+            const float s = bf16_to_f32(silu_bf16(gate[m * ldg + k]));
+            out[m * K + k] = f32_to_bf16(s * bf16_to_f32(up[m * ldu + k]));
+        }
+    if (q && sc) orc_quant_act_i8(out, M, K, q, sc);
+}
+
+/* Zero-centred RMSNorm of the reference, backends/reference/__init__.py:169-198:
+ *   xf = x.float(); scale = rsqrt(mean(xf^2) + eps); y = (xf*scale).to(bf16) * w.to(bf16)
+ * optionally after the residual add of :224-250 (x = bf16(x + add), written back).
+ * The reference leaves the fp32 summation order of the mean to torch; this oracle
+ * fixes the value every order approximates: the squares (exact in fp32: 8-bit
+ * significands) are summed in double, k ascending -- exact, hence order-free,
+ * whenever the row's magnitudes span less than 2^20 -- divided by N in double and
+ * narrowed once.  rsqrt is 1/sqrt with both operations correctly rounded, as
+ * torch's CPU kernel evaluates it.  The bf16 product of two bf16 tensors is one
+ * fp32 multiply and one narrowing.
+ * x: bf16 [M,N] with row pitch ldx, updated in place when add != NULL (pitch
+ * lda); w: bf16 [N]; y: bf16 [M,N] dense. */
+void orc_rms_norm(uint16_t *x, const uint16_t *add, const uint16_t *w, int64_t M, int64_t N,
+                  int64_t ldx, int64_t lda, float eps, uint16_t *y) {
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+        uint16_t *xr = x + m * ldx;
+        if (add)
+            for (int64_t k = 0; k < N; ++k)
+                xr[k] = f32_to_bf16(bf16_to_f32(xr[k]) + bf16_to_f32(add[m * lda + k]));
+        double ss = 0.0;
+        for (int64_t k = 0; k < N; ++k) {
+            const double v = (double)bf16_to_f32(xr[k]);
+            ss += v * v;
+        }
+        const float ms = (float)(ss / (double)N);
+        const float scale = 1.0f / sqrtf(ms + eps);
+        for (int64_t k = 0; k < N; ++k) {
+            const float normed = bf16_to_f32(f32_to_bf16(bf16_to_f32(xr[k]) * scale));
+            y[m * N + k] = f32_to_bf16(normed * bf16_to_f32(w[k]));
+        }
+    }
+}

@@ -205,3 +205,38 @@ def from_bits(a: np.ndarray):
     import torch
     return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).view(torch.bfloat16)
 
+
+
+# ------------------------------------------------------- fused quant producers
+
+def silu_bf16(g_bf16: np.ndarray) -> np.ndarray:
+    """bf16 bits of silu(g), fp32 arithmetic (backends/reference/__init__.py:253-268)."""
+    g = np.ascontiguousarray(g_bf16, dtype=np.uint16)
+    out = np.empty_like(g)
+    lib().orc_silu_bf16(_p(g), _p(out), _i(g.size))
+    return out
+
+
+def silu_mul_quant(gate: np.ndarray, up: np.ndarray, quant: bool = True):
+    """``silu_mul`` then ``kv_quant`` (backends/protocol.py:274-278).  gate, up: bf16 bits
+    [M,K] -> (out bf16 bits [M,K], q int8 [M,K] or None, s fp32 [M] or None)."""
+    m, k = gate.shape
+    out = np.empty((m, k), dtype=np.uint16)
+    q = np.empty((m, k), dtype=np.int8) if quant else None
+    s = np.empty(m, dtype=np.float32) if quant else None
+    lib().orc_silu_mul_quant(_p(np.ascontiguousarray(gate)), _p(np.ascontiguousarray(up)), _i(m), _i(k),
+                             _i(k), _i(k), _p(out), _p(q), _p(s))
+    return out, q, s
+
+
+def rms_norm(x: np.ndarray, w: np.ndarray, eps: float = 1e-6, add: np.ndarray | None = None):
+    """Reference RMSNorm (backends/reference/__init__.py:169-198), after the residual add of
+    :224-250 when ``add`` is given.  x, add: bf16 bits [M,N]; w: bf16 bits [N] ->
+    (y bf16 bits [M,N], x after the add, bf16 bits [M,N])."""
+    m, n = x.shape
+    xs = np.array(x, dtype=np.uint16, order="C", copy=True)
+    y = np.empty((m, n), dtype=np.uint16)
+    a = None if add is None else np.ascontiguousarray(add, dtype=np.uint16)
+    lib().orc_rms_norm(_p(xs), _p(a), _p(np.ascontiguousarray(w, dtype=np.uint16)), _i(m), _i(n),
+                       _i(n), _i(n), ctypes.c_float(eps), _p(y))
+    return y, xs

@@ -41,9 +41,13 @@ def _w4(n, k, g):
 def test_vendor_builds_the_native_table():
     ops = mi355x.build_ops()
     assert set(ops.implemented()) == {"linear", "linear_m", "linear_m_verify", "linear_prefill",
-                                      "kv_quant"}
+                                      "kv_quant", "silu_mul", "silu_mul_quant"}
     from coffin_amd import contract
-    assert contract.detect(mi355x.SPEC.detection) == contract.CLAIM_NAME
+    # a board that reports its name is claimed by name; a host without the amdgpu id table
+    # reports the generic "AMD Radeon Graphics", which is left to explicit selection
+    name = torch.cuda.get_device_name(0).lower()
+    named = any(m in name for m in mi355x.SPEC.detection.name_markers)
+    assert contract.detect(mi355x.SPEC.detection) == (contract.CLAIM_NAME if named else contract.CLAIM_NONE)
 
 
 def test_reference_linear_assertions_on_device():
@@ -281,8 +285,12 @@ def test_shape_and_device_errors():
             backend.linear(weight, torch.zeros(128, dtype=torch.bfloat16))
     odd = W4A8Weight(torch.full((128, 8), 0x88, dtype=torch.uint8, device=G.DEV),
                      torch.ones((4, 8), device=G.DEV), k=256, group_size=64)
-    with pytest.raises(ValueError, match="group size"):
-        backend.linear(odd, torch.zeros(256, dtype=torch.bfloat16, device=G.DEV))
+    # a group size the kernels are not built for is answered by the torch statement of the op
+    # (backends/reference/__init__.py:93-95), as the reference's adapter falls back for shapes its
+    # kernels refuse
+    xo = synth.activations(3, 256, g).to(G.DEV)
+    want = torch.nn.functional.linear(xo, odd.to(torch.bfloat16))
+    assert (backend.linear_m(odd, xo).view(torch.int16) == want.view(torch.int16)).all()
     empty = backend.linear_m(q, torch.zeros(0, 128, dtype=torch.bfloat16, device=G.DEV))
     assert empty.shape == (0, 64)
 

@@ -23,7 +23,7 @@ ROOT = Path(__file__).resolve().parent.parent
 
 def test_ops_table_names_and_errors():
     assert contract.Ops.NAMES == ("linear", "linear_m", "linear_m_verify", "linear_prefill",
-                                  "kv_quant")
+                                  "kv_quant", "silu_mul", "silu_mul_quant")
     t = contract.Ops.from_mapping({"linear": lambda w, x: x})
     assert t.implemented() == ("linear",) and "kv_quant" in t.missing()
     with pytest.raises(ValueError, match="unknown op"):
@@ -40,6 +40,8 @@ def test_vendor_spec_validation_and_declaration():
     assert spec.has_kernels and callable(spec.build_ops)
     assert spec.detection.namespace == "cuda" and spec.detection.hip
     assert all(m == m.lower() for m in spec.detection.name_markers)
+    # the generic name every id-table-less AMD host reports must not be claimed
+    assert not any(m in "amd radeon graphics" for m in spec.detection.name_markers)
     with pytest.raises(ValueError, match="weight_layout"):
         contract.VendorSpec(name="x", detection=contract.Detection("cuda"),
                             weight_layout="kk").validate()
@@ -171,15 +173,6 @@ def test_gemv_regimes_follow_row_count():
         ("linear_m", (8, 4)), ("linear_prefill", (9, 4))]
 
 
-def test_w4_one_launch_rule():
-    from coffin_amd import backend
-    assert backend._w4_fused(1, 9728, 2560) and not backend._w4_fused(2, 9728, 2560)
-    assert backend._w4_fused(2, 2560, 9728) and not backend._w4_fused(3, 2560, 9728)
-    # long rows and many workgroups: the quantiser gets a launch of its own
-    assert not backend._w4_fused(1, 25600, 5120) and not backend._w4_fused(1, 5120, 25600)
-    assert backend._w4_fused(1, 5120, 9728)
-
-
 def test_gemv_group_fuses_and_splits():
     g = synth.generator()
     qa, qb = synth.int8_weight(6, 32, g), synth.int8_weight(10, 32, g)
@@ -202,34 +195,35 @@ def test_gemv_group_fuses_and_splits():
     assert dense.g.w.shape == (5, 4)
 
 
-def test_tied_embedding_lookup_dequantises_only_the_gathered_rows(orc):
-    """ops/embed.py:64-81: bf16 rows whatever the storage, equal to the oracle's dequantisation
-    of those rows; the projection side goes through GEMV with the same weight."""
+def test_tied_embedding_routes_lookup_and_projection():
+    """Quantized storage is gathered by the native row gather (handed the weight object and the
+    ids), plain storage by index_select; both projection entries go to the table; the
+    reference's attribute surface (ops/embed.py:29-104) is kept."""
     g = synth.generator()
     ids = torch.tensor([5, 0, 39, 5, 17])
+    seen = []
+
+    def gather(w, i):
+        seen.append((w, i))
+        return torch.zeros((i.numel(), w.k), dtype=torch.bfloat16)
+
     q = synth.int8_weight(40, 96, g)
-    emb = embed.TiedEmbedding(q, ops=Recorder())
-    assert emb.shape == (40, 96) and emb.gemv.q is q and emb.w is None
-    rows = emb.lookup(ids)
-    assert rows.dtype == torch.bfloat16 and rows.shape == (5, 96)
-    want = orc.qweight_dequant_bf16(q.wq.numpy(), q.scale.numpy())[ids.numpy()]
-    assert (rows.view(torch.int16).numpy().view(np.uint16) == want).all()
-
+    emb = embed.TiedEmbedding(q, ops=Recorder(), gather=gather)
+    assert emb.shape == (40, 96) and emb.q is q and emb.q4 is None and emb.w is None and emb.gemv.q is q
+    assert emb.lookup(ids).shape == (5, 96) and seen[-1][0] is q and seen[-1][1] is ids
     w4 = synth.int4_weight(40, 256, g)
-    emb4 = embed.TiedEmbedding(w4, ops=Recorder())
-    assert emb4.shape == (40, 256) and emb4.gemv.q4 is w4
-    rows4 = emb4.lookup(ids)
-    dense = orc.w4_dequant_f32(w4.packed.numpy(), w4.scale.numpy(), 256)[ids.numpy()]
-    assert rows4.dtype == torch.bfloat16
-    assert (rows4.view(torch.int16).numpy().view(np.uint16) == orc.bf16_from_f32(dense)).all()
-
+    emb4 = embed.TiedEmbedding(w4, ops=Recorder(), gather=gather)
+    assert emb4.shape == (40, 256) and emb4.q4 is w4 and emb4.q is None and emb4.gemv.q4 is w4
+    assert emb4.lookup(ids).shape == (5, 256) and seen[-1][0] is w4
+    # no CPU path for quantized storage: the default gather refuses a CPU weight
+    with pytest.raises(ValueError, match="GPU"):
+        embed.TiedEmbedding(q, ops=Recorder()).lookup(ids)
     plain = torch.randn(12, 8, generator=g)
-    embp = embed.TiedEmbedding(plain, ops=Recorder())
-    assert embp.shape == (12, 8)
+    embp = embed.TiedEmbedding(plain, ops=Recorder(), gather=gather)
+    assert embp.shape == (12, 8) and embp.w is plain and len(seen) == 2
     assert (embp.lookup(torch.tensor([3, 3, 11])) == plain[[3, 3, 11]].to(torch.bfloat16)).all()
-    # both projection entries hand the weight to the table
     rec = Recorder()
-    proj = embed.TiedEmbedding(q, ops=rec)
+    proj = embed.TiedEmbedding(q, ops=rec, gather=gather)
     assert proj(torch.zeros(96)).shape == (40,) and proj.prefill(torch.zeros(9, 96)).shape == (9, 40)
     assert [c[0] for c in rec.calls] == ["linear", "linear_prefill"]
 
@@ -281,6 +275,7 @@ def test_scratch_and_record_pools_evict_the_least_recently_used_entry(monkeypatc
     backend._SCRATCH.clear()
     cpu = torch.device("cpu")
     a = backend._scratch(1, 16, cpu)
+    assert a.dtype == torch.uint8 and a.numel() == 512     # 16 B of rows + 4 B of scale, 256 each
     backend._scratch(2, 16, cpu)
     backend._scratch(3, 16, cpu)
     assert backend._scratch(1, 16, cpu) is a               # refreshed: now the most recent
@@ -344,7 +339,8 @@ def test_library_exports_every_declared_symbol():
     names = _declared_symbols()
     for name in names:
         assert getattr(lib, name) is not None
-    assert set(_native.SIGNATURES) | {"cmi_abi_version", "cmi_last_error"} == set(names)
+    assert (set(_native.SIGNATURES) | set(_native.OTHER_RESTYPES) | {"cmi_abi_version", "cmi_last_error"}
+            == set(names))
     assert lib.cmi_abi_version() == _native.ABI_VERSION
 
 

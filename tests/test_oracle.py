@@ -317,3 +317,100 @@ def test_linear_w4weight_is_dequant_then_linear(orc):
     # quantization error bound of the format itself: |w - dequant| <= step/2
     assert (np.abs(dense.float().numpy() - w.numpy()) <=
             np.repeat(scale.T, 128, axis=1) * 0.51 + np.abs(w.numpy()) * 2.0 ** -8).all()
+
+
+# ------------------------------------------- fused producers: silu_mul, rms_norm
+
+def _all_bf16():
+    bits = np.arange(65536, dtype=np.uint16)
+    return bits, torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16)
+
+
+def test_silu_table_matches_torch_on_every_finite_bf16_and_the_exact_function(orc):
+    """silu of a bf16 value is a function of 16 bits.  All of them against torch's CPU F.silu
+    (an independent evaluation of the reference's expression), and against the exact function
+    in 50-digit decimal arithmetic wherever the exact value is not within 2^-18 (relative) of a
+    bf16 rounding boundary -- the fp32 pipeline's own roundings stay far inside that."""
+    from decimal import Decimal, getcontext
+    bits, t = _all_bf16()
+    got = orc.silu_bf16(bits)
+    f = t.float().numpy()
+    finite = np.isfinite(f)
+    want = _bits(torch.nn.functional.silu(t))
+    assert (got[finite] == want[finite]).all()
+    # known answers and limits
+    as_f = orc.bf16_to_f32(got)
+    assert as_f[0x0000] == 0.0 and as_f[0x3F80] == np.float32(0.73046875)      # silu(1) = 0.731058... -> bf16
+    assert as_f[0x7F80] == np.inf and np.isnan(as_f[0xFF80])                    # +inf -> +inf, -inf -> nan
+    big = f > 20
+    assert (got[big & finite] == bits[big & finite]).all()                      # silu(x) -> x
+    getcontext().prec = 50
+    sample = np.concatenate([np.arange(0x3000, 0x4200, 7), np.arange(0xB000, 0xC200, 7)])   # |x| in [2^-31, 8]
+    checked = 0
+    for b in sample:
+        x = Decimal(float(f[b]))
+        exact = x / (1 + (-x).exp())
+        lo = float(orc.bf16_to_f32(np.array([got[b]], dtype=np.uint16))[0])
+        ulp = 2.0 ** (np.floor(np.log2(abs(lo))) - 7)
+        # distance from the returned bf16 value must not exceed half a step, up to the tie margin
+        assert abs(exact - Decimal(lo)) <= Decimal(ulp) * (Decimal("0.5") + Decimal(2) ** -10), hex(int(b))
+        checked += 1
+    assert checked > 1000
+
+
+def test_silu_mul_quant_is_silu_mul_then_the_quantiser(orc):
+    rng = torch.Generator().manual_seed(1234)
+    gate = (torch.randn((9, 300), generator=rng) * 3).to(torch.bfloat16)
+    up = torch.randn((9, 300), generator=rng).to(torch.bfloat16)
+    gate[4].zero_()                                                             # a zero row: q = 0, floor scale
+    out, q, s = orc.silu_mul_quant(_bits(gate), _bits(up))
+    want = torch.nn.functional.silu(gate) * up                                  # the reference statement, torch CPU
+    assert (out == _bits(want)).all()
+    q_ref, s_ref = orc.quant_act_i8(out)
+    assert (q == q_ref).all() and (s == s_ref).all()
+    assert (q[4] == 0).all() and s[4] == np.float32(1e-5) / np.float32(127)
+    out2, q2, s2 = orc.silu_mul_quant(_bits(gate), _bits(up), quant=False)
+    assert (out2 == out).all() and q2 is None and s2 is None
+
+
+def test_rms_norm_known_answers_and_the_reference_expression(orc):
+    """Closed forms (constant and zero rows), torch's CPU evaluation of the reference's lines
+    (backends/reference/__init__.py:195-198) and an fp64 evaluation.  torch sums the squares in
+    fp32 in an order of its own, so its scale may sit one fp32 step from the correctly rounded
+    one: outputs agree bit for bit except where that step crosses a bf16 boundary."""
+    rng = torch.Generator().manual_seed(1234)
+    x = (torch.randn((33, 2560), generator=rng) * 2).to(torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(2560, generator=rng)).to(torch.bfloat16)
+    x[0].zero_()
+    x[1] = 0.5
+    x[2] = -3.0
+    y, x_after = orc.rms_norm(_bits(x), _bits(w))
+    assert (x_after == _bits(x)).all()
+    yf = orc.bf16_to_f32(y)
+    wf = w.float().numpy()
+    assert (yf[0] == 0).all()
+    assert (yf[1] == wf).all() and (yf[2] == -wf).all()                         # |x| / sqrt(x^2 + 1e-6) -> 1
+    xf = x.float()
+    scale = torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + 1e-6)
+    ref = (xf * scale).to(torch.bfloat16) * w
+    same = (y == _bits(ref))
+    assert same.mean() > 0.995
+    step = np.abs(yf) * 2.0 ** -7 + 1e-30
+    assert (np.abs(yf - ref.float().numpy()) <= step).all()
+    x64 = xf.double().numpy()
+    s64 = 1.0 / np.sqrt((x64 ** 2).mean(-1, keepdims=True) + 1e-6)
+    exact = x64 * s64 * w.double().numpy()
+    assert (np.abs(yf - exact) <= np.abs(exact) * 2.0 ** -7 * 1.01 + 1e-30).all()  # two bf16 roundings
+    # the residual add: bf16(x + add) written back, then the norm of the sum
+    add = torch.randn((33, 2560), generator=rng).to(torch.bfloat16)
+    y2, x2 = orc.rms_norm(_bits(x), _bits(w), add=_bits(add))
+    summed = x + add                                                            # torch: fp32 add, one narrowing
+    assert (x2 == _bits(summed)).all()
+    y3, _ = orc.rms_norm(_bits(summed), _bits(w))
+    assert (y2 == y3).all()
+    # eps matters on small rows: x = 1e-3 -> 1e-3 / sqrt(1e-6 + 1e-6)
+    tiny = torch.full((1, 64), 1e-3).to(torch.bfloat16)
+    yt, _ = orc.rms_norm(_bits(tiny), _bits(torch.ones(64).to(torch.bfloat16)))
+    v = float(tiny[0, 0])
+    want = torch.tensor(v / np.sqrt(v * v + 1e-6)).to(torch.bfloat16)
+    assert (orc.bf16_to_f32(yt) == float(want)).all()
