@@ -34,6 +34,7 @@ SIGNATURES: dict[str, list] = {
     "cmi_gemm_w4a8": [_vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cmi_linear_w8a8_bf16": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp, _sz, _vp],
     "cmi_linear_w4a8_bf16": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp, _sz, _vp],
+    "cmi_linear_w4a8_bf16_static": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cmi_silu_mul_quant": [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _i64, _i64, _i64, _vp],
     "cmi_rms_norm_i8": [_vp, _vp, _vp, _vp, _vp, _ci, _ci, _i64, _i64, _f32, _vp],
     "cmi_add_rms_norm_i8": [_vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _i64, _i64, _i64, _f32, _vp],

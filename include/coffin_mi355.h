@@ -155,6 +155,17 @@ int cmi_linear_w8a8_bf16(const void *x, const int8_t *wq, const float *ws, void 
 int cmi_linear_w4a8_bf16(const uint8_t *w4, const float *ws, const void *x, void *y, int M, int N,
                          int K, int gs, void *workspace, size_t workspace_bytes, void *stream);
 
+/* cmi_linear_w4a8_bf16 without the workspace argument, for callers that cannot allocate device
+ * memory: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * No counterpart in the reference (its adapters allocate their scratch through torch).  The
+ * quantised rows and scales go through a fixed array inside the library -- 8 MiB + 64 KiB per
+ * GPU, held until the process ends -- so M <= 16384 and M*K <= 8 MiB (8388608), otherwise
+ * CMI_E_UNSUPPORTED and nothing is launched.  The call itself allocates and frees nothing.  All
+ * calls on one GPU share that array: calls that overlap on one GPU (different streams or
+ * threads) race and must be ordered by the caller.  Same bits as cmi_linear_w4a8_bf16. */
+int cmi_linear_w4a8_bf16_static(const uint8_t *w4, const float *ws, const void *x, void *y, int M,
+                                int N, int K, int gs, void *stream);
+
 /* silu_mul and silu_mul_quant (backends/protocol.py:265-278; native form
  * backends/corex/kernels/attn.cu:594-641, adapter backends/corex/__init__.py:1038-1071):
  *   out[m,k] = bf16( float(bf16(silu(gate[m,k]))) * float(up[m,k]) ),  silu(g) = g / (1 + exp(-g)) in fp32
