@@ -41,15 +41,13 @@
 // mid-sized weight with K in one unit) takes gemv_w8a16_wholerow_kernel instead: one
 // wavefront per weight row, all units.
 
-#include "common.hpp"
+#include "gemv_w8a16_math.hpp"
 
 #include <cstdlib>
 
 namespace {
 
 using namespace cmi;
-
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 struct GemvArgs {
     const int8_t *wq;
@@ -68,29 +66,6 @@ struct GemvArgs {
     uint32_t uw_rcp;  // ceil(2^16 / uw)
     int teams;      // row blocks per workgroup
 };
-
-// Segments per unit: the largest of 4,3,2,1 that pads K by at most a fifth.
-inline int unit_segments(int nseg) {
-    for (int u = 4; u > 1; --u) {
-        const int padded = (nseg + u - 1) / u * u;
-        if ((padded - nseg) * 5 <= padded) return u;
-    }
-    return 1;
-}
-
-// Four int8 in one dword -> two packed-bf16 pairs (k, k+1) and (k+2, k+3).
-__device__ __forceinline__ void widen4(uint32_t w, bf16x2_t &lo, bf16x2_t &hi) {
-    const float f0 = (float)(int8_t)(w);
-    const float f1 = (float)(int8_t)(w >> 8);
-    const float f2 = (float)(int8_t)(w >> 16);
-    const float f3 = (float)(int8_t)(w >> 24);
-    // Integers up to 127 occupy only the upper 16 bits of their fp32 pattern,
-    // so taking the high halves is an exact conversion to bf16.
-    const uint32_t p0 = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u);
-    const uint32_t p1 = __builtin_amdgcn_perm(__float_as_uint(f3), __float_as_uint(f2), 0x07060302u);
-    lo = __builtin_bit_cast(bf16x2_t, p0);
-    hi = __builtin_bit_cast(bf16x2_t, p1);
-}
 
 // Wavefronts per workgroup (they share one LDS copy of the activations); wide
 // batches get smaller workgroups so that each wavefront may use more registers.
