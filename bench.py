@@ -34,10 +34,107 @@ LAYERS = 32
 METRIC = "decode GEMV HBM GB/s (% of peak) + W8A8 prefill int8 TOPS, Qwen3.5-4B shapes"
 
 
-#: gemv_w8a16_kernel and gemv_w8a16_wholerow_kernel (the two instantiation families the 129 launches
-#: of the default workload, M=1, use): fetched + written bytes per launch, from the
-#: FETCH_SIZE and WRITE_SIZE runs summarised in profiles/gemv_w8a16_decode_model_M1.md
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28.51e6
+#: Summary of the rocprofv3 FETCH_SIZE / WRITE_SIZE runs of the default workload (M=1: the two
+#: instantiation families gemv_w8a16_kernel and gemv_w8a16_wholerow_kernel); it carries the
+#: line "roofline.traffic bytes per launch: <integer>", which is what `roofline.traffic` reports.
+TRAFFIC_PROFILE = ROOT / "profiles" / "gemv_w8a16_decode_model_M1.md"
+
+
+def measured_traffic_bytes_per_launch():
+    """HBM bytes per launch from the committed counter summary, or None when it is absent."""
+    import re
+    try:
+        m = re.search(r"roofline\.traffic bytes per launch:\s*([0-9][0-9,_]*)", TRAFFIC_PROFILE.read_text())
+    except OSError:
+        return None
+    return int(m.group(1).replace(",", "").replace("_", "")) if m else None
+
+
+def cpu_model() -> str:
+    try:
+        for line in Path("/proc/cpuinfo").read_text().splitlines():
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(budget_s: float, synth, torch) -> dict:
+    """The reference's CPU path on one decode layer (7 int8 weight-only GEMVs, M = 1, 101.1 MB), timed
+    on the host cores: torch eager evaluating backends/reference/__init__.py:93-95 --
+    ``dense = (wq.float() * scale[:, None]).to(bf16)``; ``y = F.linear(x, dense)`` -- *faithful*
+    (the dequantisation inside every call, as the reference does) and *hoisted* (dequantised once,
+    outside the clock), each at all cores and at one thread.  Median of up to 5 calls after up to 2
+    warm-ups per shape, fewer when the time budget (a quarter of ``budget_s`` per variant) runs
+    out.  The C oracle of the same path is reported beside it as a labelled extra."""
+    import statistics
+    import torch.nn.functional as F
+    gen = synth.generator(1234)
+    layer = []
+    for _, n_, k_ in synth.DECODE_LAYER:
+        q = synth.int8_weight(n_, k_, gen)
+        layer.append((q.wq, q.scale, synth.activations(1, k_, gen), synth.gemv_bytes(1, n_, k_)))
+    layer_bytes = sum(nb for *_, nb in layer)
+    all_cores = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0") or (os.cpu_count() or 1))))
+    prev_threads = torch.get_num_threads()
+
+    def leg(threads: int, hoisted: bool, budget: float):
+        torch.set_num_threads(threads)
+        t_start = time.perf_counter()
+        total, calls = 0.0, 0
+        for wq, sc, x, _ in layer:
+            dense = (wq.float() * sc[:, None]).to(torch.bfloat16) if hoisted else None
+            times = []
+            for i in range(7):
+                t0 = time.perf_counter()
+                d = dense if hoisted else (wq.float() * sc[:, None]).to(torch.bfloat16)
+                F.linear(x, d)
+                dt = time.perf_counter() - t0
+                if i >= 2 or time.perf_counter() - t_start > budget:
+                    times.append(dt)
+                if time.perf_counter() - t_start > budget and times:
+                    break
+            total += statistics.median(times)
+            calls += len(times)
+        return {"layer_ms": round(total * 1e3, 3), "GBps": round(layer_bytes / total / 1e9, 3), "threads": threads,
+                "timed_calls": calls}
+
+    per = budget_s / 4.0
+    variants = {}
+    for name, threads, hoisted in (("faithful_all_cores", all_cores, False), ("hoisted_all_cores", all_cores, True),
+                                   ("faithful_1_thread", 1, False), ("hoisted_1_thread", 1, True)):
+        variants[name] = leg(threads, hoisted, per)
+    torch.set_num_threads(prev_threads)
+
+    # the C oracle of the same path (fp64 inner loop, full dequantisation per call, OpenMP)
+    from oracle import oracle as orc
+    orc.set_num_threads(min(orc.num_threads(), all_cores))
+    ops = [(wq.numpy(), sc.numpy(), orc.bits(x)) for wq, sc, x, _ in layer]
+    orc.linear_qweight(*ops[1])
+    t0 = time.perf_counter()
+    for wq, sc, xb in ops:
+        orc.linear_qweight(wq, sc, xb)
+    c_dt = time.perf_counter() - t0
+
+    head = variants["faithful_all_cores"]
+    return {
+        "value": head["GBps"],
+        "unit": "GB/s",
+        "cores": head["threads"],
+        "kind": "port",
+        "sample": "one decode layer (q, k, v, o, gate, up, down: 7 int8 weight-only GEMVs, M=1, "
+                  f"{layer_bytes / 1e6:.1f} MB algorithmic) through torch eager restating the reference's CPU path "
+                  "(weight dequantised to bf16 inside every call, then F.linear), median per shape of "
+                  f"{head['timed_calls']} timed calls, all host cores",
+        "cpu_model": cpu_model(),
+        "os_cpu_count": os.cpu_count(),
+        "torch": torch.__version__,
+        "variants": variants,
+        "c_oracle_port": {"layer_ms": round(c_dt * 1e3, 3), "GBps": round(layer_bytes / c_dt / 1e9, 3),
+                          "threads": min(orc.num_threads(), all_cores),
+                          "note": "C restatement with an fp64 accumulator, dequantisation per call"},
+    }
 
 
 def parse_args():
@@ -58,6 +155,10 @@ def parse_args():
     ap.add_argument("--w4a8-prefill-only", action="store_true",
                     help="time only the W4A8 prefill GEMM (M=1024, N=25600, K=5120): the profiling target "
                          "for that kernel; prints its own JSON line")
+    ap.add_argument("--w4a8-decode-only", action="store_true",
+                    help="time only the W4A8 decode step (32 layers + lm_head at one row, one "
+                         "cmi_linear_w4a8_bf16 call per projection): the profiling target for the W4A8 decode "
+                         "kernels and the quantiser; prints its own JSON line")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (known traffic, for scaling HBM counters)")
     return ap.parse_args()
@@ -144,6 +245,65 @@ def main() -> int:
                           "w4a8_prefill_gemm_M1024_N25600_K5120": {
                               "us": round(t * 1e6, 2), "tops": round(tops, 1),
                               "frac_of_int8_peak": round(tops / INT8_PEAK_TOPS, 4)}}))
+        return 0
+
+    def w4a8_decode_step(rows: int, use_graph: bool, iters: int):
+        """The decode step of the same model with int4 group-128 weights (32 x {qkv, o, gate_up,
+        down} + lm_head, 1.84 GB of distinct packed weights), one cmi_linear_w4a8_bf16 call per
+        projection: the quantiser folded into the GEMV where that is the faster route, else two
+        launches.  Returns the result block for ``extra``."""
+        proj = []
+        xs_ = {k_: synth.activations(16, k_, gen) for k_ in (2560, 4096, 9728)}
+        for layer in range(LAYERS + 1):
+            for _, n_, k_ in (synth.DECODE_LAYER_FUSED if layer < LAYERS else (synth.LM_HEAD,)):
+                w = synth.int4_weight(n_, k_, gen)
+                d4 = torch.empty((n_, k_ // 2), dtype=torch.uint8, device=dev)
+                ds = torch.empty((n_, k_ // 128), dtype=torch.float32, device=dev)
+                _native.check(lib.cmi_w4_repack(ptr(w.packed), ptr(w.scale), ptr(d4), ptr(ds), n_, k_, 128,
+                                                cur_stream()), "repack")
+                torch.cuda.synchronize()
+                del w
+                proj.append((d4, ds, xs_[k_], torch.empty((16, n_), dtype=torch.bfloat16, device=dev), n_, k_))
+        nbytes = int(lib.cmi_linear_workspace_bytes(16, 9728))
+        work = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+        def step():
+            st = cur_stream()
+            for d4, ds, x, y, n_, k_ in proj:
+                rc = lib.cmi_linear_w4a8_bf16(ptr(d4), ptr(ds), ptr(x), ptr(y), rows, n_, k_, 128, ptr(work), nbytes, st)
+                if rc:
+                    _native.check(rc, "cmi_linear_w4a8_bf16")
+
+        runner, mode = step, "eager"
+        if use_graph:
+            step()
+            torch.cuda.synchronize()
+            want = [p_[3][:rows].clone() for p_ in proj[:4]] + [proj[-1][3][:rows].clone()]
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step()
+            for _ in range(2):
+                for p_ in proj:
+                    p_[3][:rows].zero_()
+                graph.replay()
+                torch.cuda.synchronize()
+                got = [p_[3][:rows] for p_ in proj[:4]] + [proj[-1][3][:rows]]
+                if not all(bool((a.view(torch.int16) == b_.view(torch.int16)).all()) for a, b_ in zip(want, got)):
+                    raise RuntimeError("HIP graph replay of the W4A8 step differs from the eager step")
+            runner, mode = graph.replay, "hipgraph"
+        t = timed(runner, iters, warm=2)
+        alg = sum(synth.w4_gemv_bytes(rows, n_, k_) for *_, n_, k_ in proj)
+        gbps = alg / t / 1e9
+        return {"ms_per_step": round(t * 1e3, 4), "GBps": round(gbps, 1), "launch": mode, "rows": rows,
+                "projections_per_step": len(proj), "algorithmic_bytes_per_step": alg,
+                "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                             "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                             "avg_projection_us": round(t / len(proj) * 1e6, 3),
+                             "algorithmic_bytes_per_projection": round(alg / len(proj))}}
+
+    if args.w4a8_decode_only:
+        out = {f"M{args.rows}": w4a8_decode_step(args.rows, not args.no_graph, args.steps)}
+        print(json.dumps({"metric": "W4A8 decode step HBM GB/s", "unit": "GB/s", "w4a8_decode_step": out}))
         return 0
 
     # ------------------------------------------------------------ headline: decode GEMVs
@@ -248,7 +408,7 @@ def main() -> int:
             "frac": round(value / HBM_PEAK_GBPS, 4),
             # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this same
             # command (summary under profiles/); it only describes the default workload
-            "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if (M == 1 and not args.no_graph) else None,
+            "traffic": measured_traffic_bytes_per_launch() if (M == 1 and not args.no_graph and not args.mfma) else None,
             "kernel": "gemv_w8a16_rows16_kernel" if args.mfma else ("gemv_w8a16_kernel + gemv_w8a16_wholerow_kernel" if M == 1 else "gemv_w8a16_kernel"),
             "avg_launch_us": round(step_s / n_launch * 1e6, 3),
             "algorithmic_bytes_per_launch": round(bytes_per_step / n_launch),
@@ -282,7 +442,57 @@ def main() -> int:
             per_shape[name] = {"us": round(t * 1e6, 2),
                                "GBps": round(synth.gemv_bytes(1, n_, k_) / t / 1e9, 1)}
         extra["decode_gemv_int8_M1_per_shape_eager"] = per_shape
+
+        # the same 129 projections through the table entry (backend.linear: Python adapter + ctypes +
+        # a fresh output tensor per call), eager and as a captured graph: what the host side costs
+        from coffin_amd import backend as _adapters
+        from coffin_amd.weights import QWeight as _QW
+        qws = [(_QW(wq, sc), x[0]) for wq, sc, x, *_ in launches]
+        def adapter_step():
+            for qw, x1 in qws:
+                _adapters.linear(qw, x1)
+        adapter_step()
+        torch.cuda.synchronize()
+        w0 = time.perf_counter()
+        for _ in range(5):
+            adapter_step()
+        host_s = (time.perf_counter() - w0) / 5          # enqueue time: the launches run behind it
+        t_eager = timed(adapter_step, 5)
+        ag = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(ag):
+            adapter_step()
+        t_graph = timed(ag.replay, max(3, args.steps // 2))
+        extra["decode_step_through_backend_linear_M1"] = {
+            "eager_ms": round(t_eager * 1e3, 4), "eager_GBps": round(step_bytes(1) / t_eager / 1e9, 1),
+            "host_enqueue_us_per_call": round(host_s / len(qws) * 1e6, 2),
+            "hipgraph_ms": round(t_graph * 1e3, 4), "hipgraph_GBps": round(step_bytes(1) / t_graph / 1e9, 1)}
+        del qws, ag
+
+        # q, k and v as three projections (2560 -> 4096 / 1024 / 1024) instead of the fused qkv: the
+        # 1024-row GEMVs are the smallest launches of the configuration
+        unf = {}
+        for name, n_, k_ in (("q_proj", 4096, 2560), ("k_proj", 1024, 2560), ("gate_proj", 9728, 2560)):
+            copies = max(8, int(1.2e9 // (n_ * k_)))
+            ws_ = [synth.int8_weight(n_, k_, gen) for _ in range(copies)]
+            y1 = torch.empty((1, n_), dtype=torch.bfloat16, device=dev)
+            def one(ws_=ws_, y1=y1, n_=n_, k_=k_):
+                st = cur_stream()
+                for q in ws_:
+                    lib.cmi_gemv_w8a16(ptr(q.wq), ptr(q.scale), ptr(x_by_k[k_]), ptr(y1), 1, n_, k_, st)
+            one()
+            torch.cuda.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                one()
+            t = timed(gr.replay, 5) / copies
+            unf[name] = {"us": round(t * 1e6, 2), "GBps": round(synth.gemv_bytes(1, n_, k_) / t / 1e9, 1)}
+            del ws_, gr
+        extra["decode_gemv_int8_M1_unfused_shapes_hipgraph"] = unf
         launches.clear()
+        torch.cuda.empty_cache()
+
+        # W4A8 decode step (int4 weights, per-token int8 activations), one and sixteen rows
+        extra["w4a8_decode_step"] = {f"M{m}": w4a8_decode_step(m, True, max(3, args.steps // 2)) for m in (1, 16)}
         torch.cuda.empty_cache()
 
         # W4A8 decode GEMV (quantiser + GEMV, as the adapter issues them)
@@ -473,34 +683,7 @@ def main() -> int:
 
     # ------------------------------------------------------------------ CPU baseline leg
     if args.cpu_seconds > 0:
-        from oracle import oracle as orc
-        cpu_gen = synth.generator(1234)
-        ops = []
-        for _, n_, k_ in synth.DECODE_LAYER:
-            q = synth.int8_weight(n_, k_, cpu_gen)
-            x = synth.activations(1, k_, cpu_gen)
-            ops.append((q.wq.numpy(), q.scale.numpy(), orc.bits(x), synth.gemv_bytes(1, n_, k_)))
-        threads = min(orc.num_threads(), int(os.environ.get("OMP_NUM_THREADS", "0") or orc.num_threads()))
-        orc.set_num_threads(threads)
-        for wq, sc, xb, _ in ops[:1]:
-            orc.linear_qweight(wq, sc, xb)
-        done, t0 = 0, time.perf_counter()
-        passes = 0
-        while time.perf_counter() - t0 < args.cpu_seconds:
-            for wq, sc, xb, nb in ops:
-                orc.linear_qweight(wq, sc, xb)
-                done += nb
-            passes += 1
-        dt = time.perf_counter() - t0
-        result["cpu_baseline"] = {
-            "value": round(done / dt / 1e9, 3),
-            "unit": "GB/s",
-            "cores": threads,
-            "kind": "port",
-            "sample": f"{passes} passes over one decode layer (7 int8 GEMVs, M=1, 101.1 MB) through the C "
-                      f"oracle of the torch reference path (full weight dequant per call, as the reference does), "
-                      f"{dt:.1f} s on the host cores",
-        }
+        result["cpu_baseline"] = cpu_baseline(args.cpu_seconds, synth, torch)
 
     print(json.dumps(result))
     return 0
