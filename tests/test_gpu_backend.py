@@ -343,3 +343,23 @@ def test_launches_follow_the_current_stream():
         got = backend.linear(q, x)
     side.synchronize()
     assert (got.view(torch.int16) == want.view(torch.int16)).all()
+
+
+def test_pre_quantised_directory_feeds_the_kernels(tmp_path, orc):
+    """A coffin-int8-kn-v1 / coffin-w4a8-kn-v1 directory read straight to the GPU gives weights the
+    adapters take as they are: same bits as the weights the directory was written from."""
+    import json
+    from safetensors.torch import save_file
+    from coffin_amd import quantized_load as ql
+    g = synth.generator()
+    q = synth.int8_weight(640, 2560, g)
+    key = "model.language_model.layers.0.mlp.down_proj.weight"
+    save_file({key: q.wq.t().contiguous(), key + "#scale": q.scale}, str(tmp_path / "quant-00001-of-00001.safetensors"))
+    (tmp_path / ql.INDEX_NAME).write_text(json.dumps({"format": ql.FORMAT_INT8, "weight_dtype": "bfloat16", "tensors": {
+        key: {"kind": "q8", "shape": [2560, 640], "scale_key": key + "#scale", "shard": "quant-00001-of-00001.safetensors"}}}))
+    w = ql.load(tmp_path, device=G.DEV)[key]
+    assert w.wq.device.type == "cuda" and w.wq.is_contiguous() and tuple(w.wq.shape) == (640, 2560)
+    x = synth.activations(3, 2560, g).to(G.DEV)
+    ref = QWeight(q.wq.to(G.DEV), q.scale.to(G.DEV))
+    assert (backend.linear_m(w, x).view(torch.int16) == backend.linear_m(ref, x).view(torch.int16)).all()
+    assert (backend.linear(w, x[0]).view(torch.int16) == backend.linear(ref, x[0]).view(torch.int16)).all()
