@@ -29,6 +29,7 @@ SIGNATURES: dict[str, list] = {
     "cmi_gemv_w8a16_mfma": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp],
     "cmi_w4_repack": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp],
     "cmi_gemv_w4a8": [_vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
+    "cmi_gemv_w4a16": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp],
     "cmi_gemv_w4a8_bf16": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cmi_gemm_w8a8": [_vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cmi_gemm_w4a8": [_vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],

@@ -73,6 +73,13 @@ W8A8_VERIFY = os.environ.get("COFFIN_AMD_W8A8_VERIFY", "0").strip() == "1"
 #: independent of its batch), static batches of 4-16 requests run 1.05-2.8 times faster, and
 #: single-stream decode pays for it (7.9 us instead of 6.3 us for 2560 -> 9728).  A deployment choice.
 BATCH_MFMA = os.environ.get("COFFIN_AMD_BATCH_MFMA", "0").strip() == "1"
+#: int4 weights are answered with W4A8 arithmetic (per-token int8 activations), which is what coffin
+#: runs on its native backends.  ``COFFIN_AMD_W4A16=1`` keeps the activations unquantised instead for
+#: decode-sized calls (up to ``W4A16_MAX_ROWS`` rows, K <= 10240): the int4 weight-only GEMV, i.e. the
+#: arithmetic of the reference's torch path for an int4 weight (backends/reference/__init__.py:93-95)
+#: up to fp32 summation order; one launch per row, so it is meant for single-stream decode.
+W4A16 = os.environ.get("COFFIN_AMD_W4A16", "0").strip() == "1"
+W4A16_MAX_ROWS = 4
 #: Rows from which the matrix-pipe GEMV beats the dot-product one (measured on every layer shape).
 MFMA_MIN_ROWS = 3
 def _vp(address: int) -> int:
@@ -314,6 +321,18 @@ def _rows_w4(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> N
         _native.check(rc, "linear_w4a8_bf16")
 
 
+def _rows_w4a16(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> None:
+    """int4 weight-only GEMV on unquantised activations, one launch per row."""
+    n, k = rec.n, rec.k
+    lib = _native.load()
+    stream = _stream()
+    x0, y0 = act.data_ptr(), out.data_ptr()
+    for r in range(rows):
+        rc = lib.cmi_gemv_w4a16(rec.a, rec.b, x0 + r * k * 2, y0 + r * n * 2, n, k, rec.gs, stream)
+        if rc:
+            _native.check(rc, "gemv_w4a16")
+
+
 # ------------------------------------------------------------------ dispatch
 
 def _dense(w, x: torch.Tensor) -> torch.Tensor:
@@ -365,7 +384,10 @@ def _project(w, x: torch.Tensor, prefill: bool, min_rows: int = PREFILL_MIN_ROWS
     if rows == 0:
         return out
     if rec.kind == 4:
-        _rows_w4(rec, act, rows, out)
+        if W4A16 and rows <= W4A16_MAX_ROWS and rec.k <= 10240:
+            _rows_w4a16(rec, act, rows, out)
+        else:
+            _rows_w4(rec, act, rows, out)
     elif prefill and rows >= min_rows:
         _gemm_q8(rec, act, rows, out)
     else:

@@ -106,6 +106,16 @@ int cmi_w4_repack(const uint8_t *packed, const float *scale, uint8_t *w4, float 
 int cmi_gemv_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs,
                   void *y, int32_t *group_acc, int M, int N, int K, int gs, void *stream);
 
+/* int4 weight-only GEMV on *unquantised* bf16 activations (W4A16), one activation row, on the
+ * re-laid-out weight:
+ *   y[n] = bf16( sum_g ws[n,g] * sum_{k in g} (code - 8) * x[k] ),  fp32 sums in an order that
+ * depends on K only.  K % 128 == 0, gs == 128, K <= 10240.  This is what the reference's torch
+ * path computes for an int4 weight (backends/reference/__init__.py:93-95 with
+ * w4a8_weights.py:96-99: no activation quantisation) up to fp32 summation order, and stands where
+ * gemv_kn_w4 is bound (backends/corex/kernels/gemv.cu:1918-1930, 1935-1975). */
+int cmi_gemv_w4a16(const uint8_t *w4, const float *ws, const void *x, void *y, int N, int K,
+                   int gs, void *stream);
+
 /* cmi_gemv_w4a8 with the activation quantiser folded in, 1 <= M <= 4: x is bf16
  * [M,K]; every workgroup quantises it on the fly with the arithmetic of
  * cmi_quant_act_i8 (same bits), so one launch replaces quant_act_i8 + w4a8_gemv

@@ -98,3 +98,11 @@ def gemv_w4a8_bf16(w4, ws, x, k, gs=128):
     _native.check(_native.load().cmi_gemv_w4a8_bf16(ptr(w4), ptr(ws), ptr(x), ptr(y), ptr(gacc), ptr(xq),
                                                     ptr(xs), m, n, k, gs, stream()), "gemv_w4a8_bf16")
     return gacc, y, xq, xs
+
+
+def gemv_w4a16(w4, ws, x, k, gs=128):
+    """int4 weight-only GEMV on one unquantised bf16 row x [K] -> y [N]."""
+    n = w4.shape[0]
+    y = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+    _native.check(_native.load().cmi_gemv_w4a16(ptr(w4), ptr(ws), ptr(x), ptr(y), n, k, gs, stream()), "gemv_w4a16")
+    return y

@@ -147,3 +147,58 @@ def test_w4a8_kernels_stay_within_quantisation_error_of_the_unquantised_referenc
     err = np.sqrt(((got - ref) ** 2).mean())
     assert err <= W4_VS_UNQUANTISED_RMS * rms, (err / rms)
     assert err >= 1e-3 * rms            # and they do differ: the reference does not quantise x
+
+
+# ------------------------------------------------------------- W4A16 (int4 weight-only) GEMV
+
+@pytest.mark.parametrize("n,k", [(9728, 2560), (2560, 9728), (2560, 4096), (6144, 2560), (37, 128), (1001, 384),
+                                 (300, 2048), (64, 10240), (5, 6272)])
+def test_gemv_w4a16_against_the_exact_sum_and_the_unquantised_reference(orc, n, k):
+    """The int4 weight-only GEMV is a floating-point path (fp32 sums in the kernel's own order):
+    held to the exact value of sum_k (code - 8) * scale * x within its final bf16 rounding plus
+    fp32 accumulation noise, and to the reference's torch statement for an int4 weight
+    (dequantised to bf16, bf16 product; orc.linear_w4weight) within 1e-2 of the output RMS plus
+    one bf16 step -- the bound of the int8 weight-only path."""
+    g = synth.generator(1234)
+    w = synth.int4_weight(n, k, g)
+    x = synth.activations(1, k, g)
+    w4, ws = G.w4_repack(w.packed.to(G.DEV), w.scale.to(G.DEV), k)
+    y = G.gemv_w4a16(w4, ws, x[0].contiguous().to(G.DEV), k)
+    got = y.float().cpu().numpy().astype(np.float64)
+    dense = orc.w4_dequant_f32(w.packed.numpy(), w.scale.numpy(), k, 128).astype(np.float64)     # exact: 4-bit x fp16 scale
+    exact = dense @ x[0].float().numpy().astype(np.float64)
+    rms = np.sqrt((exact ** 2).mean()) + 1e-30
+    assert (np.abs(got - exact) <= np.abs(exact) * 2.0 ** -8 * 1.01 + 2e-5 * rms).all()
+    ref = orc.bf16_to_f32(orc.linear_w4weight(w.packed.numpy(), w.scale.numpy(), G.bits(x), k, 128))[0]
+    assert (np.abs(got - ref) <= 1e-2 * rms + np.abs(ref) * 2.0 ** -7).all()
+    assert np.sqrt(((got - exact) ** 2).mean()) / rms < 3e-3
+    # zero activations give exact zeros; a power-of-two scaling of the group scales scales exactly
+    assert (G.gemv_w4a16(w4, ws, torch.zeros(k, dtype=torch.bfloat16, device=G.DEV), k).float() == 0).all()
+    y2 = G.gemv_w4a16(w4, ws * 4.0, x[0].contiguous().to(G.DEV), k)
+    assert (y2.float() == y.float() * 4.0).all()
+
+
+def test_w4a16_switch_in_the_adapter(monkeypatch, orc):
+    from coffin_amd import backend
+    from coffin_amd.weights import W4A8Weight
+    g = synth.generator(3)
+    w = synth.int4_weight(512, 2560, g)
+    wd = W4A8Weight(w.packed.to(G.DEV), w.scale.to(G.DEV), k=2560)
+    x = synth.activations(3, 2560, g).to(G.DEV)
+    quantised = backend.linear_m(wd, x)
+    monkeypatch.setattr(backend, "W4A16", True)
+    unquantised = backend.linear_m(wd, x)
+    w4, ws = G.w4_repack(wd.packed, wd.scale, 2560)
+    for r in range(3):
+        assert (unquantised[r].view(torch.int16) == G.gemv_w4a16(w4, ws, x[r].contiguous(), 2560).view(torch.int16)).all()
+    assert (backend.linear(wd, x[1]).view(torch.int16) == unquantised[1].view(torch.int16)).all()
+    # the two arithmetics differ by the activation-quantisation error, no more
+    diff = (unquantised.float() - quantised.float()).abs()
+    rms = unquantised.float().pow(2).mean().sqrt()
+    assert 1e-4 * rms < diff.mean() < 2e-2 * rms
+    # wider batches keep W4A8
+    x8 = synth.activations(8, 2560, g).to(G.DEV)
+    monkeypatch.setattr(backend, "W4A16", False)
+    want8 = backend.linear_m(wd, x8)
+    monkeypatch.setattr(backend, "W4A16", True)
+    assert (backend.linear_m(wd, x8).view(torch.int16) == want8.view(torch.int16)).all()
