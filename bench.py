@@ -159,6 +159,9 @@ def parse_args():
                     help="time only the W4A8 decode step (32 layers + lm_head at one row, one "
                          "cmi_linear_w4a8_bf16 call per projection): the profiling target for the W4A8 decode "
                          "kernels and the quantiser; prints its own JSON line")
+    ap.add_argument("--quant-only", action="store_true",
+                    help="time only the per-token quantiser (8192 x 2560, 2048 x 9728, 16 x 9728 and 1 x 2560 rows): "
+                         "the profiling target for quant_act_i8; prints its own JSON line")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (known traffic, for scaling HBM counters)")
     return ap.parse_args()
@@ -300,6 +303,19 @@ def main() -> int:
                              "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
                              "avg_projection_us": round(t / len(proj) * 1e6, 3),
                              "algorithmic_bytes_per_projection": round(alg / len(proj))}}
+
+    if args.quant_only:
+        out = {}
+        for m, k_ in ((8192, 2560), (2048, 9728), (16, 9728), (1, 2560)):
+            x = synth.activations(m, k_, gen, outliers=True)
+            xq = torch.empty((m, k_), dtype=torch.int8, device=dev)
+            xs = torch.empty(m, dtype=torch.float32, device=dev)
+            t = timed(lambda: lib.cmi_quant_act_i8(ptr(x), ptr(xq), ptr(xs), m, k_, cur_stream()), args.steps, args.warmup)
+            gbps = synth.quant_bytes(m, k_) / t / 1e9
+            out[f"M{m}_K{k_}"] = {"us": round(t * 1e6, 2), "GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4),
+                                  "algorithmic_bytes": synth.quant_bytes(m, k_)}
+        print(json.dumps({"metric": "per-token int8 quantiser HBM GB/s", "unit": "GB/s", "quant_act_i8": out}))
+        return 0
 
     if args.w4a8_decode_only:
         out = {f"M{args.rows}": w4a8_decode_step(args.rows, not args.no_graph, args.steps)}
