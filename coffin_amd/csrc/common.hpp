@@ -21,6 +21,7 @@ int reserve_lds(const void *kernel, int bytes, std::atomic<uint64_t> &devices, c
 // Kernel-selection overrides (cmi_set_option / CMI_GEMM_TILE, CMI_GEMV_WHOLEROW read once).
 int option_gemm_tile();      // 0 = the library chooses, else 64 / 128 / 256 / 320
 int option_gemv_wholerow();  // -1 = the library chooses, 0 = never, 1 = where it can
+int option_w4_decode_waves();  // 0 = the library chooses, else 4 or 16 wavefronts per workgroup
 
 #define CMI_REQUIRE(cond, code, ...)                 \
     do {                                             \

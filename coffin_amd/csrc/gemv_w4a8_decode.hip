@@ -27,9 +27,10 @@ using namespace cmi;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int GS = 128;
-constexpr int ROWS_PER_WAVE = 4, WAVES = 4, ROWS_PER_BLOCK = ROWS_PER_WAVE * WAVES;
-constexpr int XV = 5;           // 16-byte bf16 vectors per thread and activation row: K <= 5*256*8
-constexpr int MAX_K = XV * 256 * 8;
+constexpr int ROWS_PER_WAVE = 4;
+constexpr int MAX_K = 10240;
+// 16-byte bf16 vectors per thread and activation row so that a workgroup of WV wavefronts carries K <= MAX_K
+constexpr int xv_of(int wv) { return (MAX_K / 8 + 64 * wv - 1) / (64 * wv); }
 
 struct Args {
     const uint8_t *w4;
@@ -48,9 +49,13 @@ struct Args {
 struct Lds {
     int xq, xsum, wsc, sums, xs, part, total;
 };
-__host__ __device__ inline Lds lds_layout(int mt, int K, bool ksplit) {
+// Weight rows of a workgroup of wv wavefronts: every wavefront four rows of its own, or (ksplit)
+// every four wavefronts four shared rows.
+__host__ __device__ constexpr int rows_per_block(int wv, bool ksplit) { return ROWS_PER_WAVE * (ksplit ? wv / 4 : wv); }
+
+__host__ __device__ inline Lds lds_layout(int mt, int K, bool ksplit, int wv) {
     const int G = K / GS;
-    const int rows = ksplit ? ROWS_PER_WAVE : ROWS_PER_BLOCK;
+    const int rows = rows_per_block(wv, ksplit);
     Lds l;
     l.xq = 0;
     l.xsum = l.xq + mt * K;                           // int8 [mt][K]
@@ -58,7 +63,7 @@ __host__ __device__ inline Lds lds_layout(int mt, int K, bool ksplit) {
     l.sums = l.wsc + ((rows * G * 4 + 15) & ~15);     // float [rows][G]
     l.xs = l.sums + rows * ((G + 3) & ~3) * mt * 4;   // int32 [rows][mt][G padded to 4]
     l.part = l.xs + 16 * 4;                           // float [mt] (padded to 16)
-    l.total = l.part + 16 * 4 * 4;                    // float [mt][4]
+    l.total = l.part + 4 * wv * 4;                    // float [mt][wv], mt <= 4
     return l;
 }
 
@@ -67,11 +72,14 @@ __host__ __device__ inline Lds lds_layout(int mt, int K, bool ksplit) {
 //         256-byte piece each (few, long rows: more workgroups, same bytes in flight);
 //         otherwise each wavefront owns four rows of its own.
 // PREQ:   activations arrive already quantised (a.xq, a.xs) instead of as bf16.
-template <int M, int NL, bool KSPLIT, bool PREQ>
-__global__ void __launch_bounds__(256)
+// WV:     wavefronts per workgroup, 4 or 16.  Every workgroup quantises the whole activation row for
+//         itself; sixteen wavefronts do that once for four times as many weight rows.
+template <int M, int NL, bool KSPLIT, bool PREQ, int WV>
+__global__ void __launch_bounds__(64 * WV)
 gemv_w4a8_decode_kernel(const Args a) {
+    constexpr int THREADS = 64 * WV;
     extern __shared__ __align__(16) uint8_t lds[];
-    const Lds L = lds_layout(M, a.K, KSPLIT);
+    const Lds L = lds_layout(M, a.K, KSPLIT, WV);
     int8_t *xq_lds = reinterpret_cast<int8_t *>(lds + L.xq);
     int32_t *xsum_lds = reinterpret_cast<int32_t *>(lds + L.xsum);
     float *ws_lds = reinterpret_cast<float *>(lds + L.wsc);
@@ -79,16 +87,19 @@ gemv_w4a8_decode_kernel(const Args a) {
     float *xs_lds = reinterpret_cast<float *>(lds + L.xs);
     float *part = reinterpret_cast<float *>(lds + L.part);
 
-    constexpr int RPB = KSPLIT ? ROWS_PER_WAVE : ROWS_PER_BLOCK;
+    constexpr int RPB = rows_per_block(WV, KSPLIT);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int q16 = lane & 15, r = lane >> 4;
     const int n0 = blockIdx.x * RPB;
-    const int nrow = min(n0 + (KSPLIT ? 0 : wave * ROWS_PER_WAVE) + r, a.N - 1);
+    // first row of this wavefront inside the workgroup, and (ksplit) which quarter of each row it takes
+    const int wrow0 = (KSPLIT ? (wave >> 2) : wave) * ROWS_PER_WAVE;
+    const int kpart = wave & 3;
+    const int nrow = min(n0 + wrow0 + r, a.N - 1);
     const int row_bytes = a.K / 2;
     const int nchunks = a.K / 32;
 
     // 1. activations first (memory answers in request order and they are needed first)
-    constexpr int XVN = PREQ ? 3 : XV;  // 16-byte vectors per thread and row
+    constexpr int XVN = PREQ ? (xv_of(WV) + 1) / 2 : xv_of(WV);  // 16-byte vectors per thread and row
     const int xvecs = PREQ ? a.K / 16 : a.K / 8;
     uint4 v[M][XVN];
 #pragma unroll
@@ -98,32 +109,32 @@ gemv_w4a8_decode_kernel(const Args a) {
                                : reinterpret_cast<const uint4 *>(a.x + (size_t)mrow * a.K);
 #pragma unroll
         for (int j = 0; j < XVN; ++j) {
-            const int idx = threadIdx.x + j * 256;
+            const int idx = threadIdx.x + j * THREADS;
             v[m][j] = idx < xvecs ? xg[idx] : make_uint4(0, 0, 0, 0);
         }
     }
     // 2. the per-group scales of the workgroup's rows (contiguous in memory), into registers
     // for now: they must not be waited for after the weights, which return in request order
-    constexpr int WSV = 5;  // floats per thread: 16 rows x G <= 16 x 80
+    constexpr int WSV = (RPB * (MAX_K / GS) + THREADS - 1) / THREADS;  // floats per thread: RPB rows x G <= 80
     const int ws_total = min(RPB, a.N - n0) * a.G;
     float wsreg[WSV];
     {
         const float *src = a.ws + (size_t)n0 * a.G;
 #pragma unroll
         for (int i = 0; i < WSV; ++i) {
-            const int idx = threadIdx.x + i * 256;
+            const int idx = threadIdx.x + i * THREADS;
             wsreg[i] = idx < ws_total ? src[idx] : 0.f;
         }
     }
     // 3. every weight byte this wavefront is responsible for
     const u32x4 *wrow = reinterpret_cast<const u32x4 *>(a.w4 + (size_t)nrow * row_bytes);
-    auto chunk_of = [&](int j) { return (KSPLIT ? j * 4 + wave : j) * 16 + q16; };  // 16-byte chunk = 32 k
+    auto chunk_of = [&](int j) { return (KSPLIT ? j * 4 + kpart : j) * 16 + q16; };  // 16-byte chunk = 32 k
     u32x4 w[NL];
 #pragma unroll
     for (int j = 0; j < NL; ++j) w[j] = __builtin_nontemporal_load(wrow + min(chunk_of(j), nchunks - 1));
 #pragma unroll
     for (int i = 0; i < WSV; ++i) {
-        const int idx = threadIdx.x + i * 256;
+        const int idx = threadIdx.x + i * THREADS;
         if (idx < ws_total) ws_lds[idx] = wsreg[i];
     }
 
@@ -134,8 +145,8 @@ gemv_w4a8_decode_kernel(const Args a) {
             if (threadIdx.x == 0) xs_lds[m] = a.xs[m < a.M ? m : a.M - 1];
 #pragma unroll
             for (int j = 0; j < XVN; ++j) {
-                if (j * 256 >= xvecs) break;  // uniform
-                const int idx = threadIdx.x + j * 256;
+                if (j * THREADS >= xvecs) break;  // uniform
+                const int idx = threadIdx.x + j * THREADS;
                 const uint4 q = v[m][j];
                 int s8 = __builtin_amdgcn_sdot4((int)q.x, 0x01010101, 0, false);
                 s8 = __builtin_amdgcn_sdot4((int)q.y, 0x01010101, s8, false);
@@ -154,15 +165,16 @@ gemv_w4a8_decode_kernel(const Args a) {
             float amax = 0.f;
 #pragma unroll
             for (int j = 0; j < XVN; ++j)
-                if (j * 256 < xvecs) amax = absmax8(v[m][j], amax);  // uniform: skip vectors past K
+                if (j * THREADS < xvecs) amax = absmax8(v[m][j], amax);  // uniform: skip vectors past K
             amax = wave_max_to_lane63(amax);
-            if (lane == 63) part[m * 4 + wave] = amax;
+            if (lane == 63) part[m * WV + wave] = amax;
         }
         __syncthreads();
 #pragma unroll
         for (int m = 0; m < M; ++m) {
-            const float amax =
-                fmaxf(fmaxf(part[m * 4], part[m * 4 + 1]), fmaxf(part[m * 4 + 2], part[m * 4 + 3]));
+            float amax = part[m * WV];
+#pragma unroll
+            for (int w = 1; w < WV; ++w) amax = fmaxf(amax, part[m * WV + w]);
             const RowScale rs = row_scale(amax);
             const float sc = rs.sc;
             if (threadIdx.x == 0) {
@@ -171,8 +183,8 @@ gemv_w4a8_decode_kernel(const Args a) {
             }
 #pragma unroll
             for (int j = 0; j < XVN; ++j) {
-                if (j * 256 >= xvecs) break;  // uniform
-                const int idx = threadIdx.x + j * 256;
+                if (j * THREADS >= xvecs) break;  // uniform
+                const int idx = threadIdx.x + j * THREADS;
                 const uint2 q = quant8(v[m][j], rs);
                 // four consecutive vectors (adjacent lanes) = one chunk
                 int s8 = __builtin_amdgcn_sdot4((int)q.x, 0x01010101, 0, false);
@@ -193,10 +205,10 @@ gemv_w4a8_decode_kernel(const Args a) {
     // 5. integer group sums
     // [row of the wavefront][m][group]: the lane that walks a row's groups reads them 16 bytes at a time
     const int Gpad = (a.G + 3) & ~3;
-    int32_t *wsums = sums + (KSPLIT ? 0 : wave * (Gpad * ROWS_PER_WAVE * M));
+    int32_t *wsums = sums + (wrow0 / ROWS_PER_WAVE) * (Gpad * ROWS_PER_WAVE * M);
 #pragma unroll
     for (int j = 0; j < NL; ++j) {
-        if ((KSPLIT ? j * 4 + wave : j) * 16 >= nchunks) break;  // uniform per wavefront
+        if ((KSPLIT ? j * 4 + kpart : j) * 16 >= nchunks) break;  // uniform per wavefront
         const int c = chunk_of(j);
         const bool live = c < nchunks;
         const int cs = live ? c : nchunks - 1;
@@ -222,7 +234,7 @@ gemv_w4a8_decode_kernel(const Args a) {
     }
     if constexpr (KSPLIT) {
         __syncthreads();
-        if (wave != 0) return;
+        if (kpart != 0) return;
     } else {
         // the group sums below were written by this wavefront itself
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -236,13 +248,13 @@ gemv_w4a8_decode_kernel(const Args a) {
         for (int i = lane; i < n_out; i += 64) {
             const int rm = i / a.G, g = i - rm * a.G;
             const int rr = rm / M, m = rm - rr * M;
-            const int n = n0 + (KSPLIT ? 0 : wave * ROWS_PER_WAVE) + rr;
+            const int n = n0 + wrow0 + rr;
             if (n < a.N && m < a.M) a.group_acc[((size_t)m * a.G + g) * a.N + n] = wsums[rm * Gpad + g];
         }
     }
     if (lane < ROWS_PER_WAVE * M) {
         const int rr = lane / M, m = lane - rr * M;
-        const int brow = (KSPLIT ? 0 : wave * ROWS_PER_WAVE) + rr;  // row within the workgroup
+        const int brow = wrow0 + rr;  // row within the workgroup
         const int n = n0 + brow;
         if (n < a.N && m < a.M) {
             const float *wsn = ws_lds + brow * a.G;
@@ -286,34 +298,51 @@ gemv_w4a8_decode_kernel(const Args a) {
     }
 }
 
-template <int M, int NL, bool KSPLIT, bool PREQ>
+template <int M, int NL, bool KSPLIT, bool PREQ, int WV>
 int launch(const Args &a, hipStream_t st) {
-    const Lds L = lds_layout(M, a.K, KSPLIT);
+    const Lds L = lds_layout(M, a.K, KSPLIT, WV);
     if (L.total > 64 * 1024) return CMI_E_UNSUPPORTED;
-    constexpr int RPB = KSPLIT ? ROWS_PER_WAVE : ROWS_PER_BLOCK;
+    constexpr int RPB = rows_per_block(WV, KSPLIT);
     const dim3 grid((a.N + RPB - 1) / RPB);
-    gemv_w4a8_decode_kernel<M, NL, KSPLIT, PREQ><<<grid, dim3(256), L.total, st>>>(a);
+    gemv_w4a8_decode_kernel<M, NL, KSPLIT, PREQ, WV><<<grid, dim3(64 * WV), L.total, st>>>(a);
     return check_launch("cmi_gemv_w4a8");
+}
+
+template <int M, bool PREQ, int WV>
+int dispatch_wv(const Args &a, hipStream_t st, bool ksplit) {
+    const int pieces = (a.K + 511) / 512;  // 256-byte pieces per weight row
+    if (ksplit) {
+        const int nl = (pieces + 3) / 4;
+        if (nl <= 2) return launch<M, 2, true, PREQ, WV>(a, st);
+        if (nl <= 5) return launch<M, 5, true, PREQ, WV>(a, st);
+        return CMI_E_UNSUPPORTED;
+    }
+    if (pieces <= 5) return launch<M, 5, false, PREQ, WV>(a, st);
+    if (pieces <= 8) return launch<M, 8, false, PREQ, WV>(a, st);
+    if (pieces <= 10) return launch<M, 10, false, PREQ, WV>(a, st);
+    if (pieces <= 20) return launch<M, 20, false, PREQ, WV>(a, st);
+    return CMI_E_UNSUPPORTED;
 }
 
 template <int M, bool PREQ>
 int dispatch(const Args &a, hipStream_t st) {
-    const int pieces = (a.K + 511) / 512;  // 256-byte pieces per weight row
-    // few rows: share each row among the four wavefronts so that the grid still covers the chip
-    // (below one workgroup per compute unit; at 384 workgroups whole rows per wavefront are faster:
-    // 2560 -> 6144 takes 5.1 us against 6.3)
-    const bool ksplit = (a.N + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK < 256 && pieces >= 4;
-    if (ksplit) {
-        const int nl = (pieces + 3) / 4;
-        if (nl <= 2) return launch<M, 2, true, PREQ>(a, st);
-        if (nl <= 5) return launch<M, 5, true, PREQ>(a, st);
-        return CMI_E_UNSUPPORTED;
+    const int pieces = (a.K + 511) / 512;
+    // few rows: share each row among four wavefronts so that the grid still covers the chip
+    // (below one 16-row workgroup per compute unit; at 384 workgroups whole rows per wavefront are
+    // faster: 2560 -> 6144 takes 5.1 us against 6.3)
+    const bool ksplit = (a.N + 15) / 16 < 256 && pieces >= 4;
+    // Quantising from bf16, every workgroup redoes the whole activation row: with sixteen
+    // wavefronts a workgroup does it for four times the weight rows.  That pays where rows are
+    // shared among wavefronts (few long rows, each workgroup quantising a long row for four
+    // weight rows: 4096 -> 2560 4.8 -> 4.2 us, 9728 -> 2560 8.6 -> 8.2 us); with whole rows per
+    // wavefront the wider barriers cost more than the quantisation saved (2560 -> 19456
+    // 8.5 -> 9.9 us).  One bf16 row only (the decode case).
+    const int opt = option_w4_decode_waves();
+    const bool wide = opt ? opt == 16 : (!PREQ && M == 1 && ksplit);
+    if constexpr (M == 1) {
+        if (wide) return dispatch_wv<M, PREQ, 16>(a, st, ksplit);
     }
-    if (pieces <= 5) return launch<M, 5, false, PREQ>(a, st);
-    if (pieces <= 8) return launch<M, 8, false, PREQ>(a, st);
-    if (pieces <= 10) return launch<M, 10, false, PREQ>(a, st);
-    if (pieces <= 20) return launch<M, 20, false, PREQ>(a, st);
-    return CMI_E_UNSUPPORTED;
+    return dispatch_wv<M, PREQ, 4>(a, st, ksplit);
 }
 
 }  // namespace

@@ -52,6 +52,7 @@ namespace {
 constexpr int UNREAD = INT32_MIN;
 std::atomic<int> g_gemm_tile{UNREAD};      // 0 = the library chooses
 std::atomic<int> g_gemv_wholerow{UNREAD};  // -1 = the library chooses, 0 = never, 1 = where it can
+std::atomic<int> g_w4_decode_waves{0};     // 0 = the library chooses, 4 or 16 wavefronts per workgroup
 
 bool valid_gemm_tile(int v) { return v == 0 || v == 64 || v == 128 || v == 256 || v == 320; }
 bool valid_wholerow(int v) { return v >= -1 && v <= 1; }
@@ -87,6 +88,8 @@ int option_gemv_wholerow() {
     return v;
 }
 
+int option_w4_decode_waves() { return g_w4_decode_waves.load(std::memory_order_relaxed); }
+
 }  // namespace cmi
 
 extern "C" int cmi_set_option(const char *name, int value) {
@@ -102,6 +105,12 @@ extern "C" int cmi_set_option(const char *name, int value) {
         CMI_REQUIRE(valid_wholerow(value), CMI_E_ARG,
                     "cmi_set_option: gemv_wholerow=%d, expected -1 (library's choice), 0 or 1", value);
         g_gemv_wholerow.store(value, std::memory_order_relaxed);
+        return CMI_OK;
+    }
+    if (!strcmp(name, "w4_decode_waves")) {
+        CMI_REQUIRE(value == 0 || value == 4 || value == 16, CMI_E_ARG,
+                    "cmi_set_option: w4_decode_waves=%d, expected 0 (library's choice), 4 or 16", value);
+        g_w4_decode_waves.store(value, std::memory_order_relaxed);
         return CMI_OK;
     }
     return fail(CMI_E_ARG, "cmi_set_option: unknown option '%s'", name);

@@ -40,7 +40,9 @@ int cmi_abi_version(void);
  *   "gemm_tile"     0 (the library chooses) | 64 | 128 | 256 | 320: block tile of cmi_gemm_w8a8 /
  *                   cmi_gemm_w4a8 (non-zero also bypasses their few-row routes);
  *   "gemv_wholerow" -1 (the library chooses) | 0 (never) | 1: the one-wavefront-per-weight-row
- *                   kernel of cmi_gemv_w8a16.
+ *                   kernel of cmi_gemv_w8a16;
+ *   "w4_decode_waves" 0 (the library chooses) | 4 | 16: wavefronts per workgroup of the W4A8
+ *                   decode GEMV (one bf16 or quantised row).
  * The environment variables CMI_GEMM_TILE and CMI_GEMV_WHOLEROW give the initial values; they are
  * read once, at the first call that needs them.  Unknown names or values: CMI_E_ARG.  Every choice
  * gives the same bits. */

@@ -420,9 +420,12 @@ def test_gemv_w4a8_bit_exact(orc, m, n, k):
 @pytest.mark.parametrize("m,n,k", [(1, 9728, 2560), (1, 2560, 9728), (4, 512, 256), (2, 333, 1280),
                                    (3, 7, 128), (4, 6144, 2560), (1, 2560, 4096), (4, 2560, 9728),
                                    (2, 640, 16384), (1, 256, 10240), (3, 100, 7680), (4, 8200, 128)])
-def test_gemv_w4a8_bf16_fused_quantiser_bit_exact(orc, m, n, k):
+@pytest.mark.parametrize("waves", [0, 4, 16])
+def test_gemv_w4a8_bf16_fused_quantiser_bit_exact(orc, m, n, k, waves):
     """One launch from bf16 activations: the quantised rows, the scales, the group
-    sums and the output all carry the bits of quantiser + GEMV run separately."""
+    sums and the output all carry the bits of quantiser + GEMV run separately -- with four and
+    with sixteen wavefronts per workgroup of the decode kernel (one-row calls)."""
+    G.set_option("w4_decode_waves", waves)
     g = seeded()
     w = synth.int4_weight(n, k, g)
     x = synth.activations(m, k, g, outliers=True)
