@@ -40,31 +40,43 @@ __device__ __forceinline__ RowScale row_scale(float absmax) {
     return s;
 }
 
-__device__ __forceinline__ uint32_t quant1(float x, const RowScale &s) {
-    float t;
+// 1.5 * 2^23: q + MAGIC has a unit in the last place of 1 for |q| < 2^22, so the sum is q rounded to
+// the nearest integer (ties to even) and its low mantissa bits are that integer in two's complement.
+constexpr float ROUND_MAGIC = 12582912.0f;
+
+// The quantised value of one element in the LOW BYTE of the result (the other bytes are not
+// zero: callers pick the byte out with a permute or a mask).  Finite rows: corrected quotient,
+// rounding and narrowing in one addition, no clamp -- |x / scale| <= 127 up to one rounding, so
+// the rounded value cannot leave [-127, 127] (part of the exhaustive CPU check).  Rows without a
+// finite scale divide, round and clamp as the reference statement does.
+__device__ __forceinline__ uint32_t quant1_lowbyte(float x, const RowScale &s) {
     if (s.rc != 0.f) {
         const float q0 = __fmul_rn(x, s.rc);
         const float e = __fmaf_rn(-q0, s.sc, x);
-        t = __fmaf_rn(e, s.rc, q0);
-    } else {
-        t = __fdiv_rn(x, s.sc);
+        const float t = __fmaf_rn(e, s.rc, q0);
+        return __float_as_uint(__fadd_rn(t, ROUND_MAGIC));
     }
-    float q = rintf(t);
+    float q = rintf(__fdiv_rn(x, s.sc));
     q = fminf(fmaxf(q, -127.f), 127.f);
-    return (uint32_t)((int)q) & 0xffu;
+    return (uint32_t)((int)q);
 }
+
+__device__ __forceinline__ uint32_t quant1(float x, const RowScale &s) { return quant1_lowbyte(x, s) & 0xffu; }
 
 __device__ __forceinline__ uint2 quant8(const uint4 &v, const RowScale &s) {
     const uint32_t w[4] = {v.x, v.y, v.z, v.w};
     uint32_t b[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        b[2 * i] = quant1(bf16_bits_to_f32(w[i] & 0xffffu), s);
-        b[2 * i + 1] = quant1(__uint_as_float(w[i] & 0xffff0000u), s);
+        b[2 * i] = quant1_lowbyte(bf16_bits_to_f32(w[i] & 0xffffu), s);
+        b[2 * i + 1] = quant1_lowbyte(__uint_as_float(w[i] & 0xffff0000u), s);
     }
+    // low bytes of four results -> one dword: two permutes gather pairs, a third joins them
     uint2 o;
-    o.x = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
-    o.y = b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24);
+    o.x = __builtin_amdgcn_perm(__builtin_amdgcn_perm(b[3], b[2], 0x0c0c0400u), __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u),
+                                0x05040100u);
+    o.y = __builtin_amdgcn_perm(__builtin_amdgcn_perm(b[7], b[6], 0x0c0c0400u), __builtin_amdgcn_perm(b[5], b[4], 0x0c0c0400u),
+                                0x05040100u);
     return o;
 }
 

@@ -131,7 +131,7 @@ void orc_quant_act_i8(const uint16_t *x, int64_t M, int64_t K, int8_t *q,
  * argument.  The kernels do not divide per element: with r = 1.0f / sc (one IEEE
  * division per row) they form
  *     q0 = x * r;  e = fma(-q0, sc, x);  q1 = fma(e, r, q0)
- * and round q1.  This counts the (amax, x) pairs for which that differs from
+ * and round q1 (by adding 1.5 * 2^23 and taking the low byte of the sum, unclamped).  This counts the (amax, x) pairs for which that differs from
  * rintf(x / sc) clamped to +-127 -- over every scale a row can have (amax = any
  * finite non-negative bf16 with bit pattern in [amax_lo, amax_hi)) and every
  * finite bf16 x with |x| <= amax.  With check_quotient != 0 the quotients
@@ -155,9 +155,15 @@ int64_t orc_quant_division_mismatches(int32_t amax_lo, int32_t amax_hi, int32_t 
                 const float q0 = x * r;
                 const float e = fmaf(-q0, sc, x);
                 const float q1 = fmaf(e, r, q0);
-                float got = rintf(q1);
-                got = fminf(fmaxf(got, -127.f), 127.f);
-                int differ = (int)got != (int)ref;
+                /* the kernels round and narrow in one addition: q1 + 1.5 * 2^23 has a unit in the
+                 * last place of 1, so the sum is q1 rounded to the nearest integer, ties to even, and
+                 * its low byte is that integer in two's complement -- with no clamp, which is only
+                 * right if the rounded value never leaves [-127, 127]; both are part of this check */
+                const float magic = q1 + 12582912.0f;
+                uint32_t mbits;
+                memcpy(&mbits, &magic, 4);
+                const int got = (int)(int8_t)(mbits & 0xffu);
+                int differ = got != (int)ref || (mbits - 0x4B400000u + 127u) > 254u;
                 if (check_quotient && fabsf(ref_q) >= 1.17549435e-38f) {
                     uint32_t u0, u1;
                     memcpy(&u0, &ref_q, 4);
