@@ -250,11 +250,13 @@ def main() -> int:
                               "frac_of_int8_peak": round(tops / INT8_PEAK_TOPS, 4)}}))
         return 0
 
-    def w4a8_decode_step(rows: int, use_graph: bool, iters: int):
+    def w4a8_decode_step(rows: int, use_graph: bool, iters: int, prequantised: bool = False):
         """The decode step of the same model with int4 group-128 weights (32 x {qkv, o, gate_up,
         down} + lm_head, 1.84 GB of distinct packed weights), one cmi_linear_w4a8_bf16 call per
         projection: the quantiser folded into the GEMV where that is the faster route, else two
-        launches.  Returns the result block for ``extra``."""
+        launches.  ``prequantised``: the activations arrive as int8 rows + scales, as they do
+        behind cmi_rms_norm_i8 / cmi_silu_mul_quant (the producer has quantised them), and every
+        projection is one cmi_gemv_w4a8 call.  Returns the result block for ``extra``."""
         proj = []
         xs_ = {k_: synth.activations(16, k_, gen) for k_ in (2560, 4096, 9728)}
         for layer in range(LAYERS + 1):
@@ -269,13 +271,24 @@ def main() -> int:
                 proj.append((d4, ds, xs_[k_], torch.empty((16, n_), dtype=torch.bfloat16, device=dev), n_, k_))
         nbytes = int(lib.cmi_linear_workspace_bytes(16, 9728))
         work = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        xq_ = {}
+        if prequantised:
+            for k_, x in xs_.items():
+                q_ = torch.empty((16, k_), dtype=torch.int8, device=dev)
+                s_ = torch.empty(16, dtype=torch.float32, device=dev)
+                _native.check(lib.cmi_quant_act_i8(ptr(x), ptr(q_), ptr(s_), 16, k_, cur_stream()), "quant")
+                xq_[k_] = (q_, s_)
 
         def step():
             st = cur_stream()
             for d4, ds, x, y, n_, k_ in proj:
-                rc = lib.cmi_linear_w4a8_bf16(ptr(d4), ptr(ds), ptr(x), ptr(y), rows, n_, k_, 128, ptr(work), nbytes, st)
+                if prequantised:
+                    rc = lib.cmi_gemv_w4a8(ptr(d4), ptr(ds), ptr(xq_[k_][0]), ptr(xq_[k_][1]), ptr(y), vp(0), rows, n_, k_,
+                                           128, st)
+                else:
+                    rc = lib.cmi_linear_w4a8_bf16(ptr(d4), ptr(ds), ptr(x), ptr(y), rows, n_, k_, 128, ptr(work), nbytes, st)
                 if rc:
-                    _native.check(rc, "cmi_linear_w4a8_bf16")
+                    _native.check(rc, "w4a8 projection")
 
         runner, mode = step, "eager"
         if use_graph:
@@ -295,9 +308,11 @@ def main() -> int:
                     raise RuntimeError("HIP graph replay of the W4A8 step differs from the eager step")
             runner, mode = graph.replay, "hipgraph"
         t = timed(runner, iters, warm=2)
-        alg = sum(synth.w4_gemv_bytes(rows, n_, k_) for *_, n_, k_ in proj)
+        # pre-quantised rows are one byte per element plus a scale per row instead of two bytes
+        alg = sum(synth.w4_gemv_bytes(rows, n_, k_) - (rows * k_ - 4 * rows if prequantised else 0) for *_, n_, k_ in proj)
         gbps = alg / t / 1e9
         return {"ms_per_step": round(t * 1e3, 4), "GBps": round(gbps, 1), "launch": mode, "rows": rows,
+                "activations": "int8 rows + scales (quantised upstream)" if prequantised else "bf16 (quantised inside the call)",
                 "projections_per_step": len(proj), "algorithmic_bytes_per_step": alg,
                 "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                              "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
@@ -509,6 +524,10 @@ def main() -> int:
 
         # W4A8 decode step (int4 weights, per-token int8 activations), one and sixteen rows
         extra["w4a8_decode_step"] = {f"M{m}": w4a8_decode_step(m, True, max(3, args.steps // 2)) for m in (1, 16)}
+        torch.cuda.empty_cache()
+        extra["w4a8_decode_step"]["M1_prequantised"] = w4a8_decode_step(1, True, max(3, args.steps // 2), True)
+        torch.cuda.empty_cache()
+        extra["w4a8_decode_step"]["M16_prequantised"] = w4a8_decode_step(16, True, max(3, args.steps // 2), True)
         torch.cuda.empty_cache()
 
         # W4A8 decode GEMV (quantiser + GEMV, as the adapter issues them)
