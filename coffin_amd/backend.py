@@ -553,6 +553,64 @@ def rms_norm_i8(x: torch.Tensor, w: torch.Tensor, out_q: torch.Tensor, out_s: to
     return out_q
 
 
+def _norm_native(x: torch.Tensor, w: torch.Tensor) -> bool:
+    return (_on_gpu(x) and x.dtype == torch.bfloat16 and x.dim() == 2 and (x.shape[1] == 1 or x.stride(1) == 1)
+            and w.device == x.device and w.numel() == x.shape[1])
+
+
+def _gain_bf16(w: torch.Tensor) -> torch.Tensor:
+    return w if (w.dtype == torch.bfloat16 and w.is_contiguous()) else _memo(w, lambda: w.to(torch.bfloat16).contiguous())
+
+
+def rms_norm(x: torch.Tensor, w: torch.Tensor, stride: int = 0, eps: float = 1e-6) -> torch.Tensor:
+    """``rms_norm(x, w, stride=0, eps=1e-6) -> y``: zero-centred RMSNorm over the last axis of a 2-D
+    block (backends/protocol.py:238-243, backends/reference/__init__.py:169-198).  Registered so that
+    ``rms_norm`` followed by ``kv_quant`` and :func:`rms_norm_i8` are one arithmetic (the kernel is
+    the same, with and without the quantised outputs).  ``stride`` is informational, as in the
+    reference: the row pitch is read from ``x``."""
+    del stride
+    if not _norm_native(x, w):
+        xf = x.to(torch.float32)
+        scale = torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + eps)
+        return (xf * scale).to(x.dtype) * w.to(x.dtype)
+    m, n = x.shape
+    y = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    if m == 0:
+        return y
+    gain = _gain_bf16(w)
+    with torch.cuda.device(x.device):
+        rc = _native.load().cmi_rms_norm_i8(x.data_ptr(), gain.data_ptr(), y.data_ptr(), 0, 0, m, n,
+                                            x.stride(0) if m > 1 else max(x.stride(0), n), n, float(eps), _stream())
+    if rc:
+        _native.check(rc, "rms_norm")
+    return y
+
+
+def add_rms_norm(x: torch.Tensor, add: torch.Tensor, w: torch.Tensor, out: torch.Tensor, stride: int = 0,
+                 eps: float = 1e-6) -> torch.Tensor:
+    """``add_rms_norm(x, add, w, out, stride=0, eps=1e-6) -> out``: ``x += add`` in place, then the
+    RMSNorm of the sum into ``out`` (backends/protocol.py:244-248, backends/reference/__init__.py:224-250)."""
+    del stride
+    ok = (_norm_native(x, w) and add.shape == x.shape and add.dtype == torch.bfloat16 and add.device == x.device
+          and (add.shape[1] == 1 or add.stride(1) == 1) and out.shape == x.shape and out.dtype == torch.bfloat16
+          and out.device == x.device and (out.shape[1] == 1 or out.stride(1) == 1))
+    if not ok:
+        x.add_(add)
+        out.copy_(rms_norm(x, w, 0, eps))
+        return out
+    m, n = x.shape
+    if m == 0:
+        return out
+    gain = _gain_bf16(w)
+    pitch = lambda t: t.stride(0) if m > 1 else max(t.stride(0), n)
+    with torch.cuda.device(x.device):
+        rc = _native.load().cmi_add_rms_norm_i8(x.data_ptr(), add.data_ptr(), gain.data_ptr(), out.data_ptr(), 0, 0, m, n,
+                                                pitch(x), pitch(add), pitch(out), float(eps), _stream())
+    if rc:
+        _native.check(rc, "add_rms_norm")
+    return out
+
+
 def embed_rows(w, ids: torch.Tensor) -> torch.Tensor:
     """Rows ``ids`` of a quantized embedding matrix as bf16 ``[T, K]``: only the gathered rows are
     dequantised (ops/embed.py:64-81; ``QWeight.rows`` int8_weights.py:361-372,
@@ -587,7 +645,7 @@ def embed_rows(w, ids: torch.Tensor) -> torch.Tensor:
 
 #: Contract names this module answers natively.
 NATIVE_NAMES = ("linear", "linear_m", "linear_m_verify", "linear_prefill", "kv_quant",
-                "silu_mul", "silu_mul_quant")
+                "silu_mul", "silu_mul_quant", "rms_norm", "add_rms_norm")
 
 
 def native_table() -> dict:

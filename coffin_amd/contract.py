@@ -3,7 +3,7 @@
 When this package runs inside a coffin checkout the vendor file binds to coffin's
 own ``backends.protocol`` / ``backends.vendor`` classes; everywhere else (this
 repository's tests, the benchmark, a GPU box without the reference tree) these
-stand-ins carry the same names, fields and error behaviour for the seven table
+stand-ins carry the same names, fields and error behaviour for the nine table
 entries on the path:
 
 * ``Ops`` -- backends/protocol.py:130-541: a frozen table keyed by op name,
@@ -37,6 +37,8 @@ class Ops:
     kv_quant: OpFn | None = None         # kv_quant(x, out_q, out_s) -> out_q  (protocol.py:258)
     silu_mul: OpFn | None = None         # silu_mul(gate, up, out) -> out      (protocol.py:273)
     silu_mul_quant: OpFn | None = None   # (gate, up, out, out_q, out_s) -> out (protocol.py:278)
+    rms_norm: OpFn | None = None         # rms_norm(x, w, stride=0, eps=1e-6) -> y (protocol.py:243)
+    add_rms_norm: OpFn | None = None     # (x, add, w, out, stride=0, eps=1e-6) -> out (protocol.py:248)
 
     NAMES: ClassVar[tuple[str, ...]]
 

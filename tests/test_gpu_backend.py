@@ -41,7 +41,7 @@ def _w4(n, k, g):
 def test_vendor_builds_the_native_table():
     ops = mi355x.build_ops()
     assert set(ops.implemented()) == {"linear", "linear_m", "linear_m_verify", "linear_prefill",
-                                      "kv_quant", "silu_mul", "silu_mul_quant"}
+                                      "kv_quant", "silu_mul", "silu_mul_quant", "rms_norm", "add_rms_norm"}
     from coffin_amd import contract
     # a board that reports its name is claimed by name; a host without the amdgpu id table
     # reports the generic "AMD Radeon Graphics", which is left to explicit selection

@@ -175,6 +175,32 @@ def test_rms_norm_i8_adapter_and_special_rows(orc):
         backend.rms_norm_i8(x.float(), w, out_q, out_s)
 
 
+def test_rms_norm_table_entries_share_the_fused_arithmetic(orc):
+    """rms_norm / add_rms_norm of the table followed by kv_quant give what rms_norm_i8 gives."""
+    g = synth.generator(11, G.DEV)
+    x = (torch.randn((7, 2560), generator=g, device=G.DEV) * 2).to(torch.bfloat16)
+    add = torch.randn((7, 2560), generator=g, device=G.DEV).to(torch.bfloat16)
+    w = (1 + 0.1 * torch.randn(2560, generator=g, device=G.DEV)).to(torch.bfloat16)
+    y = backend.rms_norm(x, w)
+    y_ref, _ = orc.rms_norm(G.bits(x), G.bits(w))
+    assert (G.bits(y) == y_ref).all()
+    q = torch.empty((7, 2560), dtype=torch.int8, device=G.DEV)
+    s = torch.empty(7, dtype=torch.float32, device=G.DEV)
+    backend.kv_quant(y, q, s)
+    q2, s2 = torch.empty_like(q), torch.empty_like(s)
+    backend.rms_norm_i8(x, w, q2, s2)
+    assert (q == q2).all() and (s == s2).all()
+    x2, out = x.clone(), torch.empty_like(x)
+    assert backend.add_rms_norm(x2, add, w, out) is out
+    y_ref2, x_ref2 = orc.rms_norm(G.bits(x), G.bits(w), add=G.bits(add))
+    assert (G.bits(out) == y_ref2).all() and (G.bits(x2) == x_ref2).all()
+    # fp32 rows take the torch statement of the reference
+    xf = x.float()
+    want = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)) * w.float()
+    assert torch.allclose(backend.rms_norm(xf, w.float()), want)
+    assert "rms_norm" in backend.native_table() and "add_rms_norm" in backend.native_table()
+
+
 # ------------------------------------------------------------- embedding rows
 
 @pytest.mark.parametrize("n,k", [(3000, 2560), (151936, 2560), (50, 100), (64, 4096)])

@@ -23,7 +23,7 @@ ROOT = Path(__file__).resolve().parent.parent
 
 def test_ops_table_names_and_errors():
     assert contract.Ops.NAMES == ("linear", "linear_m", "linear_m_verify", "linear_prefill",
-                                  "kv_quant", "silu_mul", "silu_mul_quant")
+                                  "kv_quant", "silu_mul", "silu_mul_quant", "rms_norm", "add_rms_norm")
     t = contract.Ops.from_mapping({"linear": lambda w, x: x})
     assert t.implemented() == ("linear",) and "kv_quant" in t.missing()
     with pytest.raises(ValueError, match="unknown op"):
