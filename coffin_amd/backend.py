@@ -265,6 +265,13 @@ def _lookup(w) -> _Record | None:
 
 
 def _make_record(w) -> _Record:
+    # A weight is resolved (and an int4 weight re-laid out into a private copy) on its first use.
+    # Under stream capture that copy would live in the graph's memory pool and the re-layout would
+    # be replayed with every step: the callers' warm-up step (the reference's engine runs one
+    # before it captures, engine/llm_engine.py:116) must have touched every weight already.
+    if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
+        raise RuntimeError("coffin_amd: first use of a quantized weight inside graph capture; "
+                           "run one eager step over every projection before capturing")
     rec = _Record()
     if _is_w4(w):
         w4, ws = _w4_operands(w)

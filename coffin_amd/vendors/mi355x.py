@@ -61,15 +61,19 @@ SPEC = VendorSpec(
     ),
     act_dtype=torch.bfloat16,
     weight_dtype=torch.bfloat16,
-    graph=False,
+    # The adapters are capture-safe once a warm-up step has touched every weight (they launch on the
+    # current stream, never synchronise and keep no per-call host state); a captured 129-projection
+    # decode step runs in 0.856 ms against 0.976 ms launched eagerly (7 us of host time per call
+    # in front of a 6.7 us kernel), so decode should be captured.
+    graph=True,
     autotune=False,
     int8_weights=True,
     batch_attn=False,
     attn_split=1,
     weight_layout="nk",
     priority=50,
-    notes="native: linear, linear_m, linear_m_verify, linear_prefill, kv_quant; "
-          "everything else runs the torch reference",
+    notes="native: linear, linear_m, linear_m_verify, linear_prefill, kv_quant, silu_mul, "
+          "silu_mul_quant, rms_norm, add_rms_norm; everything else runs the torch reference",
     has_kernels=True,
     build_ops=build_ops,
 )

@@ -257,6 +257,36 @@ def test_adapters_replay_inside_a_captured_graph():
             assert (got.view(torch.int16) == want.view(torch.int16)).all()
 
 
+def test_first_use_of_a_weight_inside_capture_is_refused():
+    """The SPEC declares decode capturable; what capture cannot hold is a weight's first use (its
+    private re-laid-out copy would be allocated and rebuilt inside the graph).  The adapter says
+    so before anything is launched, and the same weight works once it has been touched eagerly."""
+    from coffin_amd.vendors import mi355x
+    assert mi355x.SPEC.graph is True
+    g = synth.generator()
+    w = _w4(256, 512, g)
+    x = synth.activations(1, 512, g).to(G.DEV)[0].contiguous()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with pytest.raises(RuntimeError, match="inside graph capture"):
+            with torch.cuda.graph(graph, stream=side):
+                _kept = x * 1                # so the abandoned graph is not an empty one
+                backend.linear(w, x)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    want = backend.linear(w, x)
+    graph2 = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph2, stream=side):
+            got = backend.linear(w, x)
+    torch.cuda.current_stream().wait_stream(side)
+    graph2.replay()
+    torch.cuda.synchronize()
+    assert (got.view(torch.int16) == want.view(torch.int16)).all()
+
+
 def test_outputs_are_fresh_and_inputs_untouched():
     g = synth.generator()
     q, w = _q8(256, 512, g), _w4(256, 512, g)

@@ -38,6 +38,7 @@ def test_vendor_spec_validation_and_declaration():
     spec.validate()
     assert spec.name == "mi355x" and spec.weight_layout == "nk" and spec.int8_weights
     assert spec.has_kernels and callable(spec.build_ops)
+    assert spec.graph is True and spec.autotune is False     # decode is captured; nothing to tune
     assert spec.detection.namespace == "cuda" and spec.detection.hip
     assert all(m == m.lower() for m in spec.detection.name_markers)
     # the generic name every id-table-less AMD host reports must not be claimed
