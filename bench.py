@@ -155,6 +155,8 @@ def parse_args():
     ap.add_argument("--w4a8-prefill-only", action="store_true",
                     help="time only the W4A8 prefill GEMM (M=1024, N=25600, K=5120): the profiling target "
                          "for that kernel; prints its own JSON line")
+    ap.add_argument("--prequantised", action="store_true",
+                    help="with --w4a8-decode-only: activations arrive as int8 rows + scales")
     ap.add_argument("--w4a8-decode-only", action="store_true",
                     help="time only the W4A8 decode step (32 layers + lm_head at one row, one "
                          "cmi_linear_w4a8_bf16 call per projection): the profiling target for the W4A8 decode "
@@ -333,7 +335,8 @@ def main() -> int:
         return 0
 
     if args.w4a8_decode_only:
-        out = {f"M{args.rows}": w4a8_decode_step(args.rows, not args.no_graph, args.steps)}
+        key = f"M{args.rows}" + ("_prequantised" if args.prequantised else "")
+        out = {key: w4a8_decode_step(args.rows, not args.no_graph, args.steps, args.prequantised)}
         print(json.dumps({"metric": "W4A8 decode step HBM GB/s", "unit": "GB/s", "w4a8_decode_step": out}))
         return 0
 

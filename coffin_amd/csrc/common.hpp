@@ -22,6 +22,7 @@ int reserve_lds(const void *kernel, int bytes, std::atomic<uint64_t> &devices, c
 int option_gemm_tile();      // 0 = the library chooses, else 64 / 128 / 256 / 320
 int option_gemv_wholerow();  // -1 = the library chooses, 0 = never, 1 = where it can
 int option_w4_decode_waves();  // 0 = the library chooses, else 4 or 16 wavefronts per workgroup
+int option_w4_decode_chain();  // 0 = the library chooses, 1 = never, else a variant code of gemv_w4a8_chain
 
 #define CMI_REQUIRE(cond, code, ...)                 \
     do {                                             \
@@ -41,6 +42,12 @@ int gemm_w8a8_rows16(const int8_t *xq, const int8_t *wq, const float *xs, const 
 int gemv_w4a8_decode(const uint8_t *w4, const float *ws, const void *x, const int8_t *xq, const float *xs,
                      void *y, int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
                      void *stream);
+// gemv_w4a8_chain.hip: the same for 1..2 rows with the fp32 chain in registers; `variant` = lanes per
+// weight row (8, 16) + 100 * wavefronts sharing a row (1, 2, 4) + 10000 * wavefronts per workgroup
+// (4, 8, 16); CMI_E_UNSUPPORTED (no error text) outside the variant's range.
+int gemv_w4a8_chain(const uint8_t *w4, const float *ws, const void *x, const int8_t *xq, const float *xs,
+                    void *y, int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
+                    int variant, void *stream);
 // gemv_w4a8_rows16.hip: W4A8 GEMV for up to 16 quantised rows (xq, xs) or up to 4 bf16 rows (x,
 // quantised in the kernel), K <= 10240, integer sums on the matrix pipe; CMI_E_UNSUPPORTED (no error text) outside that range.
 int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs, const void *x,

@@ -345,6 +345,27 @@ int dispatch(const Args &a, hipStream_t st) {
     return dispatch_wv<M, PREQ, 4>(a, st, ksplit);
 }
 
+// Variant of gemv_w4a8_chain for this shape (lanes per weight row + 100 * wavefronts per row +
+// 10000 * wavefronts per workgroup), or 0 to stay with the kernel of this file.  Measured per
+// projection, quantised rows / bf16 rows, against this file's kernel:
+//   2560 -> 6144   3.6 / 4.0 us (4.3 / 4.7)      4096 -> 2560   3.2 / 3.6 us (3.6 / 4.1)
+//   2560 -> 19456  6.2 / 7.3 us (7.1 / 8.3)      9728 -> 2560   5.6 / 7.5 us (5.9 / 8.1)
+int chain_variant(int M, int N, int K, bool from_bf16) {
+    const int opt = option_w4_decode_chain();
+    if (opt == 1 || M > 2) return 0;
+    if (opt) return opt;
+    if (K <= 5120) {
+        // sixteen lanes per row (four rows per wavefront); from bf16 rows, a grid of one to two
+        // 16-row workgroups per compute unit is better served by 32-row workgroups (half as many
+        // of them repeat the quantisation)
+        const int wgs16 = (N + 15) / 16;
+        return from_bf16 && wgs16 > 256 && wgs16 <= 512 ? 40108 : 40116;
+    }
+    // longer rows: four wavefronts (quantised rows) or two of an eight-wavefront workgroup (bf16
+    // rows) share a row
+    return from_bf16 ? 80216 : 40416;
+}
+
 }  // namespace
 
 namespace cmi {
@@ -356,6 +377,11 @@ int gemv_w4a8_decode(const uint8_t *w4, const float *ws, const void *x, const in
                      void *y, int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
                      void *stream) {
     if (M < 1 || M > 4 || K < GS || K > MAX_K || K % GS != 0 || N < 1) return CMI_E_UNSUPPORTED;
+    // the chain-in-registers kernel where it applies (and is not switched off)
+    if (const int variant = chain_variant(M, N, K, x != nullptr)) {
+        const int rc = gemv_w4a8_chain(w4, ws, x, xq, xs, y, group_acc, xq_out, xs_out, M, N, K, variant, stream);
+        if (rc != CMI_E_UNSUPPORTED) return rc;
+    }
     Args a;
     a.w4 = w4;
     a.ws = ws;

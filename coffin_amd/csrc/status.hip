@@ -53,6 +53,7 @@ constexpr int UNREAD = INT32_MIN;
 std::atomic<int> g_gemm_tile{UNREAD};      // 0 = the library chooses
 std::atomic<int> g_gemv_wholerow{UNREAD};  // -1 = the library chooses, 0 = never, 1 = where it can
 std::atomic<int> g_w4_decode_waves{0};     // 0 = the library chooses, 4 or 16 wavefronts per workgroup
+std::atomic<int> g_w4_decode_chain{0};     // 0 = the library chooses, 1 = never, else a variant code
 
 bool valid_gemm_tile(int v) { return v == 0 || v == 64 || v == 128 || v == 256 || v == 320; }
 bool valid_wholerow(int v) { return v >= -1 && v <= 1; }
@@ -89,6 +90,7 @@ int option_gemv_wholerow() {
 }
 
 int option_w4_decode_waves() { return g_w4_decode_waves.load(std::memory_order_relaxed); }
+int option_w4_decode_chain() { return g_w4_decode_chain.load(std::memory_order_relaxed); }
 
 }  // namespace cmi
 
@@ -111,6 +113,17 @@ extern "C" int cmi_set_option(const char *name, int value) {
         CMI_REQUIRE(value == 0 || value == 4 || value == 16, CMI_E_ARG,
                     "cmi_set_option: w4_decode_waves=%d, expected 0 (library's choice), 4 or 16", value);
         g_w4_decode_waves.store(value, std::memory_order_relaxed);
+        return CMI_OK;
+    }
+    if (!strcmp(name, "w4_decode_chain")) {
+        const int lanes = value % 100, split = value / 100 % 100, waves = value / 10000;
+        CMI_REQUIRE(value == 0 || value == 1 ||
+                        ((lanes == 8 || lanes == 16) && (split == 1 || split == 2 || split == 4) &&
+                         (waves == 4 || waves == 8 || waves == 16)),
+                    CMI_E_ARG,
+                    "cmi_set_option: w4_decode_chain=%d, expected 0 (library's choice), 1 (never) or lanes (8, 16) "
+                    "+ 100 * wavefronts per row (1, 2, 4) + 10000 * wavefronts per workgroup (4, 8, 16)", value);
+        g_w4_decode_chain.store(value, std::memory_order_relaxed);
         return CMI_OK;
     }
     return fail(CMI_E_ARG, "cmi_set_option: unknown option '%s'", name);

@@ -42,7 +42,11 @@ int cmi_abi_version(void);
  *   "gemv_wholerow" -1 (the library chooses) | 0 (never) | 1: the one-wavefront-per-weight-row
  *                   kernel of cmi_gemv_w8a16;
  *   "w4_decode_waves" 0 (the library chooses) | 4 | 16: wavefronts per workgroup of the W4A8
- *                   decode GEMV (one bf16 or quantised row).
+ *                   decode GEMV (one bf16 or quantised row);
+ *   "w4_decode_chain" 0 (the library chooses) | 1 (never) | lanes + 100 * split + 10000 * waves: the
+ *                   W4A8 decode kernel that keeps the fp32 chain in registers, with `lanes` (8, 16)
+ *                   lanes per weight row, `split` (1, 2, 4) wavefronts sharing a row and `waves`
+ *                   (4, 8, 16) wavefronts per workgroup, wherever the shape fits that arrangement.
  * The environment variables CMI_GEMM_TILE and CMI_GEMV_WHOLEROW give the initial values; they are
  * read once, at the first call that needs them.  Unknown names or values: CMI_E_ARG.  Every choice
  * gives the same bits. */

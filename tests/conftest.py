@@ -39,6 +39,7 @@ def _library_options_back_to_default(request):
         lib.cmi_set_option(b"gemm_tile", 0)
         lib.cmi_set_option(b"gemv_wholerow", -1)
         lib.cmi_set_option(b"w4_decode_waves", 0)
+        lib.cmi_set_option(b"w4_decode_chain", 0)
 
 
 @pytest.fixture(scope="session")

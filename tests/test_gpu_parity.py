@@ -445,6 +445,46 @@ def test_gemv_w4a8_bf16_fused_quantiser_bit_exact(orc, m, n, k, waves):
     assert (G.bits(y) == y_ref).all()
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 9728, 2560), (1, 6144, 2560), (1, 2560, 4096), (2, 9728, 2560),
+                                   (1, 5120, 5120), (2, 333, 1280), (1, 7, 128), (2, 100, 384),
+                                   (1, 1001, 2688), (2, 64, 3968), (1, 300, 10240), (1, 33, 9728),
+                                   (2, 2560, 4096), (1, 257, 1024), (1, 640, 2048)])
+@pytest.mark.parametrize("variant", [40108, 40116, 40216, 40416, 80216, 80416, 160416])
+def test_gemv_w4a8_chain_in_registers_bit_exact(orc, m, n, k, variant):
+    """The kernel that multiplies codes with nibble planes of x + 128 and keeps the fp32 chain in
+    registers -- 8 or 16 lanes per weight row, 1, 2 or 4 wavefronts per row, 4, 8 or 16 wavefronts
+    per workgroup: quantised activations and bf16 ones, with and without the integer sums asked
+    for (the second takes the variant built for an exact K)."""
+    lanes, split = variant % 100, variant // 100 % 100
+    if k > lanes * 32 * split * (20 if (lanes, split) == (8, 1) else 10):
+        pytest.skip("beyond this arrangement's K")
+    G.set_option("w4_decode_chain", variant)
+    w4, ws, xq, xs, gacc_ref, y_ref = _w4_case(orc, m, n, k, seeded())
+    gacc, y = G.w4a8(w4, ws, xq, xs, k, gemm=False)
+    assert (gacc.cpu().numpy() == gacc_ref).all()
+    assert (G.bits(y) == y_ref).all()
+    _, y2 = G.w4a8(w4, ws, xq, xs, k, gemm=False, want_acc=False)
+    assert (G.bits(y2) == y_ref).all()
+    # from bf16 rows
+    g = seeded(7)
+    x = synth.activations(m, k, g, outliers=True)
+    xq_ref, xs_ref = orc.quant_act_i8(G.bits(x))
+    w = synth.int4_weight(n, k, g)
+    gacc_ref, y_ref = orc.linear_w4a8(xq_ref, xs_ref, w.packed.numpy(), w.scale.numpy(), k, 128,
+                                      want_group_acc=True)
+    w4, ws = G.w4_repack(w.packed.to(G.DEV), w.scale.to(G.DEV), k)
+    gacc, y, xq_d, xs_d = G.gemv_w4a8_bf16(w4, ws, x.to(G.DEV), k)
+    assert (xq_d.cpu().numpy() == xq_ref).all()
+    assert (xs_d.cpu().numpy().view(np.uint32) == xs_ref.view(np.uint32)).all()
+    assert (gacc.cpu().numpy() == gacc_ref).all()
+    assert (G.bits(y) == y_ref).all()
+    yb = torch.empty((m, n), dtype=torch.bfloat16, device=G.DEV)
+    from coffin_amd import _native
+    _native.check(_native.load().cmi_gemv_w4a8_bf16(G.ptr(w4), G.ptr(ws), G.ptr(x.to(G.DEV)), G.ptr(yb), None, None,
+                                                    None, m, n, k, 128, G.stream()), "gemv_w4a8_bf16")
+    assert (G.bits(yb) == y_ref).all()
+
+
 def test_gemv_w4a8_bf16_refuses_wide_batches():
     g = seeded()
     w = synth.int4_weight(256, 256, g)
