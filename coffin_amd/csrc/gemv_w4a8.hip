@@ -344,14 +344,19 @@ extern "C" int cmi_gemv_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     CMI_REQUIRE(aligned(w4, 16) && aligned(xq, 16), CMI_E_ARG,
                 "cmi_gemv_w4a8: w4 and xq must be 16-byte aligned");
     if (gs == GS && N >= 1 && M >= 1) {
-        // One row: the dot-product kernel while a wavefront can hold its whole rows (K <= 4096) or
-        // the grid is small enough that the wavefronts of a workgroup share rows; with longer rows
-        // it runs 10-20 KiB per wavefront at low occupancy (5120 -> 25600: 40 us against 20).
-        // Two rows: the same kernel only for whole rows of a large weight (2560 -> 151936: 34.5 us
+        // One row: the dot-product kernels.  The one that keeps the fp32 chain in registers takes any
+        // K up to 20480 (5120 -> 25600: 13.0 us against 20.9 on the matrix-pipe kernel, 9728 -> 9728:
+        // 11.6 against 23.2); without it (switched off, or longer rows) the older one while a
+        // wavefront can hold its whole rows (K <= 4096) or the grid is small enough that the
+        // wavefronts of a workgroup share rows.
+        // Two rows: the same kernels only for whole rows of a large weight (2560 -> 151936: 34.5 us
         // against 42); otherwise, and from three rows, group sums on the matrix pipe.
-        const bool shared_rows = (N + 15) / 16 < 256, whole_rows = K <= 4096;
+        const bool chain_on = option_w4_decode_chain() != 1;
+        const bool shared_rows = (N + 15) / 16 < 256, whole_rows = K <= (chain_on ? 5120 : 4096);
+        const bool forced = option_w4_decode_chain() > 1 && M <= 2;  // a variant named by the caller
         int rc = CMI_E_UNSUPPORTED;
-        if ((M == 1 && (whole_rows || shared_rows)) || (M == 2 && whole_rows && N >= 12288))
+        if ((M == 1 && (whole_rows || shared_rows || (chain_on && K <= 20480))) ||
+            (M == 2 && whole_rows && N >= 12288) || forced)
             rc = gemv_w4a8_decode(w4, ws, nullptr, xq, xs, y, group_acc, nullptr, nullptr, M, N, K, stream);
         if (rc == CMI_E_UNSUPPORTED)
             rc = gemv_w4a8_rows16(w4, ws, xq, xs, nullptr, y, group_acc, nullptr, nullptr, M, N, K, stream);
@@ -384,7 +389,8 @@ extern "C" int cmi_gemv_w4a8_bf16(const uint8_t *w4, const float *ws, const void
     // rows is the exception since that kernel's walk over the groups was made branch-free:
     // 9728 -> 2560 8.6 -> 8.25 us, 6144 -> 1024 5.9 -> 4.6 us)
     const bool one_shared_row = M == 1 && (N + 15) / 16 < 256;
-    if (K > 4096 && !one_shared_row)
+    const int whole_row_k = option_w4_decode_chain() == 1 ? 4096 : 5120;
+    if (K > whole_row_k && !one_shared_row && !(option_w4_decode_chain() > 1))
         rc = gemv_w4a8_rows16(w4, ws, nullptr, nullptr, x, y, group_acc, xq_out, xs_out, M, N, K, stream);
     if (rc != CMI_E_UNSUPPORTED) return rc;
     rc = gemv_w4a8_decode(w4, ws, x, nullptr, nullptr, y, group_acc, xq_out, xs_out, M, N, K, stream);

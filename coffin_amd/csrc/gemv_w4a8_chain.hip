@@ -310,6 +310,7 @@ int dispatch_nl(const Args &a, hipStream_t st) {
         if (loads <= 16) return launch<M, LPR, 16, PREQ, S, WAVES>(a, st);
         if (loads <= 20) return launch<M, LPR, 20, PREQ, S, WAVES>(a, st);
     }
+
     return CMI_E_UNSUPPORTED;
 }
 
@@ -326,6 +327,8 @@ int dispatch(const Args &a, int lanes, int split, int waves, hipStream_t st) {
         if (split == 2 && waves == 8) return dispatch_nl<M, 16, PREQ, 2, 8>(a, st);
         if (split == 4 && waves == 8) return dispatch_nl<M, 16, PREQ, 4, 8>(a, st);
         if (split == 4 && waves == 16) return dispatch_nl<M, 16, PREQ, 4, 16>(a, st);
+        if (split == 8 && waves == 8) return dispatch_nl<M, 16, PREQ, 8, 8>(a, st);
+        if (split == 8 && waves == 16) return dispatch_nl<M, 16, PREQ, 8, 16>(a, st);
     }
     return CMI_E_UNSUPPORTED;
 }

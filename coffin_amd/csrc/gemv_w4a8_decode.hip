@@ -376,12 +376,13 @@ namespace cmi {
 int gemv_w4a8_decode(const uint8_t *w4, const float *ws, const void *x, const int8_t *xq, const float *xs,
                      void *y, int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
                      void *stream) {
-    if (M < 1 || M > 4 || K < GS || K > MAX_K || K % GS != 0 || N < 1) return CMI_E_UNSUPPORTED;
+    if (M < 1 || M > 4 || K < GS || K % GS != 0 || N < 1) return CMI_E_UNSUPPORTED;
     // the chain-in-registers kernel where it applies (and is not switched off)
     if (const int variant = chain_variant(M, N, K, x != nullptr)) {
         const int rc = gemv_w4a8_chain(w4, ws, x, xq, xs, y, group_acc, xq_out, xs_out, M, N, K, variant, stream);
         if (rc != CMI_E_UNSUPPORTED) return rc;
     }
+    if (K > MAX_K) return CMI_E_UNSUPPORTED;
     Args a;
     a.w4 = w4;
     a.ws = ws;

@@ -15,13 +15,14 @@ constexpr size_t ALIGN = 256;
 constexpr size_t round_up(size_t v) { return (v + ALIGN - 1) / ALIGN * ALIGN; }
 
 // Whether `rows` bf16 rows go through the W4A8 GEMV that quantises them itself (one launch).
-// That kernel lets every workgroup redo the quantisation: it wins for one row (two on long
-// rows), and loses where many workgroups each quantise a long row (K > 4096 with N >= 8192:
-// 5120 -> 9728 takes 16.3 us fused against 9.8 + 2.5 us as two launches); beyond K = 10240
-// only the two-launch route has a fast kernel.
+// That kernel lets every workgroup redo the quantisation.  One row of K <= 5120 always (5120 ->
+// 25600: 15.2 us against 2.3 + 13.0 us as two launches, 5120 -> 9728: 8.2 against 2.3 + 6.9); longer
+// rows lose where many workgroups each quantise them (K > 5120 with N >= 8192), and win for up to
+// two rows elsewhere; beyond K = 10240 only the two-launch route has a fast kernel.
 bool w4_fused_route(int rows, int N, int K) {
-    if ((K > 4096 && N >= 8192) || K > 10240) return false;
-    return rows <= (K > 5120 ? 2 : 1);
+    if (K <= 5120) return rows <= 1;
+    if (N >= 8192 || K > 10240) return false;
+    return rows <= 2;
 }
 
 }  // namespace

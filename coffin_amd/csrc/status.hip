@@ -118,11 +118,11 @@ extern "C" int cmi_set_option(const char *name, int value) {
     if (!strcmp(name, "w4_decode_chain")) {
         const int lanes = value % 100, split = value / 100 % 100, waves = value / 10000;
         CMI_REQUIRE(value == 0 || value == 1 ||
-                        ((lanes == 8 || lanes == 16) && (split == 1 || split == 2 || split == 4) &&
+                        ((lanes == 8 || lanes == 16) && (split == 1 || split == 2 || split == 4 || split == 8) &&
                          (waves == 4 || waves == 8 || waves == 16)),
                     CMI_E_ARG,
                     "cmi_set_option: w4_decode_chain=%d, expected 0 (library's choice), 1 (never) or lanes (8, 16) "
-                    "+ 100 * wavefronts per row (1, 2, 4) + 10000 * wavefronts per workgroup (4, 8, 16)", value);
+                    "+ 100 * wavefronts per row (1, 2, 4, 8) + 10000 * wavefronts per workgroup (4, 8, 16)", value);
         g_w4_decode_chain.store(value, std::memory_order_relaxed);
         return CMI_OK;
     }
