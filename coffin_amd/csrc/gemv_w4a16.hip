@@ -64,7 +64,7 @@ gemv_w4a16_kernel(const Args a) {
     float *xsum = reinterpret_cast<float *>(lds + (size_t)a.K * 2);     // fp32 [G]
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int n_raw = blockIdx.x * WAVES + wave;
+    const int n_raw = xcd_contiguous_block(blockIdx.x, gridDim.x) * WAVES + wave;
     const int n = n_raw < a.N ? n_raw : a.N - 1;
     const int nchunks = a.K / 32, xvecs = a.K / 8;
 

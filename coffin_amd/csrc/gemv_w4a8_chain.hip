@@ -90,7 +90,8 @@ gemv_w4a8_chain_kernel(const Args a) {
     const int c = lane % LPR, r = lane / LPR;
     const int team = wave / S, part_s = wave % S;  // which rows, which run of loads
     const int j0 = part_s * NL;                     // first load of this wavefront
-    const int n_raw = (blockIdx.x * (WAVES / S) + team) * RPW + r;
+    const int block = xcd_contiguous_block(blockIdx.x, gridDim.x);
+    const int n_raw = (block * (WAVES / S) + team) * RPW + r;
     const int n = min(n_raw, a.N - 1);
     const int nchunks = a.K / 32;
 
@@ -180,7 +181,7 @@ gemv_w4a8_chain_kernel(const Args a) {
             const RowScale rs = row_scale(amax);
             if (threadIdx.x == 0) {
                 xs_lds[m] = rs.sc;
-                if (a.xs_out && blockIdx.x == 0 && m < a.M) a.xs_out[m] = rs.sc;
+                if (a.xs_out && block == 0 && m < a.M) a.xs_out[m] = rs.sc;
             }
 #pragma unroll
             for (int j = 0; j < XVN; ++j) {
@@ -198,7 +199,7 @@ gemv_w4a8_chain_kernel(const Args a) {
                     slot[idx & 3] = hi;
                     slot[4 + (idx & 3)] = lo;
                     if ((idx & 3) == 0) xsum[m * CP + (idx >> 2)] = -8 * s8;
-                    if (a.xq_out && blockIdx.x == 0 && m < a.M)
+                    if (a.xq_out && block == 0 && m < a.M)
                         reinterpret_cast<uint2 *>(a.xq_out + (size_t)m * a.K)[idx] = q;
                 }
             }

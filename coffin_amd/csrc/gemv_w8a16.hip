@@ -132,7 +132,7 @@ gemv_w8a16_kernel(const GemvArgs a) {
     // a single unit means one wavefront per team; otherwise wave / uw through a 16-bit reciprocal
     // (exact for the at most 16 wavefronts of a workgroup)
     const int team = MODE == 0 ? wave : (int)(((uint32_t)wave * a.uw_rcp) >> 16);
-    const int rb = blockIdx.x * a.teams + team;
+    const int rb = xcd_contiguous_block(blockIdx.x, gridDim.x) * a.teams + team;
     const bool idle = rb >= a.nblocks;  // only in the last workgroup
     int u = wave - team * a.uw;         // unit in hand; the team's wavefronts stride over units
     const int xvecs = a.K / 8;          // uint4 per activation row
@@ -408,7 +408,7 @@ gemv_w8a16_wholerow_kernel(const GemvArgs a) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int waves = blockDim.x >> 6;
-    const int n_raw = blockIdx.x * waves + wave;
+    const int n_raw = xcd_contiguous_block(blockIdx.x, gridDim.x) * waves + wave;
     const int n = n_raw < a.N ? n_raw : a.N - 1;
     const int8_t *wrow = a.wq + (size_t)n * a.K;
     const int xvecs = a.K / 8;
