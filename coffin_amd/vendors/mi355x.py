@@ -63,8 +63,8 @@ SPEC = VendorSpec(
     weight_dtype=torch.bfloat16,
     # The adapters are capture-safe once a warm-up step has touched every weight (they launch on the
     # current stream, never synchronise and keep no per-call host state); a captured 129-projection
-    # decode step runs in 0.856 ms against 0.976 ms launched eagerly (7 us of host time per call
-    # in front of a 6.7 us kernel), so decode should be captured.
+    # decode step runs in 0.82 ms against 0.98 ms launched eagerly (7 us of host time per call
+    # in front of a 6.3 us kernel), so decode should be captured.
     graph=True,
     autotune=False,
     int8_weights=True,
