@@ -717,6 +717,101 @@ def main() -> int:
         t = timed(lambda: lib.cmi_quant_act_i8(ptr(x), ptr(xq), ptr(xs), m, k_, cur_stream()), 20)
         extra["quant_act_i8_M8192_K2560"] = {"us": round(t * 1e6, 2),
                                              "GBps": round(synth.quant_bytes(m, k_) / t / 1e9, 1)}
+        torch.cuda.empty_cache()
+
+        # fused producers, embedding gather and W4A16: algorithmic bytes / time against the HBM peak
+        def hbm_line(t, nbytes):
+            return {"us": round(t * 1e6, 2), "GBps": round(nbytes / t / 1e9, 1),
+                    "frac_of_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBPS, 4)}
+        prod = {}
+
+        def graph_time(calls):
+            """Mean time of one call: the calls (each on operands of its own) captured once, replayed."""
+            for c in calls:
+                c()
+            torch.cuda.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                for c in calls:
+                    c()
+            return timed(gr.replay, 5) / len(calls)
+
+        for m in (1, 2048, 8192):
+            copies = 16 if m == 1 else 6
+            kk = 9728      # silu(gate) * up over the two halves of a fused gate_up row -> bf16 + int8 + scale
+            sets = []
+            for _ in range(copies):
+                gu = synth.activations(m, 2 * kk, gen)
+                sets.append((gu, gu[:, kk:], torch.empty((m, kk), dtype=torch.bfloat16, device=dev),
+                             torch.empty((m, kk), dtype=torch.int8, device=dev),
+                             torch.empty(m, dtype=torch.float32, device=dev)))
+            t = graph_time([lambda s_=s_: lib.cmi_silu_mul_quant(ptr(s_[0]), ptr(s_[1]), ptr(s_[2]), ptr(s_[3]), ptr(s_[4]),
+                                                                  m, kk, 2 * kk, 2 * kk, kk, cur_stream()) for s_ in sets])
+            prod[f"silu_mul_quant_M{m}_K{kk}"] = hbm_line(t, m * kk * 7 + 4 * m)
+            t = graph_time([lambda s_=s_: lib.cmi_silu_mul_quant(ptr(s_[0]), ptr(s_[1]), None, ptr(s_[3]), ptr(s_[4]),
+                                                                  m, kk, 2 * kk, 2 * kk, kk, cur_stream()) for s_ in sets])
+            prod[f"silu_mul_quant_int8_only_M{m}_K{kk}"] = hbm_line(t, m * kk * 5 + 4 * m)
+            del sets
+            torch.cuda.empty_cache()
+            nn = 2560      # RMSNorm (and residual add + RMSNorm, residual written back) -> int8 row + scale
+            gain = synth.activations(1, nn, gen)[0].contiguous()
+            sets = [(synth.activations(m, nn, gen), synth.activations(m, nn, gen),
+                     torch.empty((m, nn), dtype=torch.int8, device=dev),
+                     torch.empty(m, dtype=torch.float32, device=dev)) for _ in range(copies)]
+            t = graph_time([lambda s_=s_: lib.cmi_rms_norm_i8(ptr(s_[0]), ptr(gain), None, ptr(s_[2]), ptr(s_[3]), m, nn,
+                                                               nn, nn, 1e-6, cur_stream()) for s_ in sets])
+            prod[f"rms_norm_i8_M{m}_N{nn}"] = hbm_line(t, m * nn * 3 + 2 * nn + 4 * m)
+            t = graph_time([lambda s_=s_: lib.cmi_add_rms_norm_i8(ptr(s_[0]), ptr(s_[1]), ptr(gain), None, ptr(s_[2]),
+                                                                   ptr(s_[3]), m, nn, nn, nn, nn, 1e-6, cur_stream())
+                            for s_ in sets])
+            prod[f"add_rms_norm_i8_M{m}_N{nn}"] = hbm_line(t, m * nn * 7 + 2 * nn + 4 * m)
+            t = graph_time([lambda s_=s_: lib.cmi_quant_act_i8(ptr(s_[0]), ptr(s_[2]), ptr(s_[3]), m, nn, cur_stream())
+                            for s_ in sets])
+            prod[f"quant_act_i8_M{m}_K{nn}"] = hbm_line(t, m * nn * 3 + 4 * m)
+            del sets, gain
+            torch.cuda.empty_cache()
+        extra["fused_producers"] = prod
+        torch.cuda.empty_cache()
+
+        emb = {}
+        q = synth.int8_weight(151936, 2560, gen)
+        for tkn in (1, 2048):
+            sets = [(torch.randint(0, 151936, (tkn,), device=dev, dtype=torch.int64),
+                     torch.empty((tkn, 2560), dtype=torch.bfloat16, device=dev)) for _ in range(8)]
+            t = graph_time([lambda s_=s_: lib.cmi_embed_rows_i8(ptr(q.wq), ptr(q.scale), ptr(s_[0]), ptr(s_[1]), tkn,
+                                                                 151936, 2560, cur_stream()) for s_ in sets])
+            emb[f"int8_T{tkn}_K2560"] = hbm_line(t, tkn * (2560 * 3 + 12))
+            del sets
+        del q
+        extra["embed_rows"] = emb
+        torch.cuda.empty_cache()
+
+        w16 = {}
+        for n_, k_ in ((9728, 2560), (2560, 9728)):
+            copies = 16
+            ws4 = []
+            for _ in range(copies):
+                w = synth.int4_weight(n_, k_, gen)
+                d4 = torch.empty((n_, k_ // 2), dtype=torch.uint8, device=dev)
+                ds = torch.empty((n_, k_ // 128), dtype=torch.float32, device=dev)
+                _native.check(lib.cmi_w4_repack(ptr(w.packed), ptr(w.scale), ptr(d4), ptr(ds), n_, k_, 128, cur_stream()), "repack")
+                ws4.append((d4, ds))
+                del w
+            xv = synth.activations(1, k_, gen)
+            yv = torch.empty((1, n_), dtype=torch.bfloat16, device=dev)
+            def one(ws4=ws4, xv=xv, yv=yv, n_=n_, k_=k_):
+                st = cur_stream()
+                for d4, ds in ws4:
+                    lib.cmi_gemv_w4a16(ptr(d4), ptr(ds), ptr(xv), ptr(yv), n_, k_, 128, st)
+            one()
+            torch.cuda.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                one()
+            t = timed(gr.replay, 5) / copies
+            w16[f"{k_}->{n_}"] = hbm_line(t, synth.w4_gemv_bytes(1, n_, k_))
+            del ws4, gr
+        extra["w4a16_gemv_M1_hipgraph"] = w16
         result["extra"] = extra
 
     # ------------------------------------------------------------------ CPU baseline leg

@@ -77,6 +77,14 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
     return u >> 16;
 }
 
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+// Two fp32 -> packed bf16 (lo in the low half), round to nearest even, one v_cvt_pk_bf16_f32.
+__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
+    const f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
 template <int CTRL, int ROW_MASK>
 __device__ __forceinline__ float dpp_f32(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK,

@@ -15,15 +15,16 @@ namespace {
 
 using namespace cmi;
 
-constexpr int THREADS = 256;
+constexpr int THREADS = 256;       // per row when there are rows enough to fill the chip
+constexpr int MAX_THREADS = 1024;  // per row for a few rows: the row is the only parallelism there is
+constexpr int FEW_ROWS = 256;      // up to this many rows a row gets as many threads as it has vectors
 
 __device__ __forceinline__ float block_max(float v, float *smem) {
     v = wave_max_to_lane63(v);
     if ((threadIdx.x & 63) == 63) smem[threadIdx.x >> 6] = v;
     __syncthreads();
     float r = smem[0];
-#pragma unroll
-    for (int i = 1; i < THREADS / 64; ++i) r = fmaxf(r, smem[i]);
+    for (int i = 1; i < (int)(blockDim.x >> 6); ++i) r = fmaxf(r, smem[i]);
     __syncthreads();  // smem is reused by the caller's next reduction
     return r;
 }
@@ -36,44 +37,56 @@ __device__ __forceinline__ double block_sum(double v, double *smem) {
     if ((threadIdx.x & 63) == 0) smem[threadIdx.x >> 6] = v;
     __syncthreads();
     double r = smem[0];
-#pragma unroll
-    for (int i = 1; i < THREADS / 64; ++i) r += smem[i];
+    for (int i = 1; i < (int)(blockDim.x >> 6); ++i) r += smem[i];
     __syncthreads();
     return r;
 }
 
 // ----------------------------------------------------------------- silu
 
-// bf16(silu(g)) for a bf16 g, equal to g / (1 + exp(-g)) evaluated in fp32 with exp rounded
-// once from its exact value.  The fast evaluation uses the fp32 library exp (about one unit in
-// the last place off); its result is narrowed directly unless it sits within 48 fp32 steps of
-// a bf16 rounding boundary, where the few-step error of the fast route could change the
-// narrowing: those (about 0.15 % of the inputs) are redone with the double-precision exp.
-__device__ __forceinline__ uint32_t silu_bf16_bits(float g) {
-    const float fast = __fdiv_rn(g, 1.f + expf(-g));
-    const uint32_t low = __float_as_uint(fast) & 0xffffu;
-    if (low - (0x8000u - 48u) <= 96u) {
-        const float e = (float)exp((double)(-g));
-        return f32_to_bf16_bits(__fdiv_rn(g, 1.f + e));
-    }
-    return f32_to_bf16_bits(fast);
+// silu(g) for a bf16 g as the fp32 value whose narrowing is the result: g / (1 + exp(-g))
+// evaluated in fp32 with exp rounded once from its exact value.  The fast evaluation --
+// exp(-g) = 2^p (1 + r ln 2) with p + r = -g log2(e) split exactly by an fma, v_exp_f32, v_rcp_f32 --
+// is within 3 fp32 steps of that value for every bf16 g with |g| < 64 (measured over all of
+// them); it is used unless it sits within 8 steps of a bf16 rounding boundary, where those few
+// steps could change the narrowing: such inputs (0.02 %) and |g| >= 64, infinities and NaN take
+// the double-precision exp and the correctly rounded division.
+__device__ __forceinline__ float silu_exact_f32(float g) {
+    const float e = (float)exp((double)(-g));
+    return __fdiv_rn(g, 1.f + e);
 }
+
+__device__ __forceinline__ float silu_f32(float g) {
+    if (!(fabsf(g) < 64.f)) return silu_exact_f32(g);
+    constexpr float LOG2E = 1.44269502e+00f, LOG2E_LO = 1.92596299e-08f, LN2 = 0.693147182f;
+    const float ng = -g;
+    const float p = __fmul_rn(ng, LOG2E);
+    const float r = __fadd_rn(__fmaf_rn(ng, LOG2E, -p), __fmul_rn(ng, LOG2E_LO));
+    const float ep = __builtin_amdgcn_exp2f(p);
+    const float e = __fmaf_rn(__fmul_rn(ep, LN2), r, ep);
+    const float fast = __fmul_rn(g, __builtin_amdgcn_rcpf(__fadd_rn(1.f, e)));
+    const uint32_t low = __float_as_uint(fast) & 0xffffu;
+    if (low - (0x8000u - 8u) <= 16u) return silu_exact_f32(g);
+    return fast;
+}
+
+__device__ __forceinline__ uint32_t silu_bf16_bits(float g) { return pack2_bf16(silu_f32(g), 0.f) & 0xffffu; }
 
 // product of two bf16 values as torch forms it: one fp32 multiply, one narrowing
 __device__ __forceinline__ uint32_t mul_bf16_bits(uint32_t a_bits, float b) {
-    return f32_to_bf16_bits(__fmul_rn(bf16_bits_to_f32(a_bits), b));
+    return pack2_bf16(__fmul_rn(bf16_bits_to_f32(a_bits), b), 0.f) & 0xffffu;
 }
 
+// eight elements: bf16(bf16(silu(g)) * u), two per dword
 __device__ __forceinline__ uint4 silu_mul8(const uint4 &g, const uint4 &u) {
     const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
     uint32_t o[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const uint32_t lo = mul_bf16_bits(silu_bf16_bits(bf16_bits_to_f32(gw[i] & 0xffffu)),
-                                          bf16_bits_to_f32(uw[i] & 0xffffu));
-        const uint32_t hi = mul_bf16_bits(silu_bf16_bits(__uint_as_float(gw[i] & 0xffff0000u)),
-                                          __uint_as_float(uw[i] & 0xffff0000u));
-        o[i] = lo | (hi << 16);
+        const uint32_t s2 = pack2_bf16(silu_f32(bf16_bits_to_f32(gw[i] & 0xffffu)),
+                                       silu_f32(__uint_as_float(gw[i] & 0xffff0000u)));
+        o[i] = pack2_bf16(__fmul_rn(bf16_bits_to_f32(s2 & 0xffffu), bf16_bits_to_f32(uw[i] & 0xffffu)),
+                          __fmul_rn(__uint_as_float(s2 & 0xffff0000u), __uint_as_float(uw[i] & 0xffff0000u)));
     }
     return make_uint4(o[0], o[1], o[2], o[3]);
 }
@@ -88,9 +101,11 @@ struct SiluArgs {
 };
 
 // K % 8 == 0, every row 16-byte aligned.  VPT > 0: the row fits VPT vectors per thread.
-template <int VPT>
-__global__ void __launch_bounds__(THREADS) silu_mul_quant_vec(SiluArgs a) {
-    __shared__ float smem[THREADS / 64];
+// T_MAX: the most threads a launch gives a row (blockDim.x is what it gives).
+template <int VPT, int T_MAX = THREADS>
+__global__ void __launch_bounds__(T_MAX) silu_mul_quant_vec(SiluArgs a) {
+    __shared__ float smem[MAX_THREADS / 64];
+    const int T = blockDim.x;
     const int row = blockIdx.x, nvec = a.K / 8;
     const uint4 *gr = reinterpret_cast<const uint4 *>(a.gate + (size_t)row * a.ldg);
     const uint4 *ur = reinterpret_cast<const uint4 *>(a.up + (size_t)row * a.ldu);
@@ -99,7 +114,7 @@ __global__ void __launch_bounds__(THREADS) silu_mul_quant_vec(SiluArgs a) {
     float amax = 0.f;
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-        const int idx = threadIdx.x + i * THREADS;
+        const int idx = threadIdx.x + i * T;
         if (idx < nvec) {
             v[i] = silu_mul8(gr[idx], ur[idx]);
             if (orow) orow[idx] = v[i];  // may overwrite up[idx]: read above by this same thread
@@ -116,7 +131,7 @@ __global__ void __launch_bounds__(THREADS) silu_mul_quant_vec(SiluArgs a) {
     uint2 *qr = reinterpret_cast<uint2 *>(a.q + (size_t)row * a.K);
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-        const int idx = threadIdx.x + i * THREADS;
+        const int idx = threadIdx.x + i * T;
         if (idx < nvec) qr[idx] = quant8(v[i], rs);
     }
 }
@@ -125,7 +140,7 @@ __global__ void __launch_bounds__(THREADS) silu_mul_quant_vec(SiluArgs a) {
 // product is recomputed for the quantiser (cheaper than depending on a bf16 copy that the
 // caller may not have asked for).
 __global__ void __launch_bounds__(THREADS) silu_mul_quant_scalar(SiluArgs a) {
-    __shared__ float smem[THREADS / 64];
+    __shared__ float smem[MAX_THREADS / 64];
     const int row = blockIdx.x;
     const uint16_t *gr = a.gate + (size_t)row * a.ldg, *ur = a.up + (size_t)row * a.ldu;
     int8_t *qr = a.q ? a.q + (size_t)row * a.K : nullptr;
@@ -168,16 +183,30 @@ __device__ __forceinline__ float inv_rms(double ss, int N, float eps) {
     return __fdiv_rn(1.0f, __fsqrt_rn(ms + eps));
 }
 
-__device__ __forceinline__ uint32_t add_bf16_bits(float a, float b) { return f32_to_bf16_bits(__fadd_rn(a, b)); }
+__device__ __forceinline__ uint32_t add_bf16_bits(float a, float b) { return pack2_bf16(__fadd_rn(a, b), 0.f) & 0xffffu; }
 
 __device__ __forceinline__ uint32_t norm1(float x, float scale, float w) {
-    return mul_bf16_bits(f32_to_bf16_bits(__fmul_rn(x, scale)), w);
+    return mul_bf16_bits(pack2_bf16(__fmul_rn(x, scale), 0.f) & 0xffffu, w);
 }
 
-template <int VPT>
-__global__ void __launch_bounds__(THREADS) rms_norm_i8_vec(NormArgs a) {
-    __shared__ double dsmem[THREADS / 64];
-    __shared__ float smem[THREADS / 64];
+// the two bf16 of a dword at once: bf16(bf16(x * scale) * w)
+__device__ __forceinline__ uint32_t norm2(uint32_t xw, float scale, uint32_t gw) {
+    const uint32_t t = pack2_bf16(__fmul_rn(bf16_bits_to_f32(xw & 0xffffu), scale),
+                                  __fmul_rn(__uint_as_float(xw & 0xffff0000u), scale));
+    return pack2_bf16(__fmul_rn(bf16_bits_to_f32(t & 0xffffu), bf16_bits_to_f32(gw & 0xffffu)),
+                      __fmul_rn(__uint_as_float(t & 0xffff0000u), __uint_as_float(gw & 0xffff0000u)));
+}
+
+__device__ __forceinline__ uint32_t add2(uint32_t xw, uint32_t dw) {
+    return pack2_bf16(__fadd_rn(bf16_bits_to_f32(xw & 0xffffu), bf16_bits_to_f32(dw & 0xffffu)),
+                      __fadd_rn(__uint_as_float(xw & 0xffff0000u), __uint_as_float(dw & 0xffff0000u)));
+}
+
+template <int VPT, int T_MAX = THREADS>
+__global__ void __launch_bounds__(T_MAX) rms_norm_i8_vec(NormArgs a) {
+    __shared__ double dsmem[MAX_THREADS / 64];
+    __shared__ float smem[MAX_THREADS / 64];
+    const int T = blockDim.x;
     const int row = blockIdx.x, nvec = a.N / 8;
     uint4 *xr = reinterpret_cast<uint4 *>(a.x + (size_t)row * a.ldx);
     const uint4 *ar = a.add ? reinterpret_cast<const uint4 *>(a.add + (size_t)row * a.lda) : nullptr;
@@ -186,7 +215,7 @@ __global__ void __launch_bounds__(THREADS) rms_norm_i8_vec(NormArgs a) {
     double ss = 0.0;
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-        const int idx = threadIdx.x + i * THREADS;
+        const int idx = threadIdx.x + i * T;
         if (idx < nvec) {
             v[i] = xr[idx];
             if (ar) {
@@ -194,9 +223,7 @@ __global__ void __launch_bounds__(THREADS) rms_norm_i8_vec(NormArgs a) {
                 const uint32_t xw[4] = {v[i].x, v[i].y, v[i].z, v[i].w}, dw[4] = {d.x, d.y, d.z, d.w};
                 uint32_t o[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    o[j] = add_bf16_bits(bf16_bits_to_f32(xw[j] & 0xffffu), bf16_bits_to_f32(dw[j] & 0xffffu)) |
-                           (add_bf16_bits(__uint_as_float(xw[j] & 0xffff0000u), __uint_as_float(dw[j] & 0xffff0000u)) << 16);
+                for (int j = 0; j < 4; ++j) o[j] = add2(xw[j], dw[j]);
                 v[i] = make_uint4(o[0], o[1], o[2], o[3]);
                 xr[idx] = v[i];  // the residual stream keeps the sum
             }
@@ -217,15 +244,13 @@ __global__ void __launch_bounds__(THREADS) rms_norm_i8_vec(NormArgs a) {
     float amax = 0.f;
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-        const int idx = threadIdx.x + i * THREADS;
+        const int idx = threadIdx.x + i * T;
         if (idx < nvec) {
             const uint4 g = wr[idx];
             const uint32_t xw[4] = {v[i].x, v[i].y, v[i].z, v[i].w}, gw[4] = {g.x, g.y, g.z, g.w};
             uint32_t o[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                o[j] = norm1(bf16_bits_to_f32(xw[j] & 0xffffu), scale, bf16_bits_to_f32(gw[j] & 0xffffu)) |
-                       (norm1(__uint_as_float(xw[j] & 0xffff0000u), scale, __uint_as_float(gw[j] & 0xffff0000u)) << 16);
+            for (int j = 0; j < 4; ++j) o[j] = norm2(xw[j], scale, gw[j]);
             v[i] = make_uint4(o[0], o[1], o[2], o[3]);
             if (yr) yr[idx] = v[i];
             amax = absmax8(v[i], amax);
@@ -238,7 +263,72 @@ __global__ void __launch_bounds__(THREADS) rms_norm_i8_vec(NormArgs a) {
     uint2 *qr = reinterpret_cast<uint2 *>(a.q + (size_t)row * a.N);
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
-        const int idx = threadIdx.x + i * THREADS;
+        const int idx = threadIdx.x + i * T;
+        if (idx < nvec) qr[idx] = quant8(v[i], rs);
+    }
+}
+
+// Short rows (N <= 4096): one wavefront per row, VPT vectors per lane.  The sum of squares and
+// the absmax are reduced inside the wavefront, so a row costs no LDS and no barrier -- with one
+// workgroup per 5 KB row the three barriers were most of the row's latency (8192 x 2560:
+// 22 -> 13 us).  Same arithmetic, same bits.
+template <int VPT>
+__global__ void __launch_bounds__(THREADS) rms_norm_i8_wave(NormArgs a, int rows) {
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * (THREADS / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;  // whole wavefronts: nothing below synchronises across them
+    const int nvec = a.N / 8;
+    uint4 *xr = reinterpret_cast<uint4 *>(a.x + (size_t)row * a.ldx);
+    const uint4 *ar = a.add ? reinterpret_cast<const uint4 *>(a.add + (size_t)row * a.lda) : nullptr;
+    const uint4 *wr = reinterpret_cast<const uint4 *>(a.w);
+    uint4 v[VPT];
+    double ss = 0.0;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int idx = lane + i * 64;
+        if (idx < nvec) {
+            v[i] = xr[idx];
+            if (ar) {
+                const uint4 d = ar[idx];
+                v[i] = make_uint4(add2(v[i].x, d.x), add2(v[i].y, d.y), add2(v[i].z, d.z), add2(v[i].w, d.w));
+                xr[idx] = v[i];  // the residual stream keeps the sum
+            }
+            const uint32_t w4[4] = {v[i].x, v[i].y, v[i].z, v[i].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const double lo = (double)bf16_bits_to_f32(w4[j] & 0xffffu);
+                const double hi = (double)__uint_as_float(w4[j] & 0xffff0000u);
+                ss = fma(lo, lo, ss);
+                ss = fma(hi, hi, ss);
+            }
+        } else {
+            v[i] = make_uint4(0, 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);  // exact addends: any order
+    const float scale = inv_rms(ss, a.N, a.eps);
+    uint4 *yr = a.y ? reinterpret_cast<uint4 *>(a.y + (size_t)row * a.ldy) : nullptr;
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int idx = lane + i * 64;
+        if (idx < nvec) {
+            const uint4 g = wr[idx];
+            v[i] = make_uint4(norm2(v[i].x, scale, g.x), norm2(v[i].y, scale, g.y), norm2(v[i].z, scale, g.z),
+                              norm2(v[i].w, scale, g.w));
+            if (yr) yr[idx] = v[i];
+            amax = absmax8(v[i], amax);
+        }
+    }
+    if (!a.q) return;
+    amax = lane63(wave_max_to_lane63(amax));
+    const RowScale rs = row_scale(amax);
+    if (lane == 0) a.s[row] = rs.sc;
+    uint2 *qr = reinterpret_cast<uint2 *>(a.q + (size_t)row * a.N);
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int idx = lane + i * 64;
         if (idx < nvec) qr[idx] = quant8(v[i], rs);
     }
 }
@@ -246,8 +336,8 @@ __global__ void __launch_bounds__(THREADS) rms_norm_i8_vec(NormArgs a) {
 // Any N, pitch and alignment.  Needs a bf16 destination for the normalised row when quantising
 // (y, or the quantiser would have to recompute it a third time): the host passes one.
 __global__ void __launch_bounds__(THREADS) rms_norm_i8_scalar(NormArgs a) {
-    __shared__ double dsmem[THREADS / 64];
-    __shared__ float smem[THREADS / 64];
+    __shared__ double dsmem[MAX_THREADS / 64];
+    __shared__ float smem[MAX_THREADS / 64];
     const int row = blockIdx.x;
     uint16_t *xr = a.x + (size_t)row * a.ldx;
     const uint16_t *ar = a.add ? a.add + (size_t)row * a.lda : nullptr;
@@ -301,7 +391,22 @@ int norm_entry(const char *who, uint16_t *x, const uint16_t *add, const void *w,
     const bool vec = N % 8 == 0 && vpt <= 16 && aligned(x, 16) && ldx % 8 == 0 && aligned(w, 16) &&
                      (!add || (aligned(add, 16) && lda % 8 == 0)) && (!y || (aligned(y, 16) && ldy % 8 == 0)) &&
                      (!q || aligned(q, 8));
-    if (vec)
+    if (vec && M <= FEW_ROWS && nvec <= 2 * MAX_THREADS) {
+        // a few rows: latency, not throughput -- every vector of the row gets a thread of its own
+        const int t = nvec <= MAX_THREADS ? (nvec + 63) / 64 * 64 : MAX_THREADS;
+        if (nvec <= MAX_THREADS) rms_norm_i8_vec<1, MAX_THREADS><<<dim3(M), dim3(t), 0, st>>>(a);
+        else rms_norm_i8_vec<2, MAX_THREADS><<<dim3(M), dim3(t), 0, st>>>(a);
+    } else if (vec && nvec <= 8 * 64) {
+        const dim3 grid((M + THREADS / 64 - 1) / (THREADS / 64)), block(THREADS);
+        const int wvpt = (nvec + 63) / 64;
+        if (wvpt <= 1) rms_norm_i8_wave<1><<<grid, block, 0, st>>>(a, M);
+        else if (wvpt <= 2) rms_norm_i8_wave<2><<<grid, block, 0, st>>>(a, M);
+        else if (wvpt <= 3) rms_norm_i8_wave<3><<<grid, block, 0, st>>>(a, M);
+        else if (wvpt <= 4) rms_norm_i8_wave<4><<<grid, block, 0, st>>>(a, M);
+        else if (wvpt <= 5) rms_norm_i8_wave<5><<<grid, block, 0, st>>>(a, M);
+        else if (wvpt <= 6) rms_norm_i8_wave<6><<<grid, block, 0, st>>>(a, M);
+        else rms_norm_i8_wave<8><<<grid, block, 0, st>>>(a, M);
+    } else if (vec)
         launch_vpt(vpt, a, M, st, rms_norm_i8_vec<1>, rms_norm_i8_vec<2>, rms_norm_i8_vec<4>, rms_norm_i8_vec<8>,
                    rms_norm_i8_vec<16>);
     else
@@ -326,7 +431,12 @@ extern "C" int cmi_silu_mul_quant(const void *gate, const void *up, void *out, i
     const int nvec = K / 8, vpt = (nvec + THREADS - 1) / THREADS;
     const bool vec = K % 8 == 0 && vpt <= 16 && aligned(gate, 16) && aligned(up, 16) && ld_gate % 8 == 0 &&
                      ld_up % 8 == 0 && (!out || (aligned(out, 16) && ld_out % 8 == 0)) && (!out_q || aligned(out_q, 8));
-    if (vec)
+    if (vec && M <= FEW_ROWS && nvec <= 2 * MAX_THREADS) {
+        // a few rows: latency, not throughput -- every vector of the row gets a thread of its own
+        const int t = nvec <= MAX_THREADS ? (nvec + 63) / 64 * 64 : MAX_THREADS;
+        if (nvec <= MAX_THREADS) silu_mul_quant_vec<1, MAX_THREADS><<<dim3(M), dim3(t), 0, st>>>(a);
+        else silu_mul_quant_vec<2, MAX_THREADS><<<dim3(M), dim3(t), 0, st>>>(a);
+    } else if (vec)
         launch_vpt(vpt, a, M, st, silu_mul_quant_vec<1>, silu_mul_quant_vec<2>, silu_mul_quant_vec<4>,
                    silu_mul_quant_vec<8>, silu_mul_quant_vec<16>);
     else
