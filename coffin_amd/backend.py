@@ -434,6 +434,55 @@ def linear_prefill(w, x: torch.Tensor) -> torch.Tensor:
     return _project(w, x, prefill=True, mfma=True)
 
 
+def linear_quantized(w, xq: torch.Tensor, xs: torch.Tensor) -> torch.Tensor:
+    """Projection of rows that arrive already quantised: ``xq`` int8 ``[M, K]`` and ``xs`` fp32
+    ``[M]`` as written by :func:`rms_norm_i8` / :func:`silu_mul_quant` / :func:`kv_quant`, result
+    bf16 ``[M, N]`` -- W8A8 for an int8 weight, W4A8 for an int4 one, bit for bit what
+    ``linear_prefill`` (int8, from 64 rows) or ``linear`` (int4) returns for the bf16 rows those
+    were quantised from, without reading them again.  Not a table entry of the contract (the
+    reference consumes quantised rows inside its own MoE ops, models/qwen35/moe.py:306-307,
+    backends/corex/__init__.py:736-760); offered to callers that fuse a norm or an activation with
+    the projection behind it."""
+    if not (_is_w4(w) or _is_q8(w)):
+        raise ValueError("linear_quantized needs a quantized weight")
+    if xq.dim() != 2 or xq.dtype != torch.int8 or xs.dtype != torch.float32 or xs.numel() != xq.shape[0]:
+        raise ValueError("linear_quantized expects xq int8 [M, K] and xs fp32 [M]")
+    if not (_on_gpu(xq) and xs.device == xq.device and xq.is_contiguous() and xs.is_contiguous()):
+        raise ValueError("linear_quantized: xq and xs must be contiguous on one GPU")
+    rec = _lookup(w)
+    if rec is None:
+        if not _kernels_take(w):
+            raise ValueError("linear_quantized: the kernels are not built for this weight's shape")
+        wdev = (w.packed if _is_w4(w) else w.wq).device
+        if wdev != xq.device:
+            raise ValueError(f"weight on {wdev} and activation on {xq.device} must share a device")
+        if _current_device() != xq.device.index:
+            with torch.cuda.device(xq.device):
+                return linear_quantized(w, xq, xs)
+        rec = _make_record(w)
+    if rec.dev != xq.device:
+        raise ValueError(f"weight on {rec.dev} and activation on {xq.device} must share a device")
+    if _current_device() != xq.device.index:
+        with torch.cuda.device(xq.device):
+            return linear_quantized(w, xq, xs)
+    rows, k = xq.shape
+    if k != rec.k:
+        raise ValueError(f"linear_quantized expects K={rec.k}, got {k}")
+    out = torch.empty((rows, rec.n), dtype=torch.bfloat16, device=xq.device)
+    if rows == 0:
+        return out
+    lib = _native.load()
+    if rec.kind == 4:
+        fn = lib.cmi_gemv_w4a8 if rows <= 16 else lib.cmi_gemm_w4a8
+        rc = fn(rec.a, rec.b, xq.data_ptr(), xs.data_ptr(), out.data_ptr(), None, rows, rec.n, k, rec.gs, _stream())
+    else:
+        rc = lib.cmi_gemm_w8a8(xq.data_ptr(), rec.a, xs.data_ptr(), rec.b, out.data_ptr(), None, rows, rec.n, k,
+                               rec.n, _stream())
+    if rc:
+        _native.check(rc, "linear_quantized")
+    return out
+
+
 def kv_quant(x: torch.Tensor, out_q: torch.Tensor, out_s: torch.Tensor) -> torch.Tensor:
     """Per-row symmetric int8 quantisation into caller-owned ``out_q`` / ``out_s``.
 

@@ -341,6 +341,44 @@ def test_kv_quant_writes_through_caller_buffers(orc):
     assert (out_q.cpu().numpy() == q).all()
 
 
+@pytest.mark.parametrize("rows", [1, 3, 16, 70, 200])
+def test_quantised_rows_feed_the_projection_behind_a_fused_producer(rows):
+    """rms_norm_i8 / silu_mul_quant write int8 rows + scales; linear_quantized consumes them.  The
+    result carries the bits of the bf16 route (norm written as bf16, then the projection that
+    quantises for itself): W4A8 at every row count, W8A8 through linear_prefill from 64 rows."""
+    g = synth.generator(11)
+    k, n = 2560, 1024
+    x = synth.activations(rows, k, g).to(G.DEV)
+    gain = synth.activations(1, k, g)[0].to(G.DEV).contiguous()
+    xq = torch.empty((rows, k), dtype=torch.int8, device=G.DEV)
+    xs = torch.empty(rows, dtype=torch.float32, device=G.DEV)
+    y_bf16 = torch.empty_like(x)
+    backend.rms_norm_i8(x, gain, xq, xs, out=y_bf16)
+    w4, q8 = _w4(n, k, g), _q8(n, k, g)
+    got4 = backend.linear_quantized(w4, xq, xs)
+    want4 = backend.linear(w4, y_bf16)
+    assert (got4.view(torch.int16) == want4.view(torch.int16)).all()
+    got8 = backend.linear_quantized(q8, xq, xs)
+    if rows >= 64:
+        want8 = backend.linear_prefill(q8, y_bf16)
+        assert (got8.view(torch.int16) == want8.view(torch.int16)).all()
+    else:
+        # below 64 rows linear_prefill stays weight-only: compare with quantiser + W8A8 run separately
+        q2, s2 = torch.empty_like(xq), torch.empty_like(xs)
+        backend.kv_quant(y_bf16, q2, s2)
+        assert (q2 == xq).all() and (s2.view(torch.int32) == xs.view(torch.int32)).all()
+        assert (backend.linear_quantized(q8, q2, s2).view(torch.int16) == got8.view(torch.int16)).all()
+    # the SwiGLU product in front of a down projection
+    gu = synth.activations(rows, 2 * k, g).to(G.DEV)
+    prod = torch.empty((rows, k), dtype=torch.bfloat16, device=G.DEV)
+    backend.silu_mul_quant(gu[:, :k], gu[:, k:], prod, xq, xs)
+    assert (backend.linear_quantized(w4, xq, xs).view(torch.int16) == backend.linear(w4, prod).view(torch.int16)).all()
+    with pytest.raises(ValueError):
+        backend.linear_quantized(w4, xq[:, :128], xs)
+    with pytest.raises(ValueError):
+        backend.linear_quantized(w4, xq.to(torch.int16), xs)
+
+
 def test_gemv_objects_on_device():
     g = synth.generator()
     qa, qb = _q8(512, 2560, g), _q8(256, 2560, g)
