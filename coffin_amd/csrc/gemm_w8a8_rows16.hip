@@ -65,6 +65,11 @@ gemm_w8a8_rows16_kernel(const Args a) {
                 reinterpret_cast<const v4i32 *>(a.wq + tile_src(lane, h, n0, a.N - 1, a.K, line * LINE)));
     }
 
+    // the scales of the output this thread will finish, requested behind the operands: asked for at
+    // the end they are cold loads under a saturated memory system
+    const float ws_out = a.ws[min(n0 + (int)((threadIdx.x >> 2) & 15), a.N - 1)];
+    const float xs_out = a.xs[min((int)(4 * ((threadIdx.x >> 6) & 3) + (threadIdx.x & 3)), a.M - 1)];
+
     // into the MFMA arrangement (lane: row lane%16, pieces kq and 4+kq), then the products;
     // the accumulator of lane l holds (n = l%16, m = 4*kq + v), v = 0..3
     v4i32 acc = {0, 0, 0, 0};
@@ -96,7 +101,7 @@ gemm_w8a8_rows16_kernel(const Args a) {
 #pragma unroll
             for (int wv = 0; wv < WAVES; ++wv) s += partial[wv][l][v];
             if (a.acc_out) a.acc_out[(size_t)m * a.N + n] = s;
-            a.y[(size_t)m * a.ldy + n] = (uint16_t)f32_to_bf16_bits(((float)s * a.xs[m]) * a.ws[n]);
+            a.y[(size_t)m * a.ldy + n] = (uint16_t)f32_to_bf16_bits(((float)s * xs_out) * ws_out);
         }
     }
 }
@@ -145,6 +150,9 @@ gemm_w8a8_rows128_kernel(const Args a) {
         for (int h = 0; h < 2; ++h)
             wr[i][h] = __builtin_nontemporal_load(
                 reinterpret_cast<const v4i32 *>(a.wq + tile_src(lane, h, n0, a.N - 1, a.K, line_of(i) * LINE)));
+    // the column scale of the outputs this thread will finish (n depends on the thread only),
+    // requested behind the operands instead of cold at the end
+    const float ws_out = a.ws[min(n0 + (int)((threadIdx.x >> 2) & 15), a.N - 1)];
     for (int o = threadIdx.x; o < chunks * 256; o += WAVES * 64) (&sums[0][0][0])[o] = 0;
     __syncthreads();
 #pragma unroll
@@ -180,7 +188,7 @@ gemm_w8a8_rows128_kernel(const Args a) {
         if (n < a.N && m < a.M) {
             const int sm = sums[c][l][v];
             if (a.acc_out) a.acc_out[(size_t)m * a.N + n] = sm;
-            a.y[(size_t)m * a.ldy + n] = (uint16_t)f32_to_bf16_bits(((float)sm * a.xs[m]) * a.ws[n]);
+            a.y[(size_t)m * a.ldy + n] = (uint16_t)f32_to_bf16_bits(((float)sm * a.xs[m]) * ws_out);
         }
     }
 }

@@ -116,6 +116,10 @@ gemv_w4a8_rows16_kernel(const Args a) {
             }
         }
     }
+    // the activation scale of the output this thread will finish (m depends on the thread only),
+    // requested now instead of cold at the end
+    float xs_out = 0.f;
+    if constexpr (!FUSED) xs_out = a.xs[min((int)(4 * ((threadIdx.x >> 6) & 3) + (threadIdx.x & 3)), a.M - 1)];
     // 2. the scales of the 16 rows (contiguous), into registers until the weights are asked for
     const int ws_total = min(ROWS, a.N - n0) * a.G;
     constexpr int WSN = (ROWS * (MAX_K / GS) + WAVES * 64 - 1) / (WAVES * 64);
@@ -263,7 +267,7 @@ gemv_w4a8_rows16_kernel(const Args a) {
                 if constexpr (DUMP) a.group_acc[((size_t)m * a.G + g) * a.N + n] = sg;
                 total = fmaf((float)sg, wsn[g], total);
             }
-            const float xsm = FUSED ? xs_lds[m] : a.xs[m];
+            const float xsm = FUSED ? xs_lds[m] : xs_out;
             a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * xsm);
         }
     }

@@ -261,6 +261,10 @@ gemv_w8a16_kernel(const GemvArgs a) {
         const int n = rb * R + r;
         scale[r] = a.ws[(n < a.N ? n : a.N - 1) + vzero];
     }
+    // several units: the lane that adds the unit totals of output (r, m) = (lane / M, lane % M)
+    // scales it; its scale is requested here, not cold at the end
+    float scale_fin = 0.f;
+    if constexpr (MODE != 0) scale_fin = a.ws[min(rb * R + min(lane / M, R - 1), a.N - 1)];
     if constexpr (XLDS) {
 #pragma unroll
         for (int j = 0; j < XV; ++j) {
@@ -390,7 +394,7 @@ gemv_w8a16_kernel(const GemvArgs a) {
             if (n < a.N && m < a.M) {
                 float total = unit_total[lane];
                 for (int v = 1; v < a.units; ++v) total += unit_total[v * (R * M) + lane];
-                a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(a.ws[n] * total);
+                a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(scale_fin * total);
             }
         }
     }
