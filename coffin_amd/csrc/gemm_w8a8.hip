@@ -64,11 +64,12 @@ struct Cfg {
     static constexpr int BN = 64 * TN, BM = 64 * TM;
     static constexpr int W_BYTES = BN * BK, X_BYTES = BM * BK;
     static constexpr int STAGE_BYTES = W_BYTES + X_BYTES;
-    static constexpr int LDS_BYTES = NST * STAGE_BYTES;
+    static constexpr int SCALE_BYTES = 4 * (BN + BM);   // the tile's scales, behind the stages
+    static constexpr int LDS_BYTES = NST * STAGE_BYTES + SCALE_BYTES;
     static constexpr int WL = BN / 32, XL = BM / 32;  // loads per wavefront and stage (8 rows each)
     static constexpr int LPW = WL + XL;
     static constexpr int PITCH = 64 * TN + 16;        // epilogue: one m row of the wavefront tile + 16 B
-    static_assert(4 * 32 * TM * PITCH <= LDS_BYTES, "epilogue does not fit the operand stages");
+    static_assert(4 * 32 * TM * PITCH <= NST * STAGE_BYTES, "epilogue does not fit the operand stages");
     static_assert((NST - 2) * LPW <= 63, "vmcnt range");
 };
 
@@ -107,6 +108,14 @@ __device__ __forceinline__ void tile_coords(const Args &a, int &tm, int &tn) {
     tm = first_m + (in_band - tn * rows);
 }
 
+// Scales of a BN x BM block tile into LDS at `dst` (BN column scales, then BM row scales), indices
+// clamped to the matrix; read again only behind the barrier that opens the epilogue.
+template <int BN, int BM>
+__device__ __forceinline__ void stage_scales(const Args &a, float *dst, int n0, int m0) {
+    for (int i = threadIdx.x; i < BN + BM; i += blockDim.x)
+        dst[i] = i < BN ? a.ws[min(n0 + i, a.N - 1)] : a.xs[min(m0 + i - BN, a.M - 1)];
+}
+
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
 
@@ -123,9 +132,13 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 // rows back 16 bytes per lane.  Every wavefront of the workgroup must call it
 // (one barrier inside: the operand stages are reused as parking space).
 // JP: m tiles parked per pass (the parking space of a wavefront is 32*JP rows); TM % JP == 0.
+// ws_tile / xs_tile (nullable): the scales of the block tile staged in LDS by the kernel's prologue,
+// indexed from the wavefront tile's corner (ws_tile[0] is ws[nb], xs_tile[0] is xs[mb]); fetched from
+// global memory here they are cold loads at the head of the epilogue.
 template <int TN, int TM, int JP = TM>
 __device__ __forceinline__ void epilogue(const Args &a, v16i32 (&acc)[TN][TM], int8_t *lds, int wave,
-                                         int lane, int nb, int mb) {
+                                         int lane, int nb, int mb, const float *ws_tile = nullptr,
+                                         const float *xs_tile = nullptr) {
     if (a.acc_out) {
 #pragma unroll
         for (int i = 0; i < TN; ++i)
@@ -151,7 +164,10 @@ __device__ __forceinline__ void epilogue(const Args &a, v16i32 (&acc)[TN][TM], i
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const int n = nb + i * 32 + 8 * q + 4 * (lane >> 5);
-            if (n + 3 < a.N) {
+            if (ws_tile) {
+                const float4 sc = *reinterpret_cast<const float4 *>(ws_tile + (n - nb));
+                wsv[i][q][0] = sc.x, wsv[i][q][1] = sc.y, wsv[i][q][2] = sc.z, wsv[i][q][3] = sc.w;
+            } else if (n + 3 < a.N) {
                 const float4 sc = *reinterpret_cast<const float4 *>(a.ws + n);
                 wsv[i][q][0] = sc.x, wsv[i][q][1] = sc.y, wsv[i][q][2] = sc.z, wsv[i][q][3] = sc.w;
             } else {
@@ -168,7 +184,7 @@ __device__ __forceinline__ void epilogue(const Args &a, v16i32 (&acc)[TN][TM], i
         for (int jj = 0; jj < JP; ++jj) {
             const int j = j0 + jj;
             const int ml = jj * 32 + (lane & 31);
-            const float xm = a.xs[min(mb + j * 32 + (lane & 31), a.M - 1)];
+            const float xm = xs_tile ? xs_tile[j * 32 + (lane & 31)] : a.xs[min(mb + j * 32 + (lane & 31), a.M - 1)];
 #pragma unroll
             for (int i = 0; i < TN; ++i)
 #pragma unroll
@@ -225,6 +241,8 @@ gemm_w8a8_pipe_kernel(const Args a) {
     int tm, tn;
     tile_coords(a, tm, tn);
     const int m0 = tm * C::BM, n0 = tn * C::BN;
+    float *scales = reinterpret_cast<float *>(lds + NST * C::STAGE_BYTES);
+    stage_scales<C::BN, C::BM>(a, scales, n0, m0);
 
     // Global side of the direct loads.  One load instruction moves 8 rows x 128 B
     // (whole cache lines) into 1 KiB of LDS; each wavefront fills a contiguous run
@@ -356,7 +374,8 @@ gemm_w8a8_pipe_kernel(const Args a) {
     }
     if (ks < ksteps) step(drain_t{}, ks, w0, x0, w1, x1);
 
-    epilogue<TN, TM>(a, acc, lds, wave, lane, n0 + wn * 32 * TN, m0 + wm * 32 * TM);
+    epilogue<TN, TM>(a, acc, lds, wave, lane, n0 + wn * 32 * TN, m0 + wm * 32 * TM, scales + wn * 32 * TN,
+                     scales + C::BN + wm * 32 * TM);
 }
 
 template <int TN, int TM, int NST>
@@ -561,7 +580,8 @@ namespace wide {
 constexpr int BM = 256, BN = 320, TN = 5, TM = 2;
 constexpr int W_BYTES = BN * BK, X_BYTES = BM * BK, STAGE_BYTES = W_BYTES + X_BYTES;
 constexpr int PARK_BYTES = 8 * 32 * (64 * TN + 16);  // one m tile per epilogue pass
-constexpr int LDS_BYTES = 2 * STAGE_BYTES > PARK_BYTES ? 2 * STAGE_BYTES : PARK_BYTES;
+constexpr int OPERAND_BYTES = 2 * STAGE_BYTES > PARK_BYTES ? 2 * STAGE_BYTES : PARK_BYTES;
+constexpr int LDS_BYTES = OPERAND_BYTES + 4 * (BN + BM);  // the tile's scales behind the stages
 constexpr int WL = 5, XL = 4;  // loads per wavefront and stage
 }  // namespace wide
 
@@ -576,6 +596,8 @@ gemm_w8a8_wide_kernel(const Args a) {
     int tm, tn;
     tile_coords(a, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
+    float *scales = reinterpret_cast<float *>(lds + OPERAND_BYTES);
+    stage_scales<BN, BM>(a, scales, n0, m0);
 
     // Wavefront w fills W rows 40w .. 40w+39 and X rows 32w .. 32w+31 (8 rows x 128 B per load).
     // Addresses are a uniform base (tile corner, advanced by the k step) plus a 32-bit lane
@@ -697,7 +719,8 @@ gemm_w8a8_wide_kernel(const Args a) {
     for (; ks + 2 < ksteps; ++ks) step(issue_t{}, ks);
     for (; ks < ksteps; ++ks) step(drain_t{}, ks);
 
-    epilogue<TN, TM, 1>(a, acc, lds, wave, lane, n0 + wn * 32 * TN, m0 + wm * 32 * TM);
+    epilogue<TN, TM, 1>(a, acc, lds, wave, lane, n0 + wn * 32 * TN, m0 + wm * 32 * TM, scales + wn * 32 * TN,
+                        scales + BN + wm * 32 * TM);
 }
 
 int launch_wide(Args &a, hipStream_t st) {
