@@ -1,5 +1,6 @@
 // W4A8 decode GEMV with the fp32 chain kept in registers: bf16 or already quantised activations,
-// one or two rows, rows short enough that one wavefront can request all of them up front.
+// one or two rows, every wavefront requesting all of its weight bytes up front (K <= 5120 per
+// wavefront; longer rows, up to 20480, are shared by two to eight wavefronts).
 //
 //   xq, xs  = per-token int8 quantisation of x (arithmetic of cmi_quant_act_i8)
 //   sum_g   = sum_{k in group g} xq[m,k] * (code(n,k) - 8)     int32, exact
