@@ -61,17 +61,20 @@ __device__ __forceinline__ void widen4(uint32_t w, uint32_t &lo, uint32_t &hi) {
 // K above 128*NLP*WAVES (the second round's bytes are requested line by line as the first
 // round frees their registers; asking for all weight bytes at the start took 179 registers
 // and measured slower).
-template <int NLP, int WAVES, int ROUNDS>
+// T: 16-row tiles of weight rows per workgroup (the activation tiles a wavefront fetched and
+// rearranged serve all of them: at 16 rows they are two thirds of the bytes a wavefront asks for).
+template <int NLP, int WAVES, int ROUNDS, int T = 1>
 __global__ void __launch_bounds__(WAVES * 64)
 gemv_w8a16_rows16_kernel(const Args a) {
+    static_assert(T == 1 || ROUNDS == 1, "several tiles only in the single-round arrangement");
     extern __shared__ __align__(16) uint8_t lds[];
-    float(*partial)[64][4] = reinterpret_cast<float(*)[64][4]>(lds);  // [WAVES][64][4]
-    uint8_t *patches = lds + WAVES * 1024;                            // per wavefront: weights, activations
+    float(*partial)[64][4] = reinterpret_cast<float(*)[64][4]>(lds);  // [T * WAVES][64][4]
+    uint8_t *patches = lds + T * WAVES * 1024;                            // per wavefront: weights, activations
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int kq = lane >> 4;
-    const int n0 = blockIdx.x * ROWS;
+    const int n0 = blockIdx.x * (T * ROWS);
     const int lines = a.K / LINE;
     uint8_t *wpatch = patches + wave * (PATCH_BYTES + XPATCH_BYTES), *xpatch = wpatch + PATCH_BYTES;
     const uint8_t *xbytes = reinterpret_cast<const uint8_t *>(a.x);
@@ -80,7 +83,7 @@ gemv_w8a16_rows16_kernel(const Args a) {
     // Activations first (L2 resident; memory answers in request order), then every weight byte.
     // An activation line is 256 bytes: parts 0 and 1, each fetched as two half tiles; rows past
     // M repeat the last one, their sums are dropped.
-    v4i32 xr[NLP][4], wr[NLP][2];
+    v4i32 xr[NLP][4], wr[T][NLP][2];
     // One or two activation rows: every lane's row is one of two, so the MFMA arrangement (row
     // lane%16, bytes 64*kq .. +63 of the line) can be loaded as it is -- the requests collapse
     // onto a few cache lines -- and the LDS rearrangement is skipped.
@@ -104,9 +107,11 @@ gemv_w8a16_rows16_kernel(const Args a) {
         const int line = line_of(r, i);
         if (line >= lines) return;
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
-            wr[i][h] = __builtin_nontemporal_load(
-                reinterpret_cast<const v4i32 *>(a.wq + tile_src(lane, h, n0, a.N - 1, a.K, line * LINE)));
+        for (int t = 0; t < T; ++t)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                wr[t][i][h] = __builtin_nontemporal_load(reinterpret_cast<const v4i32 *>(
+                    a.wq + tile_src(lane, h, n0 + t * ROWS, a.N - 1, a.K, line * LINE)));
     };
 #pragma unroll
     for (int i = 0; i < NLP; ++i) request_x(0, i);
@@ -115,10 +120,14 @@ gemv_w8a16_rows16_kernel(const Args a) {
     // The row scale of the output this thread will finish, requested now, behind everything the
     // arithmetic waits for: asked for at the end it is a cold load under a saturated memory system
     // (1.4 us of every workgroup's 4.6 us, by in-kernel timestamps).
-    const float ws_out = a.ws[min(n0 + (int)((threadIdx.x >> 2) & 15), a.N - 1)];
+    float ws_out[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) ws_out[t] = a.ws[min(n0 + t * ROWS + (int)((threadIdx.x >> 2) & 15), a.N - 1)];
 
-    // the accumulator of lane l holds (n = l%16, m = 4*kq + v), v = 0..3
-    v4f32 acc = {0.f, 0.f, 0.f, 0.f};
+    // the accumulator of lane l holds (n = l%16, m = 4*kq + v), v = 0..3, per tile
+    v4f32 acc[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) acc[t] = v4f32{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int r = 0; r < ROUNDS; ++r) {
         // activations into the MFMA arrangement: row lane%16, bytes 64*kq .. +63 of the line
@@ -137,18 +146,21 @@ gemv_w8a16_rows16_kernel(const Args a) {
 #pragma unroll
         for (int i = 0; i < NLP; ++i) {
             if (line_of(r, i) >= lines) break;
-            tile_park(wpatch, lane, wr[i][0], wr[i][1]);
-            const v4i32 w0 = tile_take(wpatch, lane, 2 * kq), w1 = tile_take(wpatch, lane, 2 * kq + 1);
-            const uint32_t d[8] = {(uint32_t)w0.x, (uint32_t)w0.y, (uint32_t)w0.z, (uint32_t)w0.w,
-                                   (uint32_t)w1.x, (uint32_t)w1.y, (uint32_t)w1.z, (uint32_t)w1.w};
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {  // k = 32*kq + 8*s .. +7 of the line
-                uint32_t b[4];
-                widen4(d[2 * s], b[0], b[1]);
-                widen4(d[2 * s + 1], b[2], b[3]);
-                const v4i32 bw = {(int)b[0], (int)b[1], (int)b[2], (int)b[3]};
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xr[i][s]),
-                                                              __builtin_bit_cast(bf16x8, bw), acc, 0, 0, 0);
+            for (int t = 0; t < T; ++t) {
+                tile_park(wpatch, lane, wr[t][i][0], wr[t][i][1]);
+                const v4i32 w0 = tile_take(wpatch, lane, 2 * kq), w1 = tile_take(wpatch, lane, 2 * kq + 1);
+                const uint32_t d[8] = {(uint32_t)w0.x, (uint32_t)w0.y, (uint32_t)w0.z, (uint32_t)w0.w,
+                                       (uint32_t)w1.x, (uint32_t)w1.y, (uint32_t)w1.z, (uint32_t)w1.w};
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {  // k = 32*kq + 8*s .. +7 of the line
+                    uint32_t b[4];
+                    widen4(d[2 * s], b[0], b[1]);
+                    widen4(d[2 * s + 1], b[2], b[3]);
+                    const v4i32 bw = {(int)b[0], (int)b[1], (int)b[2], (int)b[3]};
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xr[i][s]),
+                                                                     __builtin_bit_cast(bf16x8, bw), acc[t], 0, 0, 0);
+                }
             }
             if (r + 1 < ROUNDS) {
                 request_x(r + 1, i);
@@ -156,30 +168,35 @@ gemv_w8a16_rows16_kernel(const Args a) {
             }
         }
     }
-    *reinterpret_cast<v4f32 *>(&partial[wave][lane][0]) = acc;
+#pragma unroll
+    for (int t = 0; t < T; ++t) *reinterpret_cast<v4f32 *>(&partial[t * WAVES + wave][lane][0]) = acc[t];
     __syncthreads();
 
     if (threadIdx.x < 256) {
         const int l = threadIdx.x >> 2, v = threadIdx.x & 3;
-        const int n = n0 + (l & 15), m = 4 * (l >> 4) + v;
-        if (n < a.N && m < a.M) {
-            float total = partial[0][l][v];
+        const int m = 4 * (l >> 4) + v;
 #pragma unroll
-            for (int wv = 1; wv < WAVES; ++wv) total += partial[wv][l][v];
-            a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * ws_out);
+        for (int t = 0; t < T; ++t) {
+            const int n = n0 + t * ROWS + (l & 15);
+            if (n < a.N && m < a.M) {
+                float total = partial[t * WAVES][l][v];
+#pragma unroll
+                for (int wv = 1; wv < WAVES; ++wv) total += partial[t * WAVES + wv][l][v];
+                a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * ws_out[t]);
+            }
         }
     }
 }
 
-template <int NLP, int WAVES, int ROUNDS = 1>
+template <int NLP, int WAVES, int ROUNDS = 1, int T = 1>
 int launch(const Args &a, hipStream_t st) {
-    constexpr int LDS_BYTES = WAVES * (1024 + PATCH_BYTES + XPATCH_BYTES);
+    constexpr int LDS_BYTES = WAVES * (T * 1024 + PATCH_BYTES + XPATCH_BYTES);
     static std::atomic<uint64_t> devices{0};
-    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w8a16_rows16_kernel<NLP, WAVES, ROUNDS>),
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w8a16_rows16_kernel<NLP, WAVES, ROUNDS, T>),
                                    LDS_BYTES, devices, "cmi_gemv_w8a16_mfma"))
         return rc;
-    const dim3 grid((a.N + ROWS - 1) / ROWS);
-    gemv_w8a16_rows16_kernel<NLP, WAVES, ROUNDS><<<grid, dim3(WAVES * 64), LDS_BYTES, st>>>(a);
+    const dim3 grid((a.N + T * ROWS - 1) / (T * ROWS));
+    gemv_w8a16_rows16_kernel<NLP, WAVES, ROUNDS, T><<<grid, dim3(WAVES * 64), LDS_BYTES, st>>>(a);
     return check_launch("cmi_gemv_w8a16_mfma");
 }
 
@@ -341,9 +358,14 @@ extern "C" int cmi_gemv_w8a16_mfma(const int8_t *wq, const float *ws, const void
     }
     // eight wavefronts (shorter chains of dependent steps) up to 2048 workgroups, four beyond
     // (2560 -> 151936: 72 us against 84)
+    // From four rows and 300 tiles of weight rows up, a workgroup owns two tiles: the activation
+    // tiles its wavefronts fetched and rearranged serve both (16 rows: 2560 -> 6144 6.9 -> 6.3 us,
+    // 2560 -> 151936 86 -> 78 us; with fewer rows or tiles one tile per workgroup stays faster).
+    const int tiles = (N + ROWS - 1) / ROWS;
+    const bool two = M >= 4 && tiles >= 300;
     if (lines <= 8) return launch<2, 4>(a, st);
-    if (lines <= 20 && (N + ROWS - 1) / ROWS > 2048) return launch<5, 4>(a, st);
-    if (lines <= 24) return launch<3, 8>(a, st);
-    if (lines <= 40) return launch<5, 8>(a, st);
+    if (lines <= 20 && tiles > 2048) return two ? launch<5, 4, 1, 2>(a, st) : launch<5, 4>(a, st);
+    if (lines <= 24) return two ? launch<3, 8, 1, 2>(a, st) : launch<3, 8>(a, st);
+    if (lines <= 40) return two ? launch<5, 8, 1, 2>(a, st) : launch<5, 8>(a, st);
     return launch<5, 8, 2>(a, st);
 }
