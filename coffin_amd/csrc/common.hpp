@@ -36,6 +36,8 @@ int gemm_w8a8_generic(const int8_t *xq, const int8_t *wq, const float *xs, const
 // K <= 10240); CMI_E_UNSUPPORTED (no error text) outside that range.
 int gemm_w8a8_rows16(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws, void *y,
                      int32_t *acc_out, int M, int N, int K, int ldy, void *stream);
+// 16-row weight tiles per workgroup (1 or 2) that gemm_w8a8_rows16 uses for 17..128 rows.
+int gemm_w8a8_rows_tiles(int N);
 
 // gemv_w4a8_decode.hip: W4A8 GEMV for 1..4 rows, K <= 10240, from bf16 activations (x) or
 // quantised ones (xq, xs); returns CMI_E_UNSUPPORTED (no error text) for other shapes.

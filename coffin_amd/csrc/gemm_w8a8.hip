@@ -83,7 +83,10 @@ __device__ __forceinline__ void wait_vmcnt() {
     else if constexpr (N == 12) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 16) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 18) asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)" ::: "memory");
+    else if constexpr (N == 20) asm volatile("s_waitcnt vmcnt(20) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 24) asm volatile("s_waitcnt vmcnt(24) lgkmcnt(0)" ::: "memory");
+    else if constexpr (N == 28) asm volatile("s_waitcnt vmcnt(28) lgkmcnt(0)" ::: "memory");
+    else if constexpr (N == 30) asm volatile("s_waitcnt vmcnt(30) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 32) asm volatile("s_waitcnt vmcnt(32) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 36) asm volatile("s_waitcnt vmcnt(36) lgkmcnt(0)" ::: "memory");
     else static_assert(N < 0, "add the vmcnt literal");
@@ -752,17 +755,29 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
         const int rc = gemm_w8a8_rows16(xq, wq, xs, ws, y, acc_out, M, N, K, ldy, stream);
         if (rc != CMI_E_UNSUPPORTED) return rc;
     }
-    if (M > 16 && M <= 256 && K % 128 == 0 && K <= 10240 && !force) {
-        // Few rows: the tile pipeline is latency-bound (K/128 dependent steps of 0.45-1.4 us, growing
-        // with the number of tiles that share the chip, whatever M is); the read-once kernel asks
-        // for the weight once per 128 rows and pays per 16-row chunk only the chunk's trip through
-        // the matrix pipe; same bits.  Cost models fitted to measurements on the layer shapes with
-        // cold weights (us).
+    int mid = 0;  // 17..256 rows: the tile kernel the cost models below chose (64 x 64: 6464), if any
+    if (M > 16 && M <= 256 && K % BK == 0 && N >= 8 && !force) {
+        // Between the GEMV-like batch and the full tile pipeline every kernel is bound by what its
+        // workgroups pull through L2 per dependent step, and which one is fastest changes with the
+        // shape: the read-once kernel pays per 16-row chunk, a tile kernel K / 128 steps whose
+        // length grows with N (bytes per step) and with the rounds of workgroups on the 256 CUs.
+        // Cost models (us) fitted to cold-weight measurements of all five kernels on eleven layer
+        // shapes x ten batch sizes; their choice is within 1 % of the best measured in total
+        // (the two-candidate rule this replaces: 19 % above).
         const double steps = K / 128.0, wbytes = (double)N * K;
-        const double tiles = (double)((M + 127) / 128) * ((N + 127) / 128);
-        const double t_tiled = 2.5 + steps * (tiles <= 512 ? 0.42 + 0.0033 * tiles : 2.1 * ceil(tiles / 512.0));
-        const double t_rows = ((M + 127) / 128) * (3.2 + wbytes / 6.0e6) + ((M + 15) / 16) * (0.5 + wbytes / 2.0e7);
-        if (t_rows < t_tiled) {
+        auto rounds = [](double tiles) { return ceil(tiles / 256.0); };
+        const double tiles_h = (double)((M + 63) / 64) * ((N + 63) / 64);
+        const double tiles_g = (double)((M + 127) / 128) * ((N + 63) / 64);
+        const double tiles_t = (double)((M + 127) / 128) * ((N + 127) / 128);
+        const double t_h = 2.5 + steps * (0.22 + N * 1.6e-5) * (1.0 + 0.50 * (rounds(tiles_h) - 1));
+        const double t_g = 2.5 + steps * (0.36 + N * 1.2e-5) * (1.0 + 0.75 * (rounds(tiles_g) - 1));
+        const double t_t = 2.5 + steps * (0.50 + N * 1.5e-5) * (1.0 + 0.65 * (rounds(tiles_t) - 1));
+        double t_rows = 1e30;
+        if (K <= 10240) {
+            const double per_chunk = 0.5 + wbytes / (gemm_w8a8_rows_tiles(N) * 2.0e7);
+            t_rows = ((M + 127) / 128) * (3.2 + wbytes / 6.0e6) + ((M + 15) / 16) * per_chunk;
+        }
+        if (t_rows <= t_h && t_rows <= t_g && t_rows <= t_t) {
             for (int lo = 0; lo < M; lo += 128) {
                 const int m = M - lo < 128 ? M - lo : 128;
                 const int rc = gemm_w8a8_rows16(xq + (size_t)lo * K, wq, xs + lo, ws,
@@ -772,6 +787,7 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
             }
             return CMI_OK;
         }
+        mid = t_h <= t_g && t_h <= t_t ? 6464 : t_g <= t_t ? 64 : 128;
     }
     if (K % BK != 0 || N < 8) return gemm_w8a8_generic(xq, wq, xs, ws, y, acc_out, M, N, K, ldy, stream);
     Args a;
@@ -789,10 +805,10 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
     // Tile choice: how full the last round of workgroups is (256 CUs; one large workgroup or
     // two 128 x 128 workgroups per CU) and how much of the tiles' area is real output, times
     // the steady-state advantage of the larger tiles.  CMI_GEMM_TILE=64|128|256|320 overrides
-    // (tests, tuning).
-    int pick;  // 64, 128, 256 or 320: block tile along n
-    if (force) {
-        pick = force;
+    // (tests, tuning); 6464 forces the 64 x 64 tile of the mid-batch route.
+    int pick;  // 64, 128, 256 or 320: block tile along n; 6464: 64 x 64
+    if (force || mid) {
+        pick = force ? force : mid;
     } else {
         auto fill = [](double tiles, double slots) { return tiles / (ceil(tiles / slots) * slots); };
         const double t128 = (double)((M + 127) / 128) * ((N + 127) / 128);
@@ -810,7 +826,10 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
     // instead, twice as many workgroups with half the MFMAs per dependent step each (512 x 4096 x 2560
     // 16.8 -> 12.7 us, 512 x 2560 x 9728 47 -> 34 us; with more tiles than that it measured 10-30 % slower).
     const int tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
-    if (pick == 128 && !force && tiles128 <= 128 && N > 64) pick = 64;
+    if (pick == 128 && !force && !mid && tiles128 <= 128 && N > 64) pick = 64;
+    // 64 x 64 tiles, four LDS stages (more stages measured the same): half the bytes per step and
+    // twice the workgroups of the 128 x 64 tile for batches of up to 64 rows or few n tiles
+    if (pick == 6464) return launch<1, 1, 4>(a, st);
     if (pick == 64) {
         const int tiles64 = ((M + 127) / 128) * ((N + 63) / 64);
         if (tiles64 <= 256) return launch<1, 2, 3>(a, st);

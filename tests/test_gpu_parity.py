@@ -287,9 +287,9 @@ def test_sixteen_row_kernels_at_lm_head_size_sampled_columns(orc):
 
 # ------------------------------------------------------------------ W8A8 GEMM
 
-@pytest.fixture(params=["auto", "64", "128", "256", "320"])
+@pytest.fixture(params=["auto", "64", "128", "256", "320", "6464"])
 def gemm_tile(request):
-    """Force the 128 x 64, 128 x 128, 256 x 256 or 256 x 320 block-tile kernel through
+    """Force the 128 x 64, 128 x 128, 256 x 256, 256 x 320 or 64 x 64 block-tile kernel through
     cmi_set_option, or leave the choice to the library (conftest resets it after each test)."""
     if request.param != "auto":
         G.set_option("gemm_tile", int(request.param))
@@ -320,7 +320,13 @@ def test_gemm_w8a8_bit_exact(orc, gemm_tile, m, n, k):
                                    # 17..128 rows per launch with the weight kept in registers (and two
                                    # such launches): every lines-per-wavefront variant, ragged N and M
                                    (17, 100, 9728), (48, 2560, 2560), (128, 333, 4096), (100, 77, 1024),
-                                   (33, 40, 10240), (200, 64, 9728), (64, 1200, 5120)])
+                                   (33, 40, 10240), (200, 64, 9728), (64, 1200, 5120),
+                                   # two 16-row weight tiles per workgroup (160..256 workgroups of 32
+                                   # rows), ragged N and M, every lines-per-wavefront variant
+                                   (40, 6144, 2560), (100, 5100, 1024), (17, 8192, 640), (128, 5120, 5120),
+                                   (30, 5500, 9728),
+                                   # batches the cost models hand to the 64 x 64 tile kernel
+                                   (64, 9728, 2560), (200, 2560, 4096), (20, 1000, 11008)])
 def test_gemm_w8a8_verify_batches_bit_exact(orc, m, n, k):
     """Few rows take the read-the-weight-once kernels: exact against the oracle, and the
     same bits as the tiled kernel gives for the same rows (also with a row stride)."""
