@@ -55,6 +55,10 @@ int gemv_w4a8_chain(const uint8_t *w4, const float *ws, const void *x, const int
 int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs, const void *x,
                      void *y, int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
                      void *stream);
+// gemm_w4a8_ring.hip: W4A8 tile GEMM with a ring of LDS stages for launches of few tiles; tile =
+// 6464 (64 x 64) or 64 (128 m x 64 n); arguments already checked.
+int gemm_w4a8_ring(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs, void *y, int M, int N,
+                   int K, int tile, void *stream);
 // linear_bf16.hip: quantiser + W4A8 GEMV / GEMM (or the GEMV that quantises by itself where that
 // is faster) on bf16 rows, with xq int8 [M,K] / xs fp32 [M] as staging; arguments already checked.
 int linear_w4a8_rows(const uint8_t *w4, const float *ws, const void *x, void *y, int M, int N, int K, int gs,

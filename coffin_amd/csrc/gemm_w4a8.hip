@@ -304,20 +304,35 @@ extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     CMI_REQUIRE(K % BK == 0, CMI_E_UNSUPPORTED, "cmi_gemm_w4a8: K=%d is not a multiple of %d", K, BK);
     CMI_REQUIRE(aligned(xq, 16) && aligned(w4, 16), CMI_E_ARG,
                 "cmi_gemm_w4a8: xq and w4 must be 16-byte aligned");
-    // Few rows: the tile pipeline is latency-bound (K/128 steps of ~1.2 us whatever M is), while the
-    // matrix-pipe GEMV reads the weight once per 16 rows at memory speed; same integer sums, same
-    // fp32 chain, same bits.  Cost model fitted to measurements on the layer shapes (us).
-    if (M <= 256 && !option_gemm_tile()) {
+    // Which kernel: with few tiles a launch is a chain of K/128 dependent steps and the kernels differ
+    // in the length of a step (two-stage 128 x 128 tiles: 1.15 us and up; ring of stages with
+    // 64 x 64 tiles 0.5 us, with 128 x 64 tiles 0.7 us), with many tiles in how a step's time grows
+    // with the tiles per CU, and up to 256 rows the matrix-pipe GEMV reads the weight once per 128
+    // rows at memory speed and pays per 16-row chunk.  Same integer sums, same fp32 chain, same
+    // bits from all of them.  Cost models (us) fitted to cold-weight measurements on ten layer
+    // shapes x eleven batch sizes.  The ring kernels do not write the group sums.
+    const int forced = option_gemm_tile();
+    int ring = !group_acc && (forced == 64 || forced == 6464) ? forced : 0;
+    if (!forced) {
         const double steps = K / 128.0, wn = (double)N * K;
         const double tiles = (double)a_ceil(M, BM) * a_ceil(N, BN);
-        const double t_tiled = 3.0 + steps * (tiles <= 512 ? 1.15 + 0.0013 * tiles : 1.8 * ceil(tiles / 512.0));
+        const double t_tiled = 3.0 + steps * (tiles <= 512 ? 1.15 + 0.0013 * tiles : 1.6 * ceil(tiles / 512.0));
         // up to 10240 elements per row the GEMV keeps the weight in registers for 128 rows per launch
         // and pays per 16-row chunk only the chunk's sums and chain; longer rows run it in passes,
         // 16 rows per launch, at about half the speed
         const double t_rows16 =
-            K <= 10240 ? a_ceil(M, 128) * (2.0 + wn / 2 / 4.2e6) + a_ceil(M, 16) * (0.6 + wn / 1.3e7 + steps * 0.012)
-                       : a_ceil(M, 16) * (3.6 + wn / 2 / 2.1e6);
-        if (t_rows16 < t_tiled) {
+            M > 256 ? 1e30
+            : K <= 10240 ? a_ceil(M, 128) * (2.0 + wn / 2 / 4.2e6) + a_ceil(M, 16) * (0.6 + wn / 1.3e7 + steps * 0.012)
+                         : a_ceil(M, 16) * (3.6 + wn / 2 / 2.1e6);
+        const double tiles_h = (double)a_ceil(M, 64) * a_ceil(N, 64), tiles_g = (double)a_ceil(M, 128) * a_ceil(N, 64);
+        // a step of the ring kernels: flat while every tile has a CU to itself, a second level up to
+        // two tiles per CU, then linear in the tiles
+        const double s_h = tiles_h <= 256 ? 0.5 + 6e-6 * N : tiles_h <= 512 ? 0.65 + 1e-5 * N : 0.4 + 0.00137 * tiles_h;
+        const double s_g = tiles_g <= 256 ? 0.7 + 8e-6 * N : tiles_g <= 512 ? 1.0 + 4e-6 * N : 0.4 + 0.00205 * tiles_g;
+        const double t_h = group_acc ? 1e30 : 2.5 + steps * s_h;
+        const double t_g = group_acc ? 1e30 : 2.5 + steps * s_g;
+        // (the GEMV's model is the optimistic one of the four at four chunks and more: it has to win by 10 %)
+        if (t_rows16 <= t_tiled && t_rows16 <= 0.9 * t_h && t_rows16 <= 0.9 * t_g) {
             const int G = K / BK;
             const int step = K <= 10240 ? 128 : 16;
             for (int lo = 0; lo < M; lo += step) {
@@ -330,7 +345,10 @@ extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
             }
             return CMI_OK;
         }
+        if (t_h <= t_tiled && t_h <= t_g) ring = 6464;
+        else if (t_g <= t_tiled) ring = 64;
     }
+    if (ring) return gemm_w4a8_ring(w4, ws, xq, xs, y, M, N, K, ring, stream);
     Args a;
     a.xq = xq;
     a.w4 = w4;

@@ -516,6 +516,24 @@ def test_gemm_w4a8_bit_exact(orc, m, n, k):
     gacc, y = G.w4a8(w4, ws, xq, xs, k, gemm=True)
     assert (gacc.cpu().numpy() == gacc_ref).all()
     assert (G.bits(y) == y_ref).all()
+    # without the group sums the entry may pick a kernel that cannot write them: same bits
+    _, y2 = G.w4a8(w4, ws, xq, xs, k, gemm=True, want_acc=False)
+    assert (G.bits(y2) == y_ref).all()
+
+
+@pytest.mark.parametrize("tile", [64, 6464])
+@pytest.mark.parametrize("m,n,k", [(64, 64, 128), (128, 256, 256), (64, 2560, 2560), (100, 200, 384),
+                                   (17, 1000, 6656), (200, 77, 1024), (256, 1280, 5120), (33, 130, 10240),
+                                   (1, 1024, 2560), (300, 333, 640), (64, 9728, 2560), (96, 300, 11008)])
+def test_gemm_w4a8_ring_of_stages_bit_exact(orc, tile, m, n, k):
+    """The W4A8 tile kernels that keep several steps of operands in flight (128 x 64 and 64 x 64
+    block tiles), forced through cmi_set_option: one to eight steps, fewer steps than ring slots,
+    ragged M and N, against the oracle."""
+    w4, ws, xq, xs, _, y_ref = _w4_case(orc, m, n, k, seeded())
+    G.set_option("gemm_tile", tile)
+    _, y = G.w4a8(w4, ws, xq, xs, k, gemm=True, want_acc=False)
+    G.set_option("gemm_tile", 0)
+    assert (G.bits(y) == y_ref).all()
 
 
 def test_w4a8_golden_and_chain_order(golden):
