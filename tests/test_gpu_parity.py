@@ -536,6 +536,35 @@ def test_gemm_w4a8_ring_of_stages_bit_exact(orc, tile, m, n, k):
     assert (G.bits(y) == y_ref).all()
 
 
+def test_mid_batch_dispatch_agrees_with_the_forced_tile_on_random_shapes():
+    """Whatever kernel the cost models of cmi_gemm_w8a8 / cmi_gemm_w4a8 pick between 17 and 300
+    rows -- read-once kernels with one or two weight tiles, 64 x 64, 128 x 64, 128 x 128 tiles,
+    ring of stages -- the bits are those of the forced 128 x 128 tile kernel (which the other
+    tests pin against the oracle): 24 seeded random shapes per format, ragged M and N."""
+    rnd = np.random.RandomState(20240611)
+    g = synth.generator(77, G.DEV)
+    for case in range(24):
+        m = int(rnd.randint(17, 301))
+        n = int(rnd.choice([rnd.randint(8, 400), rnd.randint(400, 3000), rnd.randint(3000, 12000)]))
+        k = 128 * int(rnd.choice([rnd.randint(1, 9), rnd.randint(9, 41), rnd.randint(41, 90)]))
+        x = synth.activations(m, k, g, outliers=bool(case & 1))
+        xq, xs = G.quant(x)
+        q = synth.int8_weight(n, k, g)
+        G.set_option("gemm_tile", 0)
+        _, y = G.gemm_w8a8(xq, q.wq, xs, q.scale, want_acc=False)
+        G.set_option("gemm_tile", 128)
+        _, y_ref = G.gemm_w8a8(xq, q.wq, xs, q.scale, want_acc=False)
+        assert (y.view(torch.int16) == y_ref.view(torch.int16)).all(), ("w8a8", m, n, k)
+        w = synth.int4_weight(n, k, g)
+        w4, ws = G.w4_repack(w.packed, w.scale, k)
+        G.set_option("gemm_tile", 0)
+        _, y4 = G.w4a8(w4, ws, xq, xs, k, gemm=True, want_acc=False)
+        G.set_option("gemm_tile", 128)
+        _, y4_ref = G.w4a8(w4, ws, xq, xs, k, gemm=True, want_acc=False)
+        assert (y4.view(torch.int16) == y4_ref.view(torch.int16)).all(), ("w4a8", m, n, k)
+    G.set_option("gemm_tile", 0)
+
+
 def test_w4a8_golden_and_chain_order(golden):
     g = golden("linear_w4a8")
     k = int(g["a_k"])
