@@ -44,7 +44,8 @@ SIGNATURES: dict[str, list] = {
 }
 
 #: Entry points that do not return a status.
-OTHER_RESTYPES = {"cmi_linear_workspace_bytes": ([_ci, _ci], _sz)}
+OTHER_RESTYPES = {"cmi_linear_workspace_bytes": ([_ci, _ci], _sz),
+                  "cmi_linear_w8a8_workspace_bytes": ([_ci, _ci, _ci], _sz)}
 
 
 class NativeError(RuntimeError):

@@ -124,20 +124,23 @@ def _on_gpu(t: torch.Tensor) -> bool:
 
 # --------------------------------------------------------------- private state
 
-#: (rows, k, device) -> uint8 workspace of cmi_linear_workspace_bytes(rows, k) bytes (the
+#: (rows, k, device, n) -> uint8 workspace of cmi_linear_workspace_bytes(rows, k) bytes (the
 #: quantised rows and their scales of one projection); single-threaded caller by contract
 #: (backends/corex/__init__.py:654-690 keeps the same kind of pool).
 _SCRATCH: OrderedDict = OrderedDict()
 _SCRATCH_MAX = 32
 
 
-def _scratch(rows: int, k: int, device: torch.device) -> torch.Tensor:
-    key = (rows, k, device)
+def _scratch(rows: int, k: int, device: torch.device, n: int = 0) -> torch.Tensor:
+    """Workspace of the fused quantiser + projection entries; with ``n`` (int8 weights) sized so
+    that the W8A8 entry may split K where that pays."""
+    key = (rows, k, device, n)
     hit = _SCRATCH.get(key)
     if hit is None:
         while len(_SCRATCH) >= _SCRATCH_MAX:
             _SCRATCH.popitem(last=False)          # least recently used shape goes first
-        nbytes = int(_native.load().cmi_linear_workspace_bytes(rows, k))
+        lib = _native.load()
+        nbytes = int(lib.cmi_linear_w8a8_workspace_bytes(rows, n, k) if n else lib.cmi_linear_workspace_bytes(rows, k))
         hit = torch.empty(nbytes, dtype=torch.uint8, device=device)
         _SCRATCH[key] = hit
     else:
@@ -310,7 +313,7 @@ def _gemv_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor, mfma
 
 def _gemm_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> None:
     n, k = rec.n, rec.k
-    work = _scratch(rows, k, act.device)
+    work = _scratch(rows, k, act.device, n)
     rc = _native.load().cmi_linear_w8a8_bf16(act.data_ptr(), rec.a, rec.b, out.data_ptr(), rows, n, k, n,
                                              work.data_ptr(), work.numel(), _stream())
     if rc:

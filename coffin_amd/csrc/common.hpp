@@ -36,6 +36,14 @@ int gemm_w8a8_generic(const int8_t *xq, const int8_t *wq, const float *xs, const
 // K <= 10240); CMI_E_UNSUPPORTED (no error text) outside that range.
 int gemm_w8a8_rows16(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws, void *y,
                      int32_t *acc_out, int M, int N, int K, int ldy, void *stream);
+// gemm_w8a8.hip: cmi_gemm_w8a8 with room for split-K (arrival counters, 256 ints, zero; partial
+// tiles, gemm_w8a8_split_bytes(M, N, K) bytes or fewer: the kernel choice adapts); both null = no split.
+int gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws, void *y,
+                    int32_t *acc_out, int M, int N, int K, int ldy, int *arrivals, void *partials,
+                    size_t partial_bytes, void *stream);
+size_t gemm_w8a8_split_bytes(int M, int N, int K);
+// quant_act_i8.hip: cmi_quant_act_i8 that also clears n_zero ints at `zero` (null / 0: none).
+int quant_act_i8_and_clear(const void *x, int8_t *q, float *s, int M, int K, int *zero, int n_zero, void *stream);
 // 16-row weight tiles per workgroup (1 or 2) that gemm_w8a8_rows16 uses for 17..128 rows.
 int gemm_w8a8_rows_tiles(int N);
 

@@ -53,6 +53,12 @@ struct Args {
     int32_t *acc_out;
     int M, N, K, ldy;
     int tiles_m, tiles_n;
+    // split-K launches only: how many workgroups share a tile's K range, where they leave their
+    // int32 partial tiles ([split][tile][accumulator piece][thread] x 16 bytes) and the tiles'
+    // arrival counters (zero at launch)
+    int splits;
+    int32_t *partials;
+    int *arrivals;
 };
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
@@ -98,11 +104,11 @@ __device__ __forceinline__ void wait_vmcnt() {
 // band, so the ~32-64 workgroups an XCD runs at a time form an 8 x (4..8) patch
 // that shares its X rows and W rows through that L2 instead of streaming the
 // whole of X once per n tile.
-__device__ __forceinline__ void tile_coords(const Args &a, int &tm, int &tn) {
+__device__ __forceinline__ void tile_coords(const Args &a, int &tm, int &tn, int id = blockIdx.x) {
     constexpr int GM = 8;
     const int total = a.tiles_m * a.tiles_n;
-    int t = blockIdx.x;
-    if (total % 8 == 0) t = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
+    int t = id;
+    if (total % 8 == 0) t = (id % 8) * (total / 8) + id / 8;
     const int width = GM * a.tiles_n;
     const int band = t / width, in_band = t - band * width;
     const int first_m = band * GM;
@@ -232,20 +238,32 @@ __device__ __forceinline__ void epilogue(const Args &a, v16i32 (&acc)[TN][TM], i
     }
 }
 
-template <int TN, int TM, int NST>
+// SPLIT: a.splits workgroups share a tile, each walking a contiguous part of K; they leave their
+// int32 accumulators in a.partials and the last to arrive (a.arrivals, cleared before the launch)
+// adds the others' to its own -- integer sums, exact in any order -- and runs the epilogue: the
+// bits of the unsplit kernel.  For launches of few tiles and many K steps, which are a chain of
+// dependent steps on a fraction of the CUs.
+template <int TN, int TM, int NST, bool SPLIT = false>
 __global__ void __launch_bounds__(THREADS)
 gemm_w8a8_pipe_kernel(const Args a) {
     using C = Cfg<TN, TM, NST>;
     extern __shared__ __align__(16) int8_t lds[];
+    __shared__ int arrived_before;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: keeps LDS bases scalar
     const int wn = wave & 1, wm = wave >> 1;
 
+    const int tiles = a.tiles_m * a.tiles_n;
+    const int tile = SPLIT ? blockIdx.x % tiles : blockIdx.x, split = SPLIT ? blockIdx.x / tiles : 0;
     int tm, tn;
-    tile_coords(a, tm, tn);
+    tile_coords(a, tm, tn, tile);
     const int m0 = tm * C::BM, n0 = tn * C::BN;
     float *scales = reinterpret_cast<float *>(lds + NST * C::STAGE_BYTES);
     stage_scales<C::BN, C::BM>(a, scales, n0, m0);
+    // this workgroup's K steps: all of them, or part `split` of a.splits nearly equal parts
+    const int ksteps_all = a.K / BK;
+    const int k_first = SPLIT ? (int)((long long)ksteps_all * split / a.splits) : 0;
+    const int ksteps = SPLIT ? (int)((long long)ksteps_all * (split + 1) / a.splits) - k_first : ksteps_all;
 
     // Global side of the direct loads.  One load instruction moves 8 rows x 128 B
     // (whole cache lines) into 1 KiB of LDS; each wavefront fills a contiguous run
@@ -258,13 +276,13 @@ gemm_w8a8_pipe_kernel(const Args a) {
     for (int g = 0; g < C::WL; ++g) {
         const int row = (C::WL * wave + g) * 8 + lrow;
         const int kc = (lane & 7) ^ ((row >> 1) & 7);
-        wsrc[g] = a.wq + (size_t)min(n0 + row, a.N - 1) * a.K + kc * 16;
+        wsrc[g] = a.wq + (size_t)min(n0 + row, a.N - 1) * a.K + kc * 16 + k_first * BK;
     }
 #pragma unroll
     for (int g = 0; g < C::XL; ++g) {
         const int row = (C::XL * wave + g) * 8 + lrow;
         const int kc = (lane & 7) ^ ((row >> 1) & 7);
-        xsrc[g] = a.xq + (size_t)min(m0 + row, a.M - 1) * a.K + kc * 16;
+        xsrc[g] = a.xq + (size_t)min(m0 + row, a.M - 1) * a.K + kc * 16 + k_first * BK;
     }
     auto issue = [&](int stage, int ks) {
         int8_t *base = lds + stage * C::STAGE_BYTES;
@@ -314,7 +332,6 @@ gemm_w8a8_pipe_kernel(const Args a) {
                     acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[i][h], xf[j][h], acc[i][j], 0, 0, 0);
     };
 
-    const int ksteps = a.K / BK;
     // One pipeline step.  The fragments of step ks are in registers.  Stage
     // (ks+1)%NST must have landed: of the loads this wavefront issued after it,
     // NST-2 stages' worth may still be in flight while new loads are being issued
@@ -377,6 +394,55 @@ gemm_w8a8_pipe_kernel(const Args a) {
     }
     if (ks < ksteps) step(drain_t{}, ks, w0, x0, w1, x1);
 
+    if constexpr (SPLIT) {
+        // Accumulator element e of thread t at int e * THREADS + t of the workgroup's partial tile:
+        // every instruction moves 256 contiguous bytes per wavefront.  The partials cross XCDs,
+        // whose L2s are not coherent with each other: they are written and read as relaxed
+        // device-scope atomics (stores that write through, loads that go to the coherence
+        // point), ordered by "all my stores acknowledged" (vmcnt 0) before the arrival.  A device-
+        // scope fence would do the same by writing back and invalidating the whole L2 under the
+        // other workgroups' operand streams (measured: +25 us per launch).
+        constexpr int ELEMS = TN * TM * 16;
+        int *mine = a.partials + ((size_t)split * tiles + tile) * (ELEMS * THREADS) + threadIdx.x;
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    __hip_atomic_store(mine + ((i * TM + j) * 16 + v) * THREADS, acc[i][j][v], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (threadIdx.x == 0)
+            arrived_before = __hip_atomic_fetch_add(a.arrivals + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (arrived_before != a.splits - 1) return;  // uniform: not the last workgroup of the tile
+        // all the others' elements are requested before the first is added (one trip to memory,
+        // not one per split): four splits' worth at a time, slots past the last split or on this
+        // workgroup's own partial re-read split 0 and count for nothing
+        for (int s0 = 0; s0 < a.splits; s0 += 4) {
+            int theirs[4][ELEMS];
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const int s = s0 + d < a.splits ? s0 + d : 0;
+                const int *src = a.partials + ((size_t)s * tiles + tile) * (ELEMS * THREADS) + threadIdx.x;
+#pragma unroll
+                for (int e = 0; e < ELEMS; ++e)
+                    theirs[d][e] = __hip_atomic_load(src + e * THREADS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const bool counts = s0 + d < a.splits && s0 + d != split;
+#pragma unroll
+                for (int i = 0; i < TN; ++i)
+#pragma unroll
+                    for (int j = 0; j < TM; ++j)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) acc[i][j][v] += counts ? theirs[d][(i * TM + j) * 16 + v] : 0;
+            }
+        }
+    }
     epilogue<TN, TM>(a, acc, lds, wave, lane, n0 + wn * 32 * TN, m0 + wm * 32 * TM, scales + wn * 32 * TN,
                      scales + C::BN + wm * 32 * TM);
 }
@@ -391,6 +457,19 @@ int launch(Args &a, hipStream_t st) {
                                    C::LDS_BYTES, devices, "cmi_gemm_w8a8"))
         return rc;
     gemm_w8a8_pipe_kernel<TN, TM, NST><<<dim3(a.tiles_m * a.tiles_n), dim3(THREADS), C::LDS_BYTES, st>>>(a);
+    return check_launch("cmi_gemm_w8a8");
+}
+
+// Split-K launch of the 64 x 64 tile: a.splits, a.partials and a.arrivals set by the caller.
+int launch_split(Args &a, hipStream_t st) {
+    using C = Cfg<1, 1, 4>;
+    a.tiles_m = (a.M + C::BM - 1) / C::BM;
+    a.tiles_n = (a.N + C::BN - 1) / C::BN;
+    static std::atomic<uint64_t> devices{0};
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_pipe_kernel<1, 1, 4, true>),
+                                   C::LDS_BYTES, devices, "cmi_gemm_w8a8"))
+        return rc;
+    gemm_w8a8_pipe_kernel<1, 1, 4, true><<<dim3(a.tiles_m * a.tiles_n * a.splits), dim3(THREADS), C::LDS_BYTES, st>>>(a);
     return check_launch("cmi_gemm_w8a8");
 }
 
@@ -742,6 +821,17 @@ int launch_wide(Args &a, hipStream_t st) {
 extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws,
                              void *y, int32_t *acc_out, int M, int N, int K, int ldy,
                              void *stream) {
+    return cmi::gemm_w8a8_split(xq, wq, xs, ws, y, acc_out, M, N, K, ldy, nullptr, nullptr, 0, stream);
+}
+
+size_t cmi::gemm_w8a8_split_bytes(int M, int N, int K) {
+    // up to 256 workgroups of 64 x 64 int32 each, whatever the split
+    return M > 16 && M <= 256 && K % BK == 0 && N >= 8 ? (size_t)256 * 64 * 64 * 4 : 0;
+}
+
+int cmi::gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws, void *y,
+                         int32_t *acc_out, int M, int N, int K, int ldy, int *arrivals, void *partials,
+                         size_t partial_bytes, void *stream) {
     CMI_REQUIRE(M >= 0 && N >= 1 && K >= 16, CMI_E_ARG, "cmi_gemm_w8a8: bad shape M=%d N=%d K=%d", M, N, K);
     if (M == 0) return CMI_OK;  // an empty batch has no storage to point at
     CMI_REQUIRE(xq && wq && xs && ws && y, CMI_E_ARG, "cmi_gemm_w8a8: null pointer");
@@ -777,6 +867,39 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
             const double per_chunk = 0.5 + wbytes / (gemm_w8a8_rows_tiles(N) * 2.0e7);
             t_rows = ((M + 127) / 128) * (3.2 + wbytes / 6.0e6) + ((M + 15) / 16) * per_chunk;
         }
+        // Split-K on the 64 x 64 tile where the caller brought room for the partial tiles (the
+        // arrival counters cleared): few tiles and many steps, e.g. 64 rows of 9728 -> 2560 are
+        // 40 tiles x 76 steps on 40 of 256 CUs.  As many splits as keep one workgroup per CU and
+        // four steps per split.  With the whole chip pulling, the steps run into the weight stream
+        // (about 5 TB/s in so short a launch), and the hand-over -- partial tiles written through
+        // to memory, the arrival, the last workgroup's reads: three trips to memory, the L2s of
+        // the XCDs not being coherent with each other -- costs 5 us whatever the shape.
+        int splits = 1;
+        double t_s = 1e30;
+        if (arrivals && partials && tiles_h <= 128) {
+            splits = (int)(256.0 / tiles_h);
+            if (splits > steps / 4) splits = (int)(steps / 4);
+            if (splits > 8) splits = 8;
+            if (splits >= 2 && (size_t)(splits * tiles_h) * 64 * 64 * 4 <= partial_bytes)
+                t_s = 2.5 + fmax(ceil(steps / splits) * 0.26, wbytes / 5.0e6) + 5.0;
+        }
+        if (t_s < t_rows && t_s < t_h && t_s < t_g && t_s < t_t) {
+            Args a;
+            a.xq = xq;
+            a.wq = wq;
+            a.xs = xs;
+            a.ws = ws;
+            a.y = static_cast<uint16_t *>(y);
+            a.acc_out = acc_out;
+            a.M = M;
+            a.N = N;
+            a.K = K;
+            a.ldy = ldy;
+            a.splits = splits;
+            a.partials = static_cast<int32_t *>(partials);
+            a.arrivals = arrivals;
+            return launch_split(a, static_cast<hipStream_t>(stream));
+        }
         if (t_rows <= t_h && t_rows <= t_g && t_rows <= t_t) {
             for (int lo = 0; lo < M; lo += 128) {
                 const int m = M - lo < 128 ? M - lo : 128;
@@ -801,6 +924,9 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
     a.N = N;
     a.K = K;
     a.ldy = ldy;
+    a.splits = 1;
+    a.partials = nullptr;
+    a.arrivals = nullptr;
     hipStream_t st = static_cast<hipStream_t>(stream);
     // Tile choice: how full the last round of workgroups is (256 CUs; one large workgroup or
     // two 128 x 128 workgroups per CU) and how much of the tiles' area is real output, times

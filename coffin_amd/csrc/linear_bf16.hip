@@ -59,6 +59,15 @@ extern "C" size_t cmi_linear_workspace_bytes(int M, int K) {
     return round_up((size_t)M * K) + round_up(sizeof(float) * (size_t)M);
 }
 
+constexpr int ARRIVALS = 256;  // split-K arrival counters behind xq and xs
+
+extern "C" size_t cmi_linear_w8a8_workspace_bytes(int M, int N, int K) {
+    const size_t base = cmi_linear_workspace_bytes(M, K);
+    if (base == 0 || N <= 0) return base;
+    const size_t split = gemm_w8a8_split_bytes(M, N, K);
+    return split ? base + round_up(sizeof(int) * ARRIVALS) + split : base;
+}
+
 extern "C" int cmi_linear_w8a8_bf16(const void *x, const int8_t *wq, const float *ws, void *y, int M, int N, int K,
                                     int ldy, void *workspace, size_t workspace_bytes, void *stream) {
     CMI_REQUIRE(M >= 0 && N >= 1 && K >= 16, CMI_E_ARG, "cmi_linear_w8a8_bf16: bad shape M=%d N=%d K=%d", M, N, K);
@@ -67,8 +76,19 @@ extern "C" int cmi_linear_w8a8_bf16(const void *x, const int8_t *wq, const float
     int8_t *xq;
     float *xs;
     if (const int rc = split_workspace("cmi_linear_w8a8_bf16", workspace, workspace_bytes, M, K, &xq, &xs)) return rc;
-    if (const int rc = cmi_quant_act_i8(x, xq, xs, M, K, stream)) return rc;
-    return cmi_gemm_w8a8(xq, wq, xs, ws, y, nullptr, M, N, K, ldy, stream);
+    // whatever the workspace holds beyond the quantised rows is room for split-K: 256 arrival
+    // counters, cleared by the quantiser's launch, then partial tiles
+    const size_t base = cmi_linear_workspace_bytes(M, K), counters = round_up(sizeof(int) * ARRIVALS);
+    int *arrivals = nullptr;
+    void *partials = nullptr;
+    size_t partial_bytes = 0;
+    if (workspace_bytes > base + counters && gemm_w8a8_split_bytes(M, N, K)) {
+        arrivals = reinterpret_cast<int *>(static_cast<unsigned char *>(workspace) + base);
+        partials = static_cast<unsigned char *>(workspace) + base + counters;
+        partial_bytes = workspace_bytes - base - counters;
+    }
+    if (const int rc = quant_act_i8_and_clear(x, xq, xs, M, K, arrivals, arrivals ? ARRIVALS : 0, stream)) return rc;
+    return gemm_w8a8_split(xq, wq, xs, ws, y, nullptr, M, N, K, ldy, arrivals, partials, partial_bytes, stream);
 }
 
 extern "C" int cmi_linear_w4a8_bf16(const uint8_t *w4, const float *ws, const void *x, void *y, int M, int N, int K,

@@ -27,12 +27,16 @@ __device__ __forceinline__ float block_max(float v, float *smem) {
 
 // K % 8 == 0, rows 16-byte aligned.  VPT > 0: the row fits in VPT vectors per
 // thread and stays in registers; VPT == 0: generic, second pass re-reads.
+// zero / n_zero: a few ints of the caller's that the first workgroup clears on the way (the
+// arrival counters of a split-K GEMM that follows in the stream), or null / 0.
 template <int VPT>
 __global__ void __launch_bounds__(QUANT_THREADS)
 quant_act_i8_vec(const uint4 *__restrict__ x, uint2 *__restrict__ q, float *__restrict__ s,
-                 int nvec) {
+                 int nvec, int *__restrict__ zero, int n_zero) {
     __shared__ float smem[QUANT_THREADS / 64];
     const int row = blockIdx.x;
+    if (row == 0)
+        for (int i = threadIdx.x; i < n_zero; i += QUANT_THREADS) zero[i] = 0;
     const uint4 *xr = x + (size_t)row * nvec;
     uint2 *qr = q + (size_t)row * nvec;
     float amax = 0.f;
@@ -67,9 +71,11 @@ quant_act_i8_vec(const uint4 *__restrict__ x, uint2 *__restrict__ q, float *__re
 // Any K, any alignment.
 __global__ void __launch_bounds__(QUANT_THREADS)
 quant_act_i8_scalar(const uint16_t *__restrict__ x, int8_t *__restrict__ q,
-                    float *__restrict__ s, int K) {
+                    float *__restrict__ s, int K, int *__restrict__ zero, int n_zero) {
     __shared__ float smem[QUANT_THREADS / 64];
     const int row = blockIdx.x;
+    if (row == 0)
+        for (int i = threadIdx.x; i < n_zero; i += QUANT_THREADS) zero[i] = 0;
     const uint16_t *xr = x + (size_t)row * K;
     int8_t *qr = q + (size_t)row * K;
     float amax = 0.f;
@@ -85,7 +91,7 @@ quant_act_i8_scalar(const uint16_t *__restrict__ x, int8_t *__restrict__ q,
 
 }  // namespace
 
-extern "C" int cmi_quant_act_i8(const void *x, int8_t *q, float *s, int M, int K,
+int cmi::quant_act_i8_and_clear(const void *x, int8_t *q, float *s, int M, int K, int *zero, int n_zero,
                                 void *stream) {
     CMI_REQUIRE(M >= 0 && K > 0, CMI_E_ARG, "cmi_quant_act_i8: bad shape M=%d K=%d", M, K);
     if (M == 0) return CMI_OK;  // an empty batch has no storage to point at
@@ -97,14 +103,18 @@ extern "C" int cmi_quant_act_i8(const void *x, int8_t *q, float *s, int M, int K
         const uint4 *xv = static_cast<const uint4 *>(x);
         uint2 *qv = reinterpret_cast<uint2 *>(q);
         const int vpt = (nvec + QUANT_THREADS - 1) / QUANT_THREADS;
-        if (vpt <= 1) quant_act_i8_vec<1><<<grid, block, 0, st>>>(xv, qv, s, nvec);
-        else if (vpt <= 2) quant_act_i8_vec<2><<<grid, block, 0, st>>>(xv, qv, s, nvec);
-        else if (vpt <= 4) quant_act_i8_vec<4><<<grid, block, 0, st>>>(xv, qv, s, nvec);
-        else if (vpt <= 8) quant_act_i8_vec<8><<<grid, block, 0, st>>>(xv, qv, s, nvec);
-        else if (vpt <= 16) quant_act_i8_vec<16><<<grid, block, 0, st>>>(xv, qv, s, nvec);
-        else quant_act_i8_vec<0><<<grid, block, 0, st>>>(xv, qv, s, nvec);
+        if (vpt <= 1) quant_act_i8_vec<1><<<grid, block, 0, st>>>(xv, qv, s, nvec, zero, n_zero);
+        else if (vpt <= 2) quant_act_i8_vec<2><<<grid, block, 0, st>>>(xv, qv, s, nvec, zero, n_zero);
+        else if (vpt <= 4) quant_act_i8_vec<4><<<grid, block, 0, st>>>(xv, qv, s, nvec, zero, n_zero);
+        else if (vpt <= 8) quant_act_i8_vec<8><<<grid, block, 0, st>>>(xv, qv, s, nvec, zero, n_zero);
+        else if (vpt <= 16) quant_act_i8_vec<16><<<grid, block, 0, st>>>(xv, qv, s, nvec, zero, n_zero);
+        else quant_act_i8_vec<0><<<grid, block, 0, st>>>(xv, qv, s, nvec, zero, n_zero);
     } else {
-        quant_act_i8_scalar<<<grid, block, 0, st>>>(static_cast<const uint16_t *>(x), q, s, K);
+        quant_act_i8_scalar<<<grid, block, 0, st>>>(static_cast<const uint16_t *>(x), q, s, K, zero, n_zero);
     }
     return check_launch("cmi_quant_act_i8");
+}
+
+extern "C" int cmi_quant_act_i8(const void *x, int8_t *q, float *s, int M, int K, void *stream) {
+    return cmi::quant_act_i8_and_clear(x, q, s, M, K, nullptr, 0, stream);
 }

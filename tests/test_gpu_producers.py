@@ -266,6 +266,38 @@ def test_linear_w4a8_bf16_equals_quantiser_plus_kernels(orc, m, n, k):
                                                           128, G.ptr(work), nbytes - 1, G.stream()), "short")
 
 
+@pytest.mark.parametrize("m,n,k", [(64, 2560, 9728), (128, 2560, 9728), (33, 4096, 11008), (100, 1500, 10240),
+                                   (20, 2560, 11008), (64, 1024, 2560), (256, 2560, 9728)])
+def test_linear_w8a8_bf16_split_k_same_bits(orc, m, n, k):
+    """With the larger workspace the entry may split K over the idle CUs (few tiles, many K steps:
+    the first five shapes; the last two stay unsplit): the partial sums are integers, so output
+    and quantised rows are those of the small workspace and of the oracle, also with a row stride,
+    and on a second call (the arrival counters are cleared by every call's quantiser launch)."""
+    lib = _native.load()
+    g = synth.generator(4321, G.DEV)
+    q = synth.int8_weight(n, k, g)
+    x = synth.activations(m, k, g, outliers=True)
+    small, small_bytes = _workspace(m, k)
+    big_bytes = int(lib.cmi_linear_w8a8_workspace_bytes(m, n, k))
+    assert big_bytes >= small_bytes + 1024 + 4 * 2**20
+    big = torch.full((big_bytes,), 0xA5, dtype=torch.uint8, device=G.DEV)   # counters start as garbage
+    y_small = torch.zeros((m, n), dtype=torch.bfloat16, device=G.DEV)
+    _native.check(lib.cmi_linear_w8a8_bf16(G.ptr(x), G.ptr(q.wq), G.ptr(q.scale), G.ptr(y_small), m, n, k, n,
+                                           G.ptr(small), small_bytes, G.stream()), "linear_w8a8_bf16")
+    for ldy in (n, n + 8):
+        for _ in range(2):
+            y = torch.zeros((m, ldy), dtype=torch.bfloat16, device=G.DEV)
+            _native.check(lib.cmi_linear_w8a8_bf16(G.ptr(x), G.ptr(q.wq), G.ptr(q.scale), G.ptr(y), m, n, k, ldy,
+                                                   G.ptr(big), big_bytes, G.stream()), "linear_w8a8_bf16")
+            assert (y[:, :n].contiguous().view(torch.int16) == y_small.view(torch.int16)).all()
+            assert (y[:, n:].float() == 0).all()
+    rows = [0, m // 2, m - 1]
+    xq_ref, xs_ref = orc.quant_act_i8(G.bits(x[rows]))
+    _, y_ref = orc.gemm_w8a8(xq_ref, q.wq.cpu().numpy(), xs_ref, q.scale.cpu().numpy(), want_acc=False)
+    assert (G.bits(y_small[rows].contiguous()) == y_ref).all()
+    assert (big[:m * k].view(torch.int8).view(m, k) == small[:m * k].view(torch.int8).view(m, k)).all()
+
+
 @pytest.mark.parametrize("m,n,k", [(64, 1024, 2560), (300, 4096, 2560), (5, 640, 1024), (2048, 4096, 2560)])
 def test_linear_w8a8_bf16_equals_quantiser_plus_gemm(orc, m, n, k):
     g = synth.generator(1234, G.DEV)
