@@ -618,7 +618,7 @@ def main() -> int:
 
         # 64 and 128 rows (between the GEMV and the tile pipeline) on the two MLP shapes, the three
         # weight formats as the adapter issues them: weight-only on the matrix-pipe GEMV (64 rows per
-        # call), quantiser + W8A8, quantiser + W4A8
+        # call), cmi_linear_w8a8_bf16 and cmi_linear_w4a8_bf16 (quantiser + GEMM) on the adapter's workspace
         for m in (64, 128):
             mid = {}
             for n_, k_ in ((9728, 2560), (2560, 9728)):
@@ -643,16 +643,17 @@ def main() -> int:
                         for lo in range(0, m, rows_per_call):
                             lib.cmi_gemv_w8a16_mfma(ptr(q.wq), ptr(q.scale), vp(x.data_ptr() + lo * k_ * 2),
                                                     vp(y.data_ptr() + lo * n_ * 2), rows_per_call, n_, k_, st)
+                work = torch.empty(int(lib.cmi_linear_w8a8_workspace_bytes(m, n_, k_)), dtype=torch.uint8, device=dev)
                 def w8a8():
                     st = cur_stream()
                     for q in w8:
-                        lib.cmi_quant_act_i8(ptr(x), ptr(xq), ptr(xs), m, k_, st)
-                        lib.cmi_gemm_w8a8(ptr(xq), ptr(q.wq), ptr(xs), ptr(q.scale), ptr(y), vp(0), m, n_, k_, n_, st)
+                        lib.cmi_linear_w8a8_bf16(ptr(x), ptr(q.wq), ptr(q.scale), ptr(y), m, n_, k_, n_,
+                                                 ptr(work), work.numel(), st)
                 def w4a8():
                     st = cur_stream()
                     for d4, ds in w4_:
-                        lib.cmi_quant_act_i8(ptr(x), ptr(xq), ptr(xs), m, k_, st)
-                        lib.cmi_gemm_w4a8(ptr(d4), ptr(ds), ptr(xq), ptr(xs), ptr(y), vp(0), m, n_, k_, 128, st)
+                        lib.cmi_linear_w4a8_bf16(ptr(d4), ptr(ds), ptr(x), ptr(y), m, n_, k_, 128,
+                                                 ptr(work), work.numel(), st)
                 def replayed(fn):  # the calls on `copies` cold weights, captured once
                     fn()
                     torch.cuda.synchronize()
