@@ -168,23 +168,32 @@ gemm_w4a8_ring_kernel(const Args a) {
 
     // This lane's pieces of packed weight, slot -> int8 buffer `buf` (chunks 2p, 2p+1 of the row,
     // swizzled like the activations), and the slot's scales of this lane's n.
-    auto widen = [&](int slot, int buf, float (&sc_out)[TN]) {
+    struct Fetched {
+        v4i32 packed[TN];
+        float sc[TN];
+    };
+    auto fetch = [&](int slot) {  // requests only
         const int8_t *src = lds + slot * C::SLOT_BYTES + C::X_BYTES;
         const float *s = reinterpret_cast<const float *>(src + C::P_BYTES);
+        Fetched f;
+#pragma unroll
+        for (int h = 0; h < TN; ++h) f.packed[h] = lds_read16_unseen(src + (TN * wave + h) * 1024 + lane * 16);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) f.sc[j] = lds_read4_unseen(s + wn * 32 * TN + j * 32 + (lane & 31));
+        return f;
+    };
+    auto widen = [&](Fetched &f, int buf, float (&sc_out)[TN]) {
         int8_t *wbuf = lds + NST * C::SLOT_BYTES + buf * C::W_BYTES;
-        v4i32 packed[TN];
-#pragma unroll
-        for (int h = 0; h < TN; ++h) packed[h] = lds_read16_unseen(src + (TN * wave + h) * 1024 + lane * 16);
-#pragma unroll
-        for (int j = 0; j < TN; ++j) sc_out[j] = lds_read4_unseen(s + wn * 32 * TN + j * 32 + (lane & 31));
-        if constexpr (TN == 1) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(packed[0]), "+v"(sc_out[0])::"memory");
-        else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(packed[0]), "+v"(packed[1]), "+v"(sc_out[0]), "+v"(sc_out[1])::"memory");
+        if constexpr (TN == 1) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.packed[0]), "+v"(f.sc[0])::"memory");
+        else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f.packed[0]), "+v"(f.packed[1]), "+v"(f.sc[0]), "+v"(f.sc[1])::"memory");
         static_assert(TN <= 2, "operands of the wait above");
+#pragma unroll
+        for (int j = 0; j < TN; ++j) sc_out[j] = f.sc[j];
 #pragma unroll
         for (int h = 0; h < TN; ++h) {
             const int row = (TN * wave + h) * 16 + (lane >> 2), wp = lane & 3;
-            const uint32_t w[4] = {(uint32_t)packed[h].x, (uint32_t)packed[h].y, (uint32_t)packed[h].z,
-                                   (uint32_t)packed[h].w};
+            const uint32_t w[4] = {(uint32_t)f.packed[h].x, (uint32_t)f.packed[h].y, (uint32_t)f.packed[h].z,
+                                   (uint32_t)f.packed[h].w};
             uint4 lo, hi;  // k 0..15 and 16..31 of the piece
             lo.x = rebias4(w[0] & 0x0F0F0F0Fu);
             lo.y = rebias4((w[0] >> 4) & 0x0F0F0F0Fu);
@@ -262,6 +271,12 @@ gemm_w4a8_ring_kernel(const Args a) {
     auto step = [&](auto issue_tag, int ks) {
         constexpr bool ISSUE = decltype(issue_tag)::value;
         const int slot = ks % NST, next = (ks + 1) % NST, buf = ks & 1;
+        // the next step's operands have landed (measured: long ago, the wait is free); this lane's
+        // piece of its packed weight and its scales are asked for now and used behind the three
+        // quarters (past the last step: stale bytes, widened to where nobody reads them)
+        if constexpr (ISSUE) wait_vmcnt<(NST - 2) * C::LOADS>();
+        else wait_vmcnt<0>();
+        Fetched fetched = fetch(next);
         read_q(slot, buf, 1, f1);
         mma_q(f0, true);
         pace_quarter();
@@ -271,12 +286,8 @@ gemm_w4a8_ring_kernel(const Args a) {
         read_q(slot, buf, 3, f1);
         mma_q(f0, false);
         pace_quarter();
-        if constexpr (ISSUE) wait_vmcnt<(NST - 2) * C::LOADS>();
-        else wait_vmcnt<0>();
         float sc_next[TN];
-#pragma unroll
-        for (int j = 0; j < TN; ++j) sc_next[j] = 0.f;
-        if (ks + 1 < ksteps) widen(next, buf ^ 1, sc_next);
+        widen(fetched, buf ^ 1, sc_next);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -305,7 +316,10 @@ gemm_w4a8_ring_kernel(const Args a) {
         if (s < ksteps) issue(s, s);
     if (ksteps >= NST) wait_vmcnt<(NST - 1) * C::LOADS>();
     else wait_vmcnt<0>();
-    widen(0, 0, sc);
+    {
+        Fetched first = fetch(0);
+        widen(first, 0, sc);
+    }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
