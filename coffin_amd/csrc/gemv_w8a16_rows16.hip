@@ -210,24 +210,28 @@ int launch(const Args &a, hipStream_t st) {
 // free up.  The partial tiles of all chunks meet in LDS behind one barrier.
 constexpr int MAX_CHUNKS = 4;
 
-template <int NLP, int WAVES, int ROUNDS>
+// T: 16-row tiles of weight rows per workgroup (single-round arrangements only): every workgroup
+// pulls all activation rows through L2 once per chunk, M * K * 2 bytes times N / (16 T) workgroups,
+// which from three chunks up is what the launch waits for.
+template <int NLP, int WAVES, int ROUNDS, int T = 1>
 __global__ void __launch_bounds__(WAVES * 64)
 gemv_w8a16_rows64_kernel(const Args a) {
+    static_assert(T == 1 || ROUNDS == 1, "several tiles only in the single-round arrangement");
     extern __shared__ __align__(16) uint8_t lds[];
-    float(*partial)[64][4] = reinterpret_cast<float(*)[64][4]>(lds);  // [chunk * WAVES + wave][64][4]
+    float(*partial)[64][4] = reinterpret_cast<float(*)[64][4]>(lds);  // [(chunk * T + tile) * WAVES + wave][64][4]
     const int chunks = (a.M + ROWS - 1) / ROWS;
-    uint8_t *patches = lds + chunks * WAVES * 1024;
+    uint8_t *patches = lds + chunks * T * WAVES * 1024;
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int kq = lane >> 4;
-    const int n0 = blockIdx.x * ROWS;
+    const int n0 = blockIdx.x * (T * ROWS);
     const int lines = a.K / LINE;
     uint8_t *wpatch = patches + wave * (PATCH_BYTES + XPATCH_BYTES), *xpatch = wpatch + PATCH_BYTES;
     const uint8_t *xbytes = reinterpret_cast<const uint8_t *>(a.x);
     auto line_of = [&](int r, int i) { return (r * NLP + i) * WAVES + wave; };
 
-    v4i32 xr[NLP][4], wr[ROUNDS * NLP][2];
+    v4i32 xr[NLP][4], wr[T][ROUNDS * NLP][2];
     auto request_x = [&](int c, int r, int i) {
         const int line = min(line_of(r, i), lines - 1);  // a slot past the last line is not used
 #pragma unroll
@@ -238,29 +242,37 @@ gemv_w8a16_rows64_kernel(const Args a) {
 #pragma unroll
     for (int i = 0; i < NLP; ++i) request_x(0, 0, i);
 #pragma unroll
-    for (int r = 0; r < ROUNDS; ++r)
+    for (int t = 0; t < T; ++t)
 #pragma unroll
-        for (int i = 0; i < NLP; ++i) {
-            const int line = min(line_of(r, i), lines - 1);
+        for (int r = 0; r < ROUNDS; ++r)
 #pragma unroll
-            for (int h = 0; h < 2; ++h)
-                wr[r * NLP + i][h] = __builtin_nontemporal_load(
-                    reinterpret_cast<const v4i32 *>(a.wq + tile_src(lane, h, n0, a.N - 1, a.K, line * LINE)));
-        }
-    // the row scale of the outputs this thread will finish (n depends on the thread only), requested
-    // behind the operands instead of cold at the end
-    const float ws_out = a.ws[min(n0 + (int)((threadIdx.x >> 2) & 15), a.N - 1)];
+            for (int i = 0; i < NLP; ++i) {
+                const int line = min(line_of(r, i), lines - 1);
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+                    wr[t][r * NLP + i][h] = __builtin_nontemporal_load(reinterpret_cast<const v4i32 *>(
+                        a.wq + tile_src(lane, h, n0 + t * ROWS, a.N - 1, a.K, line * LINE)));
+            }
+    // the row scales of the outputs this thread will finish (n depends on the thread and the tile only),
+    // requested behind the operands instead of cold at the end
+    float ws_out[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) ws_out[t] = a.ws[min(n0 + t * ROWS + (int)((threadIdx.x >> 2) & 15), a.N - 1)];
     // weights into the MFMA arrangement, once
 #pragma unroll
-    for (int i = 0; i < ROUNDS * NLP; ++i) {
-        tile_park(wpatch, lane, wr[i][0], wr[i][1]);
-        wr[i][0] = tile_take(wpatch, lane, 2 * kq);
-        wr[i][1] = tile_take(wpatch, lane, 2 * kq + 1);
-    }
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+        for (int i = 0; i < ROUNDS * NLP; ++i) {
+            tile_park(wpatch, lane, wr[t][i][0], wr[t][i][1]);
+            wr[t][i][0] = tile_take(wpatch, lane, 2 * kq);
+            wr[t][i][1] = tile_take(wpatch, lane, 2 * kq + 1);
+        }
 
 #pragma unroll 1
     for (int c = 0; c < chunks; ++c) {
-        v4f32 acc = {0.f, 0.f, 0.f, 0.f};
+        v4f32 acc[T];
+#pragma unroll
+        for (int t = 0; t < T; ++t) acc[t] = v4f32{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int r = 0; r < ROUNDS; ++r) {
             // this batch of activation lines into the MFMA arrangement: row lane%16, bytes 64*kq .. +63
@@ -277,20 +289,23 @@ gemv_w8a16_rows64_kernel(const Args a) {
 #pragma unroll
             for (int i = 0; i < NLP; ++i) {
                 if (line_of(r, i) < lines) {  // uniform per wavefront
-                    v4i32 w0 = wr[r * NLP + i][0], w1 = wr[r * NLP + i][1];
-                    // with two rounds of weight registers the widened copies must not be kept
-                    // across chunks (the compiler would hoist them out of the loop and spill)
-                    if (ROUNDS > 1) asm volatile("" : "+v"(w0), "+v"(w1));
-                    const uint32_t d[8] = {(uint32_t)w0.x, (uint32_t)w0.y, (uint32_t)w0.z, (uint32_t)w0.w,
-                                           (uint32_t)w1.x, (uint32_t)w1.y, (uint32_t)w1.z, (uint32_t)w1.w};
 #pragma unroll
-                    for (int s = 0; s < 4; ++s) {
-                        uint32_t b[4];
-                        widen4(d[2 * s], b[0], b[1]);
-                        widen4(d[2 * s + 1], b[2], b[3]);
-                        const v4i32 bw = {(int)b[0], (int)b[1], (int)b[2], (int)b[3]};
-                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xr[i][s]),
-                                                                      __builtin_bit_cast(bf16x8, bw), acc, 0, 0, 0);
+                    for (int t = 0; t < T; ++t) {
+                        v4i32 w0 = wr[t][r * NLP + i][0], w1 = wr[t][r * NLP + i][1];
+                        // with two rounds or several tiles of weight registers the widened copies must
+                        // not be kept across chunks (the compiler would hoist them out of the loop and spill)
+                        if (ROUNDS > 1 || T > 1) asm volatile("" : "+v"(w0), "+v"(w1));
+                        const uint32_t d[8] = {(uint32_t)w0.x, (uint32_t)w0.y, (uint32_t)w0.z, (uint32_t)w0.w,
+                                               (uint32_t)w1.x, (uint32_t)w1.y, (uint32_t)w1.z, (uint32_t)w1.w};
+#pragma unroll
+                        for (int s = 0; s < 4; ++s) {
+                            uint32_t b[4];
+                            widen4(d[2 * s], b[0], b[1]);
+                            widen4(d[2 * s + 1], b[2], b[3]);
+                            const v4i32 bw = {(int)b[0], (int)b[1], (int)b[2], (int)b[3]};
+                            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xr[i][s]),
+                                                                             __builtin_bit_cast(bf16x8, bw), acc[t], 0, 0, 0);
+                        }
                     }
                 }
                 // this line's activation registers are free: ask for the same slot of the next batch
@@ -298,33 +313,37 @@ gemv_w8a16_rows64_kernel(const Args a) {
                 else if (c + 1 < chunks) request_x(c + 1, 0, i);
             }
         }
-        *reinterpret_cast<v4f32 *>(&partial[c * WAVES + wave][lane][0]) = acc;
+#pragma unroll
+        for (int t = 0; t < T; ++t) *reinterpret_cast<v4f32 *>(&partial[(c * T + t) * WAVES + wave][lane][0]) = acc[t];
     }
     __syncthreads();
 
-    for (int o = threadIdx.x; o < chunks * 256; o += WAVES * 64) {
-        const int c = o >> 8, l = (o >> 2) & 63, v = o & 3;
-        const int n = n0 + (l & 15), m = c * ROWS + 4 * (l >> 4) + v;
+    for (int o = threadIdx.x; o < chunks * T * 256; o += WAVES * 64) {
+        const int ct = o >> 8, c = ct / T, t = ct % T, l = (o >> 2) & 63, v = o & 3;
+        const int n = n0 + t * ROWS + (l & 15), m = c * ROWS + 4 * (l >> 4) + v;
         if (n < a.N && m < a.M) {
-            float total = partial[c * WAVES][l][v];
+            float total = partial[ct * WAVES][l][v];
 #pragma unroll
-            for (int wv = 1; wv < WAVES; ++wv) total += partial[c * WAVES + wv][l][v];
-            a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * ws_out);
+            for (int wv = 1; wv < WAVES; ++wv) total += partial[ct * WAVES + wv][l][v];
+            float scale = ws_out[0];
+#pragma unroll
+            for (int tt = 1; tt < T; ++tt) scale = t == tt ? ws_out[tt] : scale;
+            a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total * scale);
         }
     }
 }
 
-template <int NLP, int WAVES, int ROUNDS = 1>
+template <int NLP, int WAVES, int ROUNDS = 1, int T = 1>
 int launch64(const Args &a, hipStream_t st) {
-    constexpr int LDS_MAX = MAX_CHUNKS * WAVES * 1024 + WAVES * (PATCH_BYTES + XPATCH_BYTES);
+    constexpr int LDS_MAX = MAX_CHUNKS * T * WAVES * 1024 + WAVES * (PATCH_BYTES + XPATCH_BYTES);
     static std::atomic<uint64_t> devices{0};
-    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w8a16_rows64_kernel<NLP, WAVES, ROUNDS>),
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w8a16_rows64_kernel<NLP, WAVES, ROUNDS, T>),
                                    LDS_MAX, devices, "cmi_gemv_w8a16_mfma"))
         return rc;
     const int chunks = (a.M + ROWS - 1) / ROWS;
-    const int lds_bytes = chunks * WAVES * 1024 + WAVES * (PATCH_BYTES + XPATCH_BYTES);
-    const dim3 grid((a.N + ROWS - 1) / ROWS);
-    gemv_w8a16_rows64_kernel<NLP, WAVES, ROUNDS><<<grid, dim3(WAVES * 64), lds_bytes, st>>>(a);
+    const int lds_bytes = chunks * T * WAVES * 1024 + WAVES * (PATCH_BYTES + XPATCH_BYTES);
+    const dim3 grid((a.N + T * ROWS - 1) / (T * ROWS));
+    gemv_w8a16_rows64_kernel<NLP, WAVES, ROUNDS, T><<<grid, dim3(WAVES * 64), lds_bytes, st>>>(a);
     return check_launch("cmi_gemv_w8a16_mfma");
 }
 
@@ -352,8 +371,20 @@ extern "C" int cmi_gemv_w8a16_mfma(const int8_t *wq, const float *ws, const void
     if (M > ROWS) {
         if (lines <= 8) return launch64<2, 4>(a, st);
         if (lines <= 20 && (N + ROWS - 1) / ROWS > 2048) return launch64<5, 4>(a, st);
-        if (lines <= 24) return launch64<3, 8>(a, st);
-        if (lines <= 40) return launch64<5, 8>(a, st);
+        // Several weight tiles per workgroup: the activation rows a workgroup pulls through L2 per
+        // chunk then serve 32 or 48 weight rows.  A launch takes (rounds of 256 workgroups) x (time of
+        // a workgroup), and a workgroup of T tiles about (2 T + 1) units -- fitted to 2560 -> 9728 /
+        // 6144 / 19456 and 4096 -> 11008 / 14336 / 5120 at 32..64 rows, where the best T follows this
+        // count every time (64 rows of 2560 -> 9728: 21.9 -> 16.6 us with three tiles, 2560 -> 6144
+        // 15.2 -> 12.6 with two, 4096 -> 14336 44 -> 39 with two; three is what LDS holds).
+        const int tiles = (N + ROWS - 1) / ROWS;
+        int T = 1, best = 1 << 30;
+        for (int t = 1; t <= 3; ++t) {
+            const int cost = ((tiles + t - 1) / t + 255) / 256 * (2 * t + 1);
+            if (cost < best) best = cost, T = t;
+        }
+        if (lines <= 24) return T == 3 ? launch64<3, 8, 1, 3>(a, st) : T == 2 ? launch64<3, 8, 1, 2>(a, st) : launch64<3, 8>(a, st);
+        if (lines <= 40) return T == 3 ? launch64<5, 8, 1, 3>(a, st) : T == 2 ? launch64<5, 8, 1, 2>(a, st) : launch64<5, 8>(a, st);
         return launch64<5, 8, 2>(a, st);
     }
     // eight wavefronts (shorter chains of dependent steps) up to 2048 workgroups, four beyond

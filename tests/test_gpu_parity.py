@@ -162,9 +162,12 @@ def test_gemv_w8a16_mfma_within_tolerance(orc, m, n, k):
 
 
 @pytest.mark.parametrize("n,k", [(9728, 2560), (300, 5120), (70, 1024), (33000, 2560), (2560, 4096),
-                                 (2560, 9728), (100, 10240), (77, 6656)])
+                                 (2560, 9728), (100, 10240), (77, 6656),
+                                 # two and three weight tiles per workgroup, both 8-wavefront line counts, ragged N
+                                 (6144, 2560), (6100, 2560), (9000, 3200), (5120, 5120), (11008, 4096)])
 def test_gemv_w8a16_mfma_wide_batches_carry_the_16_row_bits(n, k):
-    """17..64 rows in one launch: every row has the bits of a 16-row call."""
+    """17..64 rows in one launch (one, two or three 16-row weight tiles per workgroup): every row
+    has the bits of a 16-row call."""
     g = seeded()
     q = synth.int8_weight(n, k, g)
     wq, ws = q.wq.to(G.DEV), q.scale.to(G.DEV)
