@@ -306,7 +306,7 @@ extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
                 "cmi_gemm_w4a8: xq and w4 must be 16-byte aligned");
     // Which kernel: with few tiles a launch is a chain of K/128 dependent steps and the kernels differ
     // in the length of a step (two-stage 128 x 128 tiles: 1.15 us and up; ring of stages with
-    // 64 x 64 tiles 0.5 us, with 128 x 64 tiles 0.65 us), with many tiles in how a step's time grows
+    // 64 x 64 tiles 0.44 us, with 128 x 64 tiles 0.6 us), with many tiles in how a step's time grows
     // with the tiles per CU, and up to 256 rows the matrix-pipe GEMV reads the weight once per 128
     // rows at memory speed and pays per 16-row chunk.  Same integer sums, same fp32 chain, same
     // bits from all of them.  Cost models (us) fitted to cold-weight measurements on ten layer
@@ -327,8 +327,8 @@ extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
         const double tiles_h = (double)a_ceil(M, 64) * a_ceil(N, 64), tiles_g = (double)a_ceil(M, 128) * a_ceil(N, 64);
         // a step of the ring kernels: flat while every tile has a CU to itself, a second level up to
         // two tiles per CU, then linear in the tiles
-        const double s_h = tiles_h <= 256 ? 0.5 + 6e-6 * N : tiles_h <= 512 ? 0.65 + 1e-5 * N : 0.4 + 0.00137 * tiles_h;
-        const double s_g = tiles_g <= 256 ? 0.63 + 8e-6 * N : tiles_g <= 512 ? 1.0 + 4e-6 * N : 0.4 + 0.00205 * tiles_g;
+        const double s_h = tiles_h <= 256 ? 0.44 + 6e-6 * N : tiles_h <= 512 ? 0.65 + 1e-5 * N : 0.4 + 0.00137 * tiles_h;
+        const double s_g = tiles_g <= 256 ? 0.60 + 1.4e-5 * N : tiles_g <= 512 ? 1.0 + 4e-6 * N : 0.4 + 0.00205 * tiles_g;
         const double t_h = group_acc ? 1e30 : 2.5 + steps * s_h;
         const double t_g = group_acc ? 1e30 : 2.5 + steps * s_g;
         // (the GEMV's model is the optimistic one of the four at four chunks and more: it has to win by 10 %)

@@ -19,7 +19,7 @@
 //     so the scales it reads are covered by its own vmcnt as well.
 // Block tile (64 TM) x (64 TN), four wavefronts (2 x 2), v_mfma_i32_32x32x32_i8 with the
 // activation as the row operand: a lane owns one n per MFMA tile and the per-group flush needs
-// one scale per tile.  One barrier per step.
+// one scale per tile.  One barrier per step; a step's fragments are all read right behind it.
 #include "common.hpp"
 
 #include <type_traits>
@@ -249,57 +249,37 @@ gemm_w4a8_ring_kernel(const Args a) {
                 }
             }
     };
-    constexpr int N_MMA = TM * TN, N_DS = TM + TN;
-    constexpr int DS_PER = (N_DS + N_MMA - 1) / N_MMA;
-    auto pace_quarter = [&]() {  // a quarter's MFMAs with the next quarter's fragment reads between them
-#pragma unroll
-        for (int i = 0; i < N_MMA; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (i * DS_PER < N_DS) __builtin_amdgcn_sched_group_barrier(0x100, DS_PER, 0);
-        }
-    };
-
     const int ksteps = a.K / BK;
-    // Step ks: activations in slot ks % NST, widened weight in buffer ks & 1, first-quarter
-    // fragments in f0, scales in sc.  Before the barrier the operands of step ks+1 must have
-    // landed (of this wavefront's later requests NST-2 steps' worth may stay in flight while new
-    // ones are being issued, none after that) and this lane's share of its weight is widened
-    // into the other buffer, which step ks-1 has finished reading.  Behind the barrier slot
-    // ks % NST is free and takes the requests of step ks+NST.
-    Frag f0, f1;
+    // Step ks enters with all its fragments in registers (read behind the previous barrier, under
+    // the previous step's flush) and its scales in sc.  Its MFMAs go out back to back; this lane's
+    // share of the next step's weight -- landed long ago (measured: the vmcnt wait is over before
+    // it starts), asked for at the top of the step -- is widened into the other int8 buffer, which
+    // step ks-1 has finished reading.  Behind the barrier slot ks % NST is free and takes the
+    // requests of step ks+NST, the next step's fragments are requested, and the group sums are
+    // flushed into the fp32 totals while they arrive.  No branches inside a step (past the last
+    // step stale bytes are widened and read where nobody uses them).  Reading a quarter's fragments
+    // under the previous quarter's MFMAs, as the W8A8 kernels do, left every LDS latency exposed
+    // here (one MFMA per quarter and wavefront): 0.50 -> 0.44 us per step.
+    Frag f[4];
     float sc[TN];
     auto step = [&](auto issue_tag, int ks) {
         constexpr bool ISSUE = decltype(issue_tag)::value;
         const int slot = ks % NST, next = (ks + 1) % NST, buf = ks & 1;
-        // the next step's operands have landed (measured: long ago, the wait is free); this lane's
-        // piece of its packed weight and its scales are asked for now and used behind the three
-        // quarters (past the last step: stale bytes, widened to where nobody reads them)
         if constexpr (ISSUE) wait_vmcnt<(NST - 2) * C::LOADS>();
         else wait_vmcnt<0>();
         Fetched fetched = fetch(next);
-        read_q(slot, buf, 1, f1);
-        mma_q(f0, true);
-        pace_quarter();
-        read_q(slot, buf, 2, f0);
-        mma_q(f1, false);
-        pace_quarter();
-        read_q(slot, buf, 3, f1);
-        mma_q(f0, false);
-        pace_quarter();
+        mma_q(f[0], true);
+        mma_q(f[1], false);
+        mma_q(f[2], false);
+        mma_q(f[3], false);
         float sc_next[TN];
         widen(fetched, buf ^ 1, sc_next);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         if constexpr (ISSUE) issue(slot, ks + NST);
-        read_q(next, buf ^ 1, 0, f0);  // past the last step: stale operands nobody uses
-        mma_q(f1, false);
 #pragma unroll
-        for (int i = 0; i < N_MMA; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (ISSUE && i == 0) __builtin_amdgcn_sched_group_barrier(0x010, C::LOADS, 0);
-            if (i * DS_PER < N_DS) __builtin_amdgcn_sched_group_barrier(0x100, DS_PER, 0);
-        }
+        for (int q = 0; q < 4; ++q) read_q(next, buf ^ 1, q, f[q]);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -323,7 +303,8 @@ gemm_w4a8_ring_kernel(const Args a) {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    read_q(0, 0, 0, f0);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) read_q(0, 0, q, f[q]);
     const int n_issue = ksteps > NST ? ksteps - NST : 0;
     int ks = 0;
     for (; ks < n_issue; ++ks) step(issue_t{}, ks);
