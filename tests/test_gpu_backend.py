@@ -78,6 +78,21 @@ def test_kn_stored_weight_gives_the_bits_of_the_row_major_one():
     assert (backend.linear(q, x[0]).view(torch.int16) == backend.linear(kn, x[0]).view(torch.int16)).all()
 
 
+@pytest.mark.parametrize("rows", [64, 100, 192])
+def test_prefill_chunk_on_a_long_narrow_projection_splits_k_with_the_same_bits(rows):
+    """64..256 rows of a down-projection shape (few tiles, many K steps): the adapter's workspace
+    lets the fused entry split K; output is that of quantiser + cmi_gemm_w8a8 (which never splits)."""
+    g = synth.generator()
+    q = _q8(2560, 9728, g)
+    x = synth.activations(rows, 9728, g).to(G.DEV)
+    y = backend.linear_prefill(q, x)
+    xq, xs = G.quant(x)
+    _, want = G.gemm_w8a8(xq, q.wq.to(G.DEV), xs, q.scale.to(G.DEV), want_acc=False)
+    assert (y.view(torch.int16) == want.view(torch.int16)).all()
+    again = backend.linear_prefill(q, x)            # the arrival counters are cleared by every call
+    assert (again.view(torch.int16) == want.view(torch.int16)).all()
+
+
 @pytest.mark.parametrize("rows", [None, 1, 2, 8, 16, 17, 40])
 def test_int8_entries_agree_with_dequant_matmul(rows):
     g = synth.generator()
