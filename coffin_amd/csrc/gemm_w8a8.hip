@@ -460,16 +460,18 @@ int launch(Args &a, hipStream_t st) {
     return check_launch("cmi_gemm_w8a8");
 }
 
-// Split-K launch of the 64 x 64 tile: a.splits, a.partials and a.arrivals set by the caller.
+// Split-K launch of the 64 x 64 or the 128(m) x 64(n) tile: a.splits, a.partials and a.arrivals set
+// by the caller.
+template <int TM, int NST>
 int launch_split(Args &a, hipStream_t st) {
-    using C = Cfg<1, 1, 4>;
+    using C = Cfg<1, TM, NST>;
     a.tiles_m = (a.M + C::BM - 1) / C::BM;
     a.tiles_n = (a.N + C::BN - 1) / C::BN;
     static std::atomic<uint64_t> devices{0};
-    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_pipe_kernel<1, 1, 4, true>),
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_pipe_kernel<1, TM, NST, true>),
                                    C::LDS_BYTES, devices, "cmi_gemm_w8a8"))
         return rc;
-    gemm_w8a8_pipe_kernel<1, 1, 4, true><<<dim3(a.tiles_m * a.tiles_n * a.splits), dim3(THREADS), C::LDS_BYTES, st>>>(a);
+    gemm_w8a8_pipe_kernel<1, TM, NST, true><<<dim3(a.tiles_m * a.tiles_n * a.splits), dim3(THREADS), C::LDS_BYTES, st>>>(a);
     return check_launch("cmi_gemm_w8a8");
 }
 
@@ -825,8 +827,8 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
 }
 
 size_t cmi::gemm_w8a8_split_bytes(int M, int N, int K) {
-    // up to 256 workgroups of 64 x 64 int32 each, whatever the split
-    return M > 16 && M <= 256 && K % BK == 0 && N >= 8 ? (size_t)256 * 64 * 64 * 4 : 0;
+    // up to 256 workgroups of 64 x 64 or 128 x 64 int32 each, whatever the split
+    return M > 16 && M <= 256 && K % BK == 0 && N >= 8 ? (size_t)256 * 128 * 64 * 4 : 0;
 }
 
 int cmi::gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws, void *y,
@@ -874,16 +876,26 @@ int cmi::gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, co
         // (about 5 TB/s in so short a launch), and the hand-over -- partial tiles written through
         // to memory, the arrival, the last workgroup's reads: three trips to memory, the L2s of
         // the XCDs not being coherent with each other -- costs 5 us whatever the shape.
-        int splits = 1;
-        double t_s = 1e30;
+        int splits = 1, splits_g = 1;
+        double t_s = 1e30, t_sg = 1e30;
+        auto split_count = [&](double tiles) {
+            int n = (int)(256.0 / tiles);
+            if (n > steps / 4) n = (int)(steps / 4);
+            return n > 8 ? 8 : n;
+        };
         if (arrivals && partials && tiles_h <= 128) {
-            splits = (int)(256.0 / tiles_h);
-            if (splits > steps / 4) splits = (int)(steps / 4);
-            if (splits > 8) splits = 8;
+            splits = split_count(tiles_h);
             if (splits >= 2 && (size_t)(splits * tiles_h) * 64 * 64 * 4 <= partial_bytes)
                 t_s = 2.5 + fmax(ceil(steps / splits) * 0.26, wbytes / 5.0e6) + 5.0;
         }
-        if (t_s < t_rows && t_s < t_h && t_s < t_g && t_s < t_t) {
+        // the same on the 128(m) x 64(n) tile (129..256 rows): a step is longer, the hand-over twice the bytes
+        if (arrivals && partials && tiles_g <= 128 && M > 128) {
+            splits_g = split_count(tiles_g);
+            if (splits_g >= 2 && (size_t)(splits_g * tiles_g) * 128 * 64 * 4 <= partial_bytes)
+                t_sg = 2.5 + fmax(ceil(steps / splits_g) * 0.42, wbytes / 5.0e6) + 6.0;
+        }
+        if ((t_s < t_rows && t_s < t_h && t_s < t_g && t_s < t_t) || (t_sg < t_rows && t_sg < t_h && t_sg < t_g && t_sg < t_t)) {
+            const bool wide_m = t_sg < t_s;
             Args a;
             a.xq = xq;
             a.wq = wq;
@@ -895,10 +907,11 @@ int cmi::gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, co
             a.N = N;
             a.K = K;
             a.ldy = ldy;
-            a.splits = splits;
+            a.splits = wide_m ? splits_g : splits;
             a.partials = static_cast<int32_t *>(partials);
             a.arrivals = arrivals;
-            return launch_split(a, static_cast<hipStream_t>(stream));
+            return wide_m ? launch_split<2, 3>(a, static_cast<hipStream_t>(stream))
+                          : launch_split<1, 4>(a, static_cast<hipStream_t>(stream));
         }
         if (t_rows <= t_h && t_rows <= t_g && t_rows <= t_t) {
             for (int lo = 0; lo < M; lo += 128) {

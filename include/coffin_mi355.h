@@ -167,7 +167,7 @@ int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const fl
  *     entry up to 16 rows, the GEMM entry beyond. */
 size_t cmi_linear_workspace_bytes(int M, int K);
 /* A workspace of cmi_linear_w8a8_workspace_bytes(M, N, K) bytes -- the above plus, for 17..256 rows,
- * 256 arrival counters and 4 MiB of partial tiles -- lets cmi_linear_w8a8_bf16 split K over the
+ * 256 arrival counters and 8 MiB of partial tiles -- lets cmi_linear_w8a8_bf16 split K over the
  * idle CUs where a projection is few tiles and many K steps (same bits: the partial sums are
  * integers); with the smaller workspace it does not split.  No counterpart in the reference. */
 size_t cmi_linear_w8a8_workspace_bytes(int M, int N, int K);
