@@ -24,6 +24,7 @@
 // ids are remapped so that each of the 8 XCDs (private L2 each) works on a
 // contiguous band of n tiles.
 #include "common.hpp"
+#include "gemm_tiles.hpp"
 
 namespace {
 
@@ -91,11 +92,6 @@ __device__ __forceinline__ void fetch_i4(const uint8_t *base, int rows, int K, i
     }
 }
 
-// Four codes (0..15, one per byte) -> four int8 (code - 8), no cross-byte borrow.
-__device__ __forceinline__ uint32_t rebias4(uint32_t c) {
-    return ((c | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
-}
-
 __device__ __forceinline__ void stash_i4(int8_t *lds, const uint4 (&reg)[LOADS4]) {
 #pragma unroll
     for (int i = 0; i < LOADS4; ++i) {
@@ -103,14 +99,7 @@ __device__ __forceinline__ void stash_i4(int8_t *lds, const uint4 (&reg)[LOADS4]
         const int r = c / 4, kc = c % 4;
         const uint32_t w[4] = {reg[i].x, reg[i].y, reg[i].z, reg[i].w};
         uint4 lo, hi;  // k 0..15 and 16..31 of the chunk
-        lo.x = rebias4(w[0] & 0x0F0F0F0Fu);
-        lo.y = rebias4((w[0] >> 4) & 0x0F0F0F0Fu);
-        lo.z = rebias4(w[1] & 0x0F0F0F0Fu);
-        lo.w = rebias4((w[1] >> 4) & 0x0F0F0F0Fu);
-        hi.x = rebias4(w[2] & 0x0F0F0F0Fu);
-        hi.y = rebias4((w[2] >> 4) & 0x0F0F0F0Fu);
-        hi.z = rebias4(w[3] & 0x0F0F0F0Fu);
-        hi.w = rebias4((w[3] >> 4) & 0x0F0F0F0Fu);
+        widen_w4_piece(w[0], w[1], w[2], w[3], lo, hi);
         int8_t *dst = lds + r * LDS_STRIDE + kc * 32;
         *reinterpret_cast<uint4 *>(dst) = lo;
         *reinterpret_cast<uint4 *>(dst + 16) = hi;

@@ -25,6 +25,7 @@
 #include <cstdlib>
 
 #include "common.hpp"
+#include "gemm_tiles.hpp"
 
 #include <type_traits>
 
@@ -51,11 +52,6 @@ struct Args {
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
 
-// Four codes (0..15, one per byte) -> four int8 (code - 8), no cross-byte borrow.
-__device__ __forceinline__ uint32_t rebias4(uint32_t c) {
-    return ((c | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
-}
-
 // DUMP: also write the int32 group sums (parity checks); a separate instantiation, the
 // 64 extra store addresses per lane would otherwise be carried through the hot loop.
 template <bool DUMP>
@@ -66,20 +62,9 @@ gemm_w4a8_kernel(const Args a) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wn = wave & 1, wm = wave >> 1;
 
-    // banded tile order per XCD (see the W8A8 kernel)
+    // banded tile order per XCD (gemm_tiles.hpp)
     int tm, tn;
-    {
-        constexpr int GM = 8;
-        const int total = a.tiles_m * a.tiles_n;
-        int t = blockIdx.x;
-        if (total % 8 == 0) t = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
-        const int width = GM * a.tiles_n;
-        const int band = t / width, in_band = t - band * width;
-        const int first_m = band * GM;
-        const int rows = min(a.tiles_m - first_m, GM);
-        tn = in_band / rows;
-        tm = first_m + (in_band - tn * rows);
-    }
+    banded_tile(a.tiles_m, a.tiles_n, blockIdx.x, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
 
     // activations: direct loads, wavefront w fills rows 32w..32w+31 (4 loads of 8 rows x 128 B)
@@ -115,14 +100,7 @@ gemm_w4a8_kernel(const Args a) {
             const int row = wr + 64 * h;
             const uint32_t w[4] = {reg[h].x, reg[h].y, reg[h].z, reg[h].w};
             uint4 lo, hi;  // k 0..15 and 16..31 of the piece
-            lo.x = rebias4(w[0] & 0x0F0F0F0Fu);
-            lo.y = rebias4((w[0] >> 4) & 0x0F0F0F0Fu);
-            lo.z = rebias4(w[1] & 0x0F0F0F0Fu);
-            lo.w = rebias4((w[1] >> 4) & 0x0F0F0F0Fu);
-            hi.x = rebias4(w[2] & 0x0F0F0F0Fu);
-            hi.y = rebias4((w[2] >> 4) & 0x0F0F0F0Fu);
-            hi.z = rebias4(w[3] & 0x0F0F0F0Fu);
-            hi.w = rebias4((w[3] >> 4) & 0x0F0F0F0Fu);
+            widen_w4_piece(w[0], w[1], w[2], w[3], lo, hi);
             int8_t *dst = lds + stage * STAGE_BYTES + X_BYTES + row * BK;
             const int sw = (row >> 1) & 7;
             *reinterpret_cast<uint4 *>(dst + ((2 * wp) ^ sw) * 16) = lo;

@@ -21,6 +21,7 @@
 // activation as the row operand: a lane owns one n per MFMA tile and the per-group flush needs
 // one scale per tile.  One barrier per step; a step's fragments are all read right behind it.
 #include "common.hpp"
+#include "gemm_tiles.hpp"
 
 #include <type_traits>
 
@@ -42,11 +43,6 @@ struct Args {
 };
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
-
-// Four codes (0..15, one per byte) -> four int8 (code - 8), no cross-byte borrow.
-__device__ __forceinline__ uint32_t rebias4(uint32_t c) {
-    return ((c | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
-}
 
 // LDS reads of what this lane's own direct loads have written, and the LDS writes of the widened
 // weight.  The compiler keeps track of direct loads as LDS writes and puts a wait for ALL of them
@@ -109,20 +105,9 @@ gemm_w4a8_ring_kernel(const Args a) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wn = wave & 1, wm = wave >> 1;
 
-    // banded tile order per XCD (see gemm_w8a8.hip)
+    // banded tile order per XCD (gemm_tiles.hpp)
     int tm, tn;
-    {
-        constexpr int GM = 8;
-        const int total = a.tiles_m * a.tiles_n;
-        int t = blockIdx.x;
-        if (total % 8 == 0) t = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
-        const int width = GM * a.tiles_n;
-        const int band = t / width, in_band = t - band * width;
-        const int first_m = band * GM;
-        const int rows = min(a.tiles_m - first_m, GM);
-        tn = in_band / rows;
-        tm = first_m + (in_band - tn * rows);
-    }
+    banded_tile(a.tiles_m, a.tiles_n, blockIdx.x, tm, tn);
     const int m0 = tm * C::BM, n0 = tn * C::BN;
 
     // the tile's row scales, for the epilogue (read behind the loop's barriers)
@@ -195,14 +180,7 @@ gemm_w4a8_ring_kernel(const Args a) {
             const uint32_t w[4] = {(uint32_t)f.packed[h].x, (uint32_t)f.packed[h].y, (uint32_t)f.packed[h].z,
                                    (uint32_t)f.packed[h].w};
             uint4 lo, hi;  // k 0..15 and 16..31 of the piece
-            lo.x = rebias4(w[0] & 0x0F0F0F0Fu);
-            lo.y = rebias4((w[0] >> 4) & 0x0F0F0F0Fu);
-            lo.z = rebias4(w[1] & 0x0F0F0F0Fu);
-            lo.w = rebias4((w[1] >> 4) & 0x0F0F0F0Fu);
-            hi.x = rebias4(w[2] & 0x0F0F0F0Fu);
-            hi.y = rebias4((w[2] >> 4) & 0x0F0F0F0Fu);
-            hi.z = rebias4(w[3] & 0x0F0F0F0Fu);
-            hi.w = rebias4((w[3] >> 4) & 0x0F0F0F0Fu);
+            widen_w4_piece(w[0], w[1], w[2], w[3], lo, hi);
             int8_t *dst = wbuf + row * BK;
             const int sw = (row >> 1) & 7;
             lds_write16_unseen(dst + ((2 * wp) ^ sw) * 16, lo);

@@ -32,6 +32,7 @@
 //
 // The launcher picks by how well the tile count fills the 256 CUs.
 #include "common.hpp"
+#include "gemm_tiles.hpp"
 
 #include <cmath>
 #include <cstdlib>
@@ -98,23 +99,9 @@ __device__ __forceinline__ void wait_vmcnt() {
     else static_assert(N < 0, "add the vmcnt literal");
 }
 
-// Tile of this workgroup.  Workgroups are dealt round-robin to the 8 XCDs (each
-// with a private L2), so XCD x is given the contiguous run of logical tiles
-// [x*per, (x+1)*per); logical tiles walk bands of 8 m tiles, m fastest inside a
-// band, so the ~32-64 workgroups an XCD runs at a time form an 8 x (4..8) patch
-// that shares its X rows and W rows through that L2 instead of streaming the
-// whole of X once per n tile.
+// Tile of this workgroup (the XCD-banded order of gemm_tiles.hpp).
 __device__ __forceinline__ void tile_coords(const Args &a, int &tm, int &tn, int id = blockIdx.x) {
-    constexpr int GM = 8;
-    const int total = a.tiles_m * a.tiles_n;
-    int t = id;
-    if (total % 8 == 0) t = (id % 8) * (total / 8) + id / 8;
-    const int width = GM * a.tiles_n;
-    const int band = t / width, in_band = t - band * width;
-    const int first_m = band * GM;
-    const int rows = min(a.tiles_m - first_m, GM);
-    tn = in_band / rows;
-    tm = first_m + (in_band - tn * rows);
+    banded_tile(a.tiles_m, a.tiles_n, id, tm, tn);
 }
 
 // Scales of a BN x BM block tile into LDS at `dst` (BN column scales, then BM row scales), indices
