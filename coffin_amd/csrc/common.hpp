@@ -19,7 +19,7 @@ int check_launch(const char *what);
 int reserve_lds(const void *kernel, int bytes, std::atomic<uint64_t> &devices, const char *who);
 
 // Kernel-selection overrides (cmi_set_option / CMI_GEMM_TILE, CMI_GEMV_WHOLEROW read once).
-int option_gemm_tile();      // 0 = the library chooses, else 64 / 128 / 256 / 320
+int option_gemm_tile();      // 0 = the library chooses, else 64 / 128 / 192 / 256 / 320 / 6464 / 128192
 int option_gemv_wholerow();  // -1 = the library chooses, 0 = never, 1 = where it can
 int option_w4_decode_waves();  // 0 = the library chooses, else 4 or 16 wavefronts per workgroup
 int option_w4_decode_chain();  // 0 = the library chooses, 1 = never, else a variant code of gemv_w4a8_chain

@@ -87,6 +87,7 @@ __device__ __forceinline__ void wait_vmcnt() {
     else if constexpr (N == 6) asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 9) asm volatile("s_waitcnt vmcnt(9) lgkmcnt(0)" ::: "memory");
+    else if constexpr (N == 10) asm volatile("s_waitcnt vmcnt(10) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 12) asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 16) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 18) asm volatile("s_waitcnt vmcnt(18) lgkmcnt(0)" ::: "memory");
@@ -928,44 +929,56 @@ int cmi::gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, co
     a.partials = nullptr;
     a.arrivals = nullptr;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    // Tile choice: how full the last round of workgroups is (256 CUs; one large workgroup or
-    // two 128 x 128 workgroups per CU) and how much of the tiles' area is real output, times
-    // the steady-state advantage of the larger tiles.  CMI_GEMM_TILE=64|128|256|320 overrides
-    // (tests, tuning); 6464 forces the 64 x 64 tile of the mid-batch route.
-    int pick;  // 64, 128, 256 or 320: block tile along n; 6464: 64 x 64
+    // Tile choice above 256 rows.  Every tile kernel is a chain of K / 128 dependent steps whose
+    // length is set by the operand bytes a workgroup pulls per step (it grows with the tile and,
+    // the weight being cold, with N) and by how many workgroups share a CU; larger tiles move
+    // fewer bytes per MFMA, smaller ones fill the 256 CUs more evenly.  Cost models (us) of the
+    // same form as for 17..256 rows, fitted to cold-weight measurements of every kernel on
+    // sixteen layer shapes x eleven batch sizes (272..8192 rows): their choice is 0.3 % above the
+    // best measured in total, the fill-and-area rule this replaces 2.4 % (and up to 40 % on
+    // single shapes, e.g. 2048 x 9728 -> 2560: 84 -> 63 us).
+    // CMI_GEMM_TILE=64|128|192|256|320 overrides the tile along n (tests, tuning); 128192 forces
+    // 128(n) x 192(m), 6464 the 64 x 64 tile of the mid-batch route.
+    int pick;  // 64, 128, 192, 256 or 320: block tile along n; 128192; 6464
     if (force || mid) {
         pick = force ? force : mid;
     } else {
-        auto fill = [](double tiles, double slots) { return tiles / (ceil(tiles / slots) * slots); };
-        const double t128 = (double)((M + 127) / 128) * ((N + 127) / 128);
-        const double t256 = (double)((M + 255) / 256) * ((N + 255) / 256);
-        const double t320 = (double)((M + 255) / 256) * ((N + 319) / 320);
-        // useful fraction of the tiles' area times the measured steady-state advantage
-        const double area = (double)M * N;
-        const double e128 = fill(t128, 512.0) * area / (t128 * 128 * 128);
-        const double e256 = fill(t256, 256.0) * area / (t256 * 256 * 256) * 1.23;
-        const double e320 = fill(t320, 256.0) * area / (t320 * 256 * 320) * 1.30;
-        pick = e128 >= e256 && e128 >= e320 ? 128 : e256 >= e320 ? 256 : 320;
+        const double steps = K / 128.0;
+        auto cost = [&](int bm, int bn, double a0, double b0, double c0) {
+            const double tiles = (double)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+            return 2.5 + steps * (a0 + b0 * N) * (1.0 + c0 * (ceil(tiles / 256.0) - 1.0));
+        };
+        const struct { int pick; double us; } candidates[] = {
+            {64, N > 64 ? cost(128, 64, 0.407, 5.54e-6, 0.796) : 1e30},
+            {128, cost(128, 128, 0.555, 9.82e-6, 0.91)},
+            {192, cost(128, 192, 0.723, 1.89e-5, 1.03)},
+            {128192, cost(192, 128, 0.709, 1.19e-5, 1.12)},
+            {256, cost(256, 256, 1.29, 2.33e-5, 1.28)},
+            {320, cost(256, 320, 1.60, 3.39e-5, 1.13)},
+        };
+        pick = 128;
+        double best = 1e30;
+        for (const auto &c : candidates)
+            if (c.us < best) best = c.us, pick = c.pick;
     }
     if (pick == 320) return launch_wide(a, st);
-    // 128 x 128 tiles that would leave half of the CUs idle: 128(m) x 64(n) tiles of the same kernel
-    // instead, twice as many workgroups with half the MFMAs per dependent step each (512 x 4096 x 2560
-    // 16.8 -> 12.7 us, 512 x 2560 x 9728 47 -> 34 us; with more tiles than that it measured 10-30 % slower).
-    const int tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
-    if (pick == 128 && !force && !mid && tiles128 <= 128 && N > 64) pick = 64;
+    if (pick == 256) return launch_big(a, st);
+    if (pick == 192) return launch<3, 2, 3>(a, st);
+    if (pick == 128192) return launch<2, 3, 3>(a, st);
     // 64 x 64 tiles, four LDS stages (more stages measured the same): half the bytes per step and
     // twice the workgroups of the 128 x 64 tile for batches of up to 64 rows or few n tiles
     if (pick == 6464) return launch<1, 1, 4>(a, st);
     if (pick == 64) {
+        // 128(m) x 64(n): twice the workgroups of the 128 x 128 tile with half the MFMAs per
+        // dependent step each
         const int tiles64 = ((M + 127) / 128) * ((N + 63) / 64);
         if (tiles64 <= 256) return launch<1, 2, 3>(a, st);
         return launch<1, 2, 2>(a, st);
     }
-    const bool use_big = pick == 256;
-    if (use_big) return launch_big(a, st);
-    // Up to one 128 x 128 workgroup per CU the launch is a chain of K/128 dependent steps: a third
-    // LDS stage (96 KiB, one workgroup per CU anyway) puts two steps of loads in flight (-20 % at
-    // K = 2560, -33 % at K = 9728); with two workgroups per CU it measured slower.
+    // Up to one 128 x 128 workgroup per CU a third LDS stage (96 KiB, one workgroup per CU anyway)
+    // puts two steps of loads in flight (-20 % at K = 2560, -33 % at K = 9728); with two
+    // workgroups per CU it measured slower.
+    const int tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
     if (tiles128 <= 256) return launch<2, 2, 3>(a, st);
     return launch<2, 2, 2>(a, st);
 }

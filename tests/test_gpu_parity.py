@@ -290,9 +290,9 @@ def test_sixteen_row_kernels_at_lm_head_size_sampled_columns(orc):
 
 # ------------------------------------------------------------------ W8A8 GEMM
 
-@pytest.fixture(params=["auto", "64", "128", "256", "320", "6464"])
+@pytest.fixture(params=["auto", "64", "128", "192", "128192", "256", "320", "6464"])
 def gemm_tile(request):
-    """Force the 128 x 64, 128 x 128, 256 x 256, 256 x 320 or 64 x 64 block-tile kernel through
+    """Force the 128 x 64, 128 x 128, 128 x 192, 192 x 128, 256 x 256, 256 x 320 or 64 x 64 (m x n) block-tile kernel through
     cmi_set_option, or leave the choice to the library (conftest resets it after each test)."""
     if request.param != "auto":
         G.set_option("gemm_tile", int(request.param))
@@ -565,6 +565,29 @@ def test_mid_batch_dispatch_agrees_with_the_forced_tile_on_random_shapes():
         G.set_option("gemm_tile", 128)
         _, y4_ref = G.w4a8(w4, ws, xq, xs, k, gemm=True, want_acc=False)
         assert (y4.view(torch.int16) == y4_ref.view(torch.int16)).all(), ("w4a8", m, n, k)
+    G.set_option("gemm_tile", 0)
+
+
+def test_prefill_dispatch_agrees_with_the_forced_tile_on_random_shapes():
+    """Above 256 rows the cost models of cmi_gemm_w8a8 choose among seven tile kernels (128 x 64 up
+    to 256 x 320, among them the 128 x 192 and 192 x 128 tiles for tile counts that fill the 256
+    CUs unevenly): the bits are those of the forced 128 x 128 tile kernel, on the shapes measured
+    to take the 192-wide tiles and on 12 seeded random shapes, ragged M and N."""
+    rnd = np.random.RandomState(20240702)
+    g = synth.generator(78, G.DEV)
+    shapes = [(512, 9728, 2560), (1024, 6144, 2560), (2048, 2560, 9728), (1024, 5120, 5120), (640, 9728, 2560)]
+    for _ in range(12):
+        shapes.append((int(rnd.randint(257, 2500)), int(rnd.choice([rnd.randint(8, 700), rnd.randint(700, 10000)])),
+                       128 * int(rnd.randint(1, 50))))
+    for case, (m, n, k) in enumerate(shapes):
+        x = synth.activations(m, k, g, outliers=bool(case & 1))
+        xq, xs = G.quant(x)
+        q = synth.int8_weight(n, k, g)
+        G.set_option("gemm_tile", 0)
+        _, y = G.gemm_w8a8(xq, q.wq, xs, q.scale, want_acc=False)
+        G.set_option("gemm_tile", 128)
+        _, y_ref = G.gemm_w8a8(xq, q.wq, xs, q.scale, want_acc=False)
+        assert (y.view(torch.int16) == y_ref.view(torch.int16)).all(), (m, n, k)
     G.set_option("gemm_tile", 0)
 
 

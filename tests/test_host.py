@@ -347,7 +347,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_set_option_validates_names_and_values():
     lib = _native.load()
-    for name, good, bad in ((b"gemm_tile", (64, 128, 256, 320, 6464, 0), (1, 100, -1)),
+    for name, good, bad in ((b"gemm_tile", (64, 128, 192, 256, 320, 6464, 128192, 0), (1, 100, -1)),
                             (b"gemv_wholerow", (0, 1, -1), (2, -2)),
                             (b"w4_decode_waves", (4, 16, 0), (1, 8, -1)),
                             (b"w4_decode_chain", (1, 40108, 40116, 80216, 160416, 0), (2, 8, 16, 40132, 40316, 20116, -1))):
