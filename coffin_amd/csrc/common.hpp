@@ -122,6 +122,66 @@ __device__ __forceinline__ float wave_sum_to_lane63(float v) {
     return v;
 }
 
+// The wave sums of NV per-lane values (NV = 8, 16 or 32) with the pairing of wave_sum_to_lane63 --
+// lanes l^1, l^2, then quads, half rows, rows, halves; fp32 addition commutes, so the totals have
+// the same bits -- as a transposing reduction: at each level a lane forms the pair sums of only half
+// of the values it still holds and its partner those of the other half, so the work halves per
+// level (NV + NV/2 + .. adds instead of 6 NV) and the NV totals end in NV different lanes.
+// Which half a lane keeps at levels 1..4 is chosen so that the partner of the *next* levels
+// (l^2, l^7, l^15: the DPP controls of the plain tree) holds the same values: bits
+// b0^b2, b1^b2, b2^b3, b3 of the lane number; the row and half levels swap whole rows
+// (v_permlane16_swap, v_permlane32_swap).  Returns the total of value wave_sum_transposed_index<NV>(lane);
+// lanes 0..NV-1 cover every value once.
+template <int NV>
+__device__ __forceinline__ int wave_sum_transposed_index(int lane) {
+    static_assert(NV == 8 || NV == 16 || NV == 32, "8, 16 or 32 values per lane");
+    const int s1 = (lane ^ (lane >> 2)) & 1, s2 = ((lane >> 1) ^ (lane >> 2)) & 1;
+    const int s3 = ((lane >> 2) ^ (lane >> 3)) & 1, s4 = (lane >> 3) & 1, s5 = (lane >> 4) & 1;
+    if constexpr (NV == 8) return s1 * 4 + s2 * 2 + s3;
+    else if constexpr (NV == 16) return s1 * 8 + s2 * 4 + s3 * 2 + s4;
+    else return s1 * 16 + s2 * 8 + s3 * 4 + s4 * 2 + s5;
+}
+
+template <int CTRL, int H>
+__device__ __forceinline__ void transposed_level(const float (&in)[2 * H], float (&out)[H], bool upper) {
+#pragma unroll
+    for (int i = 0; i < H; ++i) {
+        const float lo = in[i] + dpp_f32<CTRL, 0xf>(in[i]);
+        const float hi = in[i + H] + dpp_f32<CTRL, 0xf>(in[i + H]);
+        out[i] = upper ? hi : lo;
+    }
+}
+
+template <int NV>
+__device__ __forceinline__ float wave_sum_transposed(const float (&v)[NV], int lane) {
+    static_assert(NV == 8 || NV == 16 || NV == 32, "8, 16 or 32 values per lane");
+    typedef unsigned u32x2_swap __attribute__((ext_vector_type(2)));
+    float a1[NV / 2], a2[NV / 4], a3[NV / 8];
+    transposed_level<0xB1, NV / 2>(v, a1, ((lane ^ (lane >> 2)) & 1) != 0);          // l ^ 1
+    transposed_level<0x4E, NV / 4>(a1, a2, (((lane >> 1) ^ (lane >> 2)) & 1) != 0);  // l ^ 2
+    transposed_level<0x141, NV / 8>(a2, a3, (((lane >> 2) ^ (lane >> 3)) & 1) != 0); // other quad of the half row
+    float t;
+    if constexpr (NV == 8) {
+        t = a3[0] + dpp_f32<0x140, 0xf>(a3[0]);                                      // other half of the row
+    } else {
+        float a4[NV / 16];
+        transposed_level<0x140, NV / 16>(a3, a4, ((lane >> 3) & 1) != 0);
+        if constexpr (NV == 32) {
+            // rows 0+1 and 2+3: even rows end with value 0, odd rows with value 1
+            const u32x2_swap r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a4[0]), __float_as_uint(a4[1]), false, false);
+            t = __uint_as_float(r.x) + __uint_as_float(r.y);
+        } else {
+            t = a4[0];
+        }
+    }
+    if constexpr (NV != 32) {
+        const u32x2_swap r = __builtin_amdgcn_permlane16_swap(__float_as_uint(t), __float_as_uint(t), false, false);
+        t = __uint_as_float(r.x) + __uint_as_float(r.y);                              // rows 0+1, 2+3
+    }
+    const u32x2_swap h = __builtin_amdgcn_permlane32_swap(__float_as_uint(t), __float_as_uint(t), false, false);
+    return __uint_as_float(h.x) + __uint_as_float(h.y);                               // the two halves
+}
+
 // Max over the 64 lanes; every lane of row 3 ends with the wave maximum, lane
 // 63 included.  Inputs must be >= 0 (masked lanes contribute 0).
 __device__ __forceinline__ float wave_max_to_lane63(float v) {

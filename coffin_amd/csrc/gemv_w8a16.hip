@@ -265,6 +265,17 @@ gemv_w8a16_kernel(const GemvArgs a) {
     // scales it; its scale is requested here, not cold at the end
     float scale_fin = 0.f;
     if constexpr (MODE != 0) scale_fin = a.ws[min(rb * R + min(lane / M, R - 1), a.N - 1)];
+    // Four rows and more: the R * M lane sums of a unit are reduced together (wave_sum_transposed:
+    // the same tree, a sixth of the adds at 32 values) and the total of output (r, m) =
+    // (tidx / M, tidx % M) ends in lane < R * M, which scales and stores it -- one store per
+    // wavefront instead of R * M from lane 63.
+    constexpr bool TRANSPOSED = R * M >= 8;
+    int tidx = 0;
+    float scale_lane = 0.f, tot = 0.f;
+    if constexpr (TRANSPOSED) {
+        tidx = wave_sum_transposed_index<R * M>(lane);
+        if constexpr (MODE == 0) scale_lane = a.ws[min(rb * R + tidx / M, a.N - 1)];
+    }
     if constexpr (XLDS) {
 #pragma unroll
         for (int j = 0; j < XV; ++j) {
@@ -355,13 +366,24 @@ gemv_w8a16_kernel(const GemvArgs a) {
             }
         }
         if (MODE != 0 && u + a.uw < a.units) load_w(w0, u + a.uw, 0);  // next unit of this wavefront
+        if constexpr (TRANSPOSED) {
+            float flat[R * M];
 #pragma unroll
-        for (int r = 0; r < R; ++r)
+            for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int m = 0; m < M; ++m) acc[r][m] = wave_sum_to_lane63(acc[r][m]);
+                for (int m = 0; m < M; ++m) flat[r * M + m] = acc[r][m];
+            tot = wave_sum_transposed<R * M>(flat, lane);
+        } else {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int m = 0; m < M; ++m) acc[r][m] = wave_sum_to_lane63(acc[r][m]);
+        }
         if constexpr (MODE == 0) break;
         // unit totals meet in LDS; one lane per output adds them in unit order below
-        if (lane == 63) {
+        if constexpr (TRANSPOSED) {
+            if (lane < R * M) unit_total[u * (R * M) + tidx] = tot;
+        } else if (lane == 63) {
 #pragma unroll
             for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -373,7 +395,12 @@ gemv_w8a16_kernel(const GemvArgs a) {
             for (int m = 0; m < M; ++m) acc[r][m] = 0.f;
     }
 
-    if constexpr (MODE == 0) {
+    if constexpr (MODE == 0 && TRANSPOSED) {
+        const int r = tidx / M, m = tidx - r * M;
+        const int n = rb * R + r;
+        if (!idle && lane < R * M && n < a.N && m < a.M)
+            a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(scale_lane * tot);
+    } else if constexpr (MODE == 0) {
         if (!idle && lane == 63) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
