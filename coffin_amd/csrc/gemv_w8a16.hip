@@ -37,7 +37,9 @@
 // weights in flight.  When K spans several units the wavefronts of a team each take units
 // of the same rows and the unit totals meet in LDS (summed in unit order by one
 // lane per output); otherwise lane 63, which holds the tree result, scales and
-// stores.  A single activation row against a K of two or three units (and against a
+// stores.  From four activation rows on the 8..32 lane sums of a wavefront go through
+// the tree together (wave_sum_transposed: same pairing, same bits, a lane keeping half
+// of its values per level) and end in as many lanes, which store in parallel.  A single activation row against a K of two or three units (and against a
 // mid-sized weight with K in one unit) takes gemv_w8a16_wholerow_kernel instead: one
 // wavefront per weight row, all units.
 
