@@ -591,6 +591,69 @@ def test_prefill_dispatch_agrees_with_the_forced_tile_on_random_shapes():
     G.set_option("gemm_tile", 0)
 
 
+def test_random_shapes_and_forced_tiles_against_the_oracle(orc):
+    """150 seeded random cases straight against the oracle, bit for bit: W8A8 and W4A8 GEMM with a
+    random forced tile (or the library's choice), the W4A8 GEMV, and the two linear entry points
+    (quantiser + GEMM through a 0xA5-filled workspace of either size); M in 1..1400 (1..16 for the
+    GEMV), N in 1..4000, K up to 11008 in steps of 128 (16 for some W8A8 cases), with and without
+    the integer sums.  The shapes are bounded so that the CPU side takes seconds."""
+    from coffin_amd import _native
+    lib = _native.load()
+    rnd = np.random.RandomState(20240815)
+    g = synth.generator(79, G.DEV)
+
+    def pick(*ranges):
+        lo, hi = ranges[rnd.randint(len(ranges))]
+        return int(rnd.randint(lo, hi))
+
+    for case in range(150):
+        kind = ("w8a8", "w4a8", "w4a8_gemv", "linear_w8a8", "linear_w4a8")[rnd.randint(5)]
+        m = pick((1, 17), (17, 130), (130, 300), (300, 1400)) if kind != "w4a8_gemv" else pick((1, 17))
+        n = pick((1, 70), (70, 700), (700, 4000))
+        step = 16 if kind in ("w8a8", "linear_w8a8") and rnd.rand() < 0.3 else 128
+        k = step * pick((1, 9), (9, 41), (41, 11008 // step + 1))
+        while m * n * k > 2e9:
+            m = max(1, m // 2)
+        tile = int(rnd.choice([0, 0, 0, 64, 128, 192, 128192, 256, 320, 6464]))
+        want_acc = bool(rnd.randint(2))
+        what = (case, kind, m, n, k, tile, want_acc)
+        x = synth.activations(m, k, g, outliers=bool(rnd.randint(2)))
+        xq, xs = G.quant(x)
+        xq_ref, xs_ref = orc.quant_act_i8(G.bits(x))
+        assert (xq.cpu().numpy() == xq_ref).all() and (xs.cpu().numpy() == xs_ref).all(), what
+        y = torch.empty((m, n), dtype=torch.bfloat16, device=G.DEV)
+        if kind in ("w8a8", "linear_w8a8"):
+            q = synth.int8_weight(n, k, g)
+            acc_ref, y_ref = orc.gemm_w8a8(xq_ref, q.wq.cpu().numpy(), xs_ref, q.scale.cpu().numpy())
+            if kind == "w8a8":
+                G.set_option("gemm_tile", tile)
+                acc, y = G.gemm_w8a8(xq, q.wq, xs, q.scale, want_acc=want_acc)
+                G.set_option("gemm_tile", 0)
+                assert not want_acc or (acc.cpu().numpy() == acc_ref).all(), what
+            else:
+                size = int(lib.cmi_linear_w8a8_workspace_bytes(m, n, k) if want_acc else lib.cmi_linear_workspace_bytes(m, k))
+                work = torch.full((size,), 0xA5, dtype=torch.uint8, device=G.DEV)
+                _native.check(lib.cmi_linear_w8a8_bf16(G.ptr(x), G.ptr(q.wq), G.ptr(q.scale), G.ptr(y), m, n, k, n,
+                                                       G.ptr(work), size, G.stream()), "linear_w8a8")
+        else:
+            w = synth.int4_weight(n, k, g)
+            w4, ws = G.w4_repack(w.packed, w.scale, k)
+            gacc_ref, y_ref = orc.linear_w4a8(xq_ref, xs_ref, w.packed.cpu().numpy(), w.scale.cpu().numpy(), k,
+                                              want_group_acc=True)
+            if kind == "linear_w4a8":
+                size = int(lib.cmi_linear_workspace_bytes(m, k))
+                work = torch.full((size,), 0xA5, dtype=torch.uint8, device=G.DEV)
+                _native.check(lib.cmi_linear_w4a8_bf16(G.ptr(w4), G.ptr(ws), G.ptr(x), G.ptr(y), m, n, k, 128,
+                                                       G.ptr(work), size, G.stream()), "linear_w4a8")
+            else:
+                if kind == "w4a8":
+                    G.set_option("gemm_tile", tile)
+                gacc, y = G.w4a8(w4, ws, xq, xs, k, gemm=(kind == "w4a8"), want_acc=want_acc)
+                G.set_option("gemm_tile", 0)
+                assert not want_acc or (gacc.cpu().numpy() == gacc_ref).all(), what
+        assert (G.bits(y) == y_ref).all(), what
+
+
 def test_w4a8_golden_and_chain_order(golden):
     g = golden("linear_w4a8")
     k = int(g["a_k"])
