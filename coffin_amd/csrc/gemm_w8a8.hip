@@ -43,6 +43,7 @@ namespace {
 using namespace cmi;
 
 constexpr int BK = 128;        // one 128-byte cache line per row and step
+constexpr double SPLIT128_HANDOVER_US = 11.0;  // split-K on 128 x 128 tiles: partials out, arrival, partials in (measured 10..11.5)
 constexpr int THREADS = 256;   // 2 x 2 wavefronts
 
 struct Args {
@@ -407,12 +408,13 @@ gemm_w8a8_pipe_kernel(const Args a) {
         __syncthreads();
         if (arrived_before != a.splits - 1) return;  // uniform: not the last workgroup of the tile
         // all the others' elements are requested before the first is added (one trip to memory,
-        // not one per split): four splits' worth at a time, slots past the last split or on this
+        // not one per split): four (two) splits' worth at a time, slots past the last split or on this
         // workgroup's own partial re-read split 0 and count for nothing
-        for (int s0 = 0; s0 < a.splits; s0 += 4) {
-            int theirs[4][ELEMS];
+        constexpr int AT_A_TIME = ELEMS <= 32 ? 4 : 2;  // registers: 4 x 32 or 2 x 64 partial elements
+        for (int s0 = 0; s0 < a.splits; s0 += AT_A_TIME) {
+            int theirs[AT_A_TIME][ELEMS];
 #pragma unroll
-            for (int d = 0; d < 4; ++d) {
+            for (int d = 0; d < AT_A_TIME; ++d) {
                 const int s = s0 + d < a.splits ? s0 + d : 0;
                 const int *src = a.partials + ((size_t)s * tiles + tile) * (ELEMS * THREADS) + threadIdx.x;
 #pragma unroll
@@ -420,7 +422,7 @@ gemm_w8a8_pipe_kernel(const Args a) {
                     theirs[d][e] = __hip_atomic_load(src + e * THREADS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
 #pragma unroll
-            for (int d = 0; d < 4; ++d) {
+            for (int d = 0; d < AT_A_TIME; ++d) {
                 const bool counts = s0 + d < a.splits && s0 + d != split;
 #pragma unroll
                 for (int i = 0; i < TN; ++i)
@@ -448,18 +450,18 @@ int launch(Args &a, hipStream_t st) {
     return check_launch("cmi_gemm_w8a8");
 }
 
-// Split-K launch of the 64 x 64 or the 128(m) x 64(n) tile: a.splits, a.partials and a.arrivals set
-// by the caller.
-template <int TM, int NST>
+// Split-K launch of the 64 x 64, the 128(m) x 64(n) or the 128 x 128 tile: a.splits, a.partials and
+// a.arrivals set by the caller.
+template <int TN, int TM, int NST>
 int launch_split(Args &a, hipStream_t st) {
-    using C = Cfg<1, TM, NST>;
+    using C = Cfg<TN, TM, NST>;
     a.tiles_m = (a.M + C::BM - 1) / C::BM;
     a.tiles_n = (a.N + C::BN - 1) / C::BN;
     static std::atomic<uint64_t> devices{0};
-    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_pipe_kernel<1, TM, NST, true>),
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_pipe_kernel<TN, TM, NST, true>),
                                    C::LDS_BYTES, devices, "cmi_gemm_w8a8"))
         return rc;
-    gemm_w8a8_pipe_kernel<1, TM, NST, true><<<dim3(a.tiles_m * a.tiles_n * a.splits), dim3(THREADS), C::LDS_BYTES, st>>>(a);
+    gemm_w8a8_pipe_kernel<TN, TM, NST, true><<<dim3(a.tiles_m * a.tiles_n * a.splits), dim3(THREADS), C::LDS_BYTES, st>>>(a);
     return check_launch("cmi_gemm_w8a8");
 }
 
@@ -815,8 +817,13 @@ extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs
 }
 
 size_t cmi::gemm_w8a8_split_bytes(int M, int N, int K) {
+    if (M <= 16 || K % BK != 0 || N < 8) return 0;
     // up to 256 workgroups of 64 x 64 or 128 x 64 int32 each, whatever the split
-    return M > 16 && M <= 256 && K % BK == 0 && N >= 8 ? (size_t)256 * 128 * 64 * 4 : 0;
+    if (M <= 256) return (size_t)256 * 128 * 64 * 4;
+    // up to 1024 rows of a narrow, long projection (at most 128 tiles of 128 x 128, 16 K steps and
+    // more): up to 256 workgroups of 128 x 128 int32
+    const int tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+    return M <= 1024 && tiles128 <= 128 && K / BK >= 16 ? (size_t)256 * 128 * 128 * 4 : 0;
 }
 
 int cmi::gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws, void *y,
@@ -898,8 +905,8 @@ int cmi::gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, co
             a.splits = wide_m ? splits_g : splits;
             a.partials = static_cast<int32_t *>(partials);
             a.arrivals = arrivals;
-            return wide_m ? launch_split<2, 3>(a, static_cast<hipStream_t>(stream))
-                          : launch_split<1, 4>(a, static_cast<hipStream_t>(stream));
+            return wide_m ? launch_split<1, 2, 3>(a, static_cast<hipStream_t>(stream))
+                          : launch_split<1, 1, 4>(a, static_cast<hipStream_t>(stream));
         }
         if (t_rows <= t_h && t_rows <= t_g && t_rows <= t_t) {
             for (int lo = 0; lo < M; lo += 128) {
@@ -960,6 +967,23 @@ int cmi::gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, co
         double best = 1e30;
         for (const auto &c : candidates)
             if (c.us < best) best = c.us, pick = c.pick;
+        // Split-K on the 128 x 128 tile where the caller brought room for the partial tiles: a long,
+        // narrow projection (9728 -> 2560 at 257..512 rows: 60..80 tiles x 76 steps) leaves most
+        // of the CUs idle for a long chain of steps (quantiser + GEMM 38..42 -> 30..34.5 us).  Model
+        // as for the smaller tiles; the hand-over moves 64 KiB per workgroup.
+        const int tiles128 = ((M + 127) / 128) * ((N + 127) / 128);
+        if (arrivals && partials && tiles128 <= 128 && steps >= 16) {
+            int splits = 256 / tiles128;
+            if (splits > steps / 4) splits = (int)(steps / 4);
+            if (splits > 8) splits = 8;
+            const double t_split = 2.5 + fmax(ceil(steps / splits) * (0.554 + 1.11e-5 * N), (double)N * K / 5.0e6) + SPLIT128_HANDOVER_US;
+            if (splits >= 2 && (size_t)splits * tiles128 * 128 * 128 * 4 <= partial_bytes && t_split < best) {
+                a.splits = splits;
+                a.partials = static_cast<int32_t *>(partials);
+                a.arrivals = arrivals;
+                return launch_split<2, 2, 3>(a, st);
+            }
+        }
     }
     if (pick == 320) return launch_wide(a, st);
     if (pick == 256) return launch_big(a, st);

@@ -168,8 +168,9 @@ int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const fl
  *     entry up to 16 rows, the GEMM entry beyond. */
 size_t cmi_linear_workspace_bytes(int M, int K);
 /* A workspace of cmi_linear_w8a8_workspace_bytes(M, N, K) bytes -- the above plus, for 17..256 rows,
- * 256 arrival counters and 8 MiB of partial tiles -- lets cmi_linear_w8a8_bf16 split K over the
- * idle CUs where a projection is few tiles and many K steps (same bits: the partial sums are
+ * 256 arrival counters and 8 MiB of partial tiles (16 MiB for 257..1024 rows of a projection of at
+ * most 128 tiles of 128 x 128 and K >= 2048) -- lets cmi_linear_w8a8_bf16 split K over the idle
+ * CUs where a projection is few tiles and many K steps (same bits: the partial sums are
  * integers); with the smaller workspace it does not split.  No counterpart in the reference. */
 size_t cmi_linear_w8a8_workspace_bytes(int M, int N, int K);
 int cmi_linear_w8a8_bf16(const void *x, const int8_t *wq, const float *ws, void *y, int M, int N,

@@ -78,9 +78,9 @@ def test_kn_stored_weight_gives_the_bits_of_the_row_major_one():
     assert (backend.linear(q, x[0]).view(torch.int16) == backend.linear(kn, x[0]).view(torch.int16)).all()
 
 
-@pytest.mark.parametrize("rows", [64, 100, 192])
+@pytest.mark.parametrize("rows", [64, 100, 192, 300, 512])
 def test_prefill_chunk_on_a_long_narrow_projection_splits_k_with_the_same_bits(rows):
-    """64..256 rows of a down-projection shape (few tiles, many K steps): the adapter's workspace
+    """64..512 rows of a down-projection shape (few tiles, many K steps): the adapter's workspace
     lets the fused entry split K; output is that of quantiser + cmi_gemm_w8a8 (which never splits)."""
     g = synth.generator()
     q = _q8(2560, 9728, g)

@@ -268,10 +268,14 @@ def test_linear_w4a8_bf16_equals_quantiser_plus_kernels(orc, m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(64, 2560, 9728), (128, 2560, 9728), (33, 4096, 11008), (100, 1500, 10240),
                                    (20, 2560, 11008), (160, 2560, 9728), (250, 2500, 11008), (64, 1024, 2560),
-                                   (256, 4096, 2560)])
+                                   (256, 4096, 2560),
+                                   # 257..1024 rows: 128 x 128 tiles in three, two, eight, five and four parts
+                                   (300, 2560, 9728), (512, 2560, 9728), (640, 2560, 9728), (400, 1000, 8192),
+                                   (700, 1024, 8192), (1024, 1024, 4096)])
 def test_linear_w8a8_bf16_split_k_same_bits(orc, m, n, k):
     """With the larger workspace the entry may split K over the idle CUs (few tiles, many K steps:
-    the first five shapes on the 64 x 64 tile, the next two on the 128 x 64 tile; the last two stay unsplit): the partial sums are integers, so output
+    the first five shapes on the 64 x 64 tile, the next two on the 128 x 64 tile, the next two stay
+    unsplit, the rest take or may take the 128 x 128 tile in parts): the partial sums are integers, so output
     and quantised rows are those of the small workspace and of the oracle, also with a row stride,
     and on a second call (the arrival counters are cleared by every call's quantiser launch)."""
     lib = _native.load()
