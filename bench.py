@@ -635,10 +635,12 @@ def main() -> int:
         # 64 and 128 rows (between the GEMV and the tile pipeline) on the two MLP shapes, the three
         # weight formats as the adapter issues them: weight-only on the matrix-pipe GEMV (64 rows per
         # call), cmi_linear_w8a8_bf16 and cmi_linear_w4a8_bf16 (quantiser + GEMM) on the adapter's workspace
-        for m in (64, 128):
+        # and a 512-row prefill chunk (a chat-sized prompt) on the four layer shapes, W8A8 and W4A8
+        for m in (64, 128, 512):
             mid = {}
-            for n_, k_ in ((9728, 2560), (2560, 9728)):
-                copies = 12
+            shapes = ((9728, 2560), (2560, 9728)) if m < 512 else ((6144, 2560), (2560, 4096), (19456, 2560), (2560, 9728))
+            for n_, k_ in shapes:
+                copies = max(12, -(-300_000_000 // (n_ * k_)))
                 w8 = [synth.int8_weight(n_, k_, gen) for _ in range(copies)]
                 w4_ = []
                 for _ in range(copies):
@@ -677,10 +679,10 @@ def main() -> int:
                     with torch.cuda.graph(gr):
                         fn()
                     return timed(gr.replay, 5) / copies
-                mid[f"{k_}->{n_}"] = {name: round(replayed(fn) * 1e6, 2)
-                                      for name, fn in (("weight_only_us", weight_only), ("w8a8_us", w8a8), ("w4a8_us", w4a8))}
+                routes = (("weight_only_us", weight_only), ("w8a8_us", w8a8), ("w4a8_us", w4a8))
+                mid[f"{k_}->{n_}"] = {name: round(replayed(fn) * 1e6, 2) for name, fn in routes[(0 if m < 512 else 1):]}
                 del w8, w4_
-            extra[f"mid_batch_M{m}"] = mid
+            extra[f"mid_batch_M{m}" if m < 512 else f"prefill_chunk_M{m}_quant_plus_gemm"] = mid
         torch.cuda.empty_cache()
         torch.cuda.empty_cache()
 
