@@ -65,7 +65,7 @@ def cpu_baseline(budget_s: float, synth, torch) -> dict:
     on the host cores: torch eager evaluating backends/reference/__init__.py:93-95 --
     ``dense = (wq.float() * scale[:, None]).to(bf16)``; ``y = F.linear(x, dense)`` -- *faithful*
     (the dequantisation inside every call, as the reference does) and *hoisted* (dequantised once,
-    outside the clock), each at all cores and at one thread.  Median of up to 5 calls after up to 2
+    outside the clock), each at all cores and at one thread.  Median of up to 25 calls after up to 2
     warm-ups per shape, fewer when the time budget (a quarter of ``budget_s`` per variant) runs
     out.  The C oracle of the same path is reported beside it as a labelled extra."""
     import statistics
@@ -86,7 +86,7 @@ def cpu_baseline(budget_s: float, synth, torch) -> dict:
         for wq, sc, x, _ in layer:
             dense = (wq.float() * sc[:, None]).to(torch.bfloat16) if hoisted else None
             times = []
-            for i in range(7):
+            for i in range(27):
                 t0 = time.perf_counter()
                 d = dense if hoisted else (wq.float() * sc[:, None]).to(torch.bfloat16)
                 F.linear(x, d)
