@@ -61,6 +61,9 @@ struct Args {
     int splits;
     int32_t *partials;
     int *arrivals;
+    // pipe kernel: workgroups launched beyond the tiles (x splits), on CUs the tiles leave idle;
+    // they read the weight through the caches (see warm_weight)
+    int warm_blocks;
 };
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
@@ -227,6 +230,30 @@ __device__ __forceinline__ void epilogue(const Args &a, v16i32 (&acc)[TN][TM], i
     }
 }
 
+// Few tiles: the launch is a chain of K / 128 steps, each as long as a CU needs to pull the
+// step's operands, and the weight comes from DRAM in 128-byte pieces of 64..128 rows per tile --
+// a third slower than from the memory-side cache (Infinity Cache, 256 MiB, shared by all CUs).
+// The CUs that have no tile therefore read the weight front to back, in whole rows, at memory
+// speed, and drop it: after a few microseconds the tiles' requests are answered by that cache.
+// Workgroup `part` of `parts`, eight 16-byte requests in flight per thread.
+__device__ __forceinline__ void warm_weight(const Args &a, int part, int parts) {
+    const uint4 *p = reinterpret_cast<const uint4 *>(a.wq);
+    const size_t n = (size_t)a.N * a.K / 16;
+    const size_t stride = (size_t)parts * THREADS;
+    size_t i = (size_t)part * THREADS + threadIdx.x;
+    for (; i + 7 * stride < n; i += 8 * stride) {
+        uint4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = p[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) asm volatile("" ::"v"(v[u].x), "v"(v[u].y), "v"(v[u].z), "v"(v[u].w));
+    }
+    for (; i < n; i += stride) {
+        const uint4 v = p[i];
+        asm volatile("" ::"v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w));
+    }
+}
+
 // SPLIT: a.splits workgroups share a tile, each walking a contiguous part of K; they leave their
 // int32 accumulators in a.partials and the last to arrive (a.arrivals, cleared before the launch)
 // adds the others' to its own -- integer sums, exact in any order -- and runs the epilogue: the
@@ -243,6 +270,11 @@ gemm_w8a8_pipe_kernel(const Args a) {
     const int wn = wave & 1, wm = wave >> 1;
 
     const int tiles = a.tiles_m * a.tiles_n;
+    const int work = SPLIT ? tiles * a.splits : tiles;
+    if ((int)blockIdx.x >= work) {  // uniform: no tile, and before any barrier
+        warm_weight(a, blockIdx.x - work, a.warm_blocks);
+        return;
+    }
     const int tile = SPLIT ? blockIdx.x % tiles : blockIdx.x, split = SPLIT ? blockIdx.x / tiles : 0;
     int tm, tn;
     tile_coords(a, tm, tn, tile);
@@ -437,6 +469,15 @@ gemm_w8a8_pipe_kernel(const Args a) {
                      scales + C::BN + wm * 32 * TM);
 }
 
+// How many workgroups beyond `work` read the weight through the caches: one per CU that would
+// otherwise idle, where at least a quarter of the chip would, the weight is at most 64 MiB and
+// its 16-byte vectors are whole.  (With every CU busy, 32 or 64 such workgroups on top measured
+// faster on some shapes and up to 30 % slower on others: not done.)
+int warm_blocks(const Args &a, int work) {
+    if (work > 192 || (size_t)a.N * a.K > ((size_t)64 << 20) || !aligned(a.wq, 16) || ((size_t)a.N * a.K) % 16 != 0) return 0;
+    return 256 - work;
+}
+
 template <int TN, int TM, int NST>
 int launch(Args &a, hipStream_t st) {
     using C = Cfg<TN, TM, NST>;
@@ -446,7 +487,8 @@ int launch(Args &a, hipStream_t st) {
     if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_pipe_kernel<TN, TM, NST>),
                                    C::LDS_BYTES, devices, "cmi_gemm_w8a8"))
         return rc;
-    gemm_w8a8_pipe_kernel<TN, TM, NST><<<dim3(a.tiles_m * a.tiles_n), dim3(THREADS), C::LDS_BYTES, st>>>(a);
+    a.warm_blocks = warm_blocks(a, a.tiles_m * a.tiles_n);
+    gemm_w8a8_pipe_kernel<TN, TM, NST><<<dim3(a.tiles_m * a.tiles_n + a.warm_blocks), dim3(THREADS), C::LDS_BYTES, st>>>(a);
     return check_launch("cmi_gemm_w8a8");
 }
 
@@ -461,7 +503,8 @@ int launch_split(Args &a, hipStream_t st) {
     if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_pipe_kernel<TN, TM, NST, true>),
                                    C::LDS_BYTES, devices, "cmi_gemm_w8a8"))
         return rc;
-    gemm_w8a8_pipe_kernel<TN, TM, NST, true><<<dim3(a.tiles_m * a.tiles_n * a.splits), dim3(THREADS), C::LDS_BYTES, st>>>(a);
+    a.warm_blocks = warm_blocks(a, a.tiles_m * a.tiles_n * a.splits);
+    gemm_w8a8_pipe_kernel<TN, TM, NST, true><<<dim3(a.tiles_m * a.tiles_n * a.splits + a.warm_blocks), dim3(THREADS), C::LDS_BYTES, st>>>(a);
     return check_launch("cmi_gemm_w8a8");
 }
 
