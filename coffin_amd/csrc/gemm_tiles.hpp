@@ -1,5 +1,5 @@
-// Pieces the block-tiled GEMM kernels share: the order in which workgroups take output tiles, and
-// the widening of a packed int4 weight piece to int8.
+// Pieces the block-tiled GEMM kernels share: the order in which workgroups take output tiles, the
+// widening of a packed int4 weight piece to int8, and the warming of the caches by idle CUs.
 #pragma once
 #include <cstdint>
 #include <hip/hip_runtime.h>
@@ -43,6 +43,42 @@ __device__ __forceinline__ void widen_w4_piece(uint32_t w0, uint32_t w1, uint32_
     hi.y = rebias4((w2 >> 4) & 0x0F0F0F0Fu);
     hi.z = rebias4(w3 & 0x0F0F0F0Fu);
     hi.w = rebias4((w3 >> 4) & 0x0F0F0F0Fu);
+}
+
+// Few tiles: a tile launch is a chain of K / 128 steps, each as long as a CU needs to pull the
+// step's operands, and the weight comes from DRAM in 128-byte pieces of 64..128 rows per tile -- a
+// third slower than from the memory-side cache (Infinity Cache, 256 MiB, shared by all CUs).  The
+// CUs that have no tile therefore read the weight front to back at memory speed and drop it:
+// after a few microseconds the tiles' requests are answered by that cache.  (W8A8 tiles: -15..-25 %
+// on cold weights.  The W4A8 ring kernels, whose step is set by the widening and the per-group
+// flush rather than by the operand stream, measured the same with and without: not used there.)
+// Workgroup `part` of `parts` (256 threads each) reads its share of `bytes` (a multiple of 16,
+// p 16-byte aligned), eight 16-byte requests in flight per thread.
+__device__ __forceinline__ void warm_caches(const void *p, size_t bytes, int part, int parts) {
+    const uint4 *v4 = static_cast<const uint4 *>(p);
+    const size_t n = bytes / 16;
+    const size_t stride = (size_t)parts * 256;
+    size_t i = (size_t)part * 256 + threadIdx.x;
+    for (; i + 7 * stride < n; i += 8 * stride) {
+        uint4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = v4[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) asm volatile("" ::"v"(v[u].x), "v"(v[u].y), "v"(v[u].z), "v"(v[u].w));
+    }
+    for (; i < n; i += stride) {
+        const uint4 v = v4[i];
+        asm volatile("" ::"v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w));
+    }
+}
+
+// How many workgroups beyond the `work` that hold tiles read `bytes` of weight through the caches:
+// one per CU that would otherwise idle, where at least a quarter of the chip would, the weight is
+// at most 64 MiB and its 16-byte vectors are whole.  (With every CU busy, 32 or 64 such workgroups
+// on top measured faster on some shapes and up to 30 % slower on others: not done.)
+inline int warm_workgroups(const void *p, size_t bytes, int work) {
+    if (work > 192 || bytes > ((size_t)64 << 20) || (reinterpret_cast<uintptr_t>(p) & 15) != 0 || bytes % 16 != 0) return 0;
+    return 256 - work;
 }
 
 }  // namespace cmi

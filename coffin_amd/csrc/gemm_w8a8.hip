@@ -62,7 +62,7 @@ struct Args {
     int32_t *partials;
     int *arrivals;
     // pipe kernel: workgroups launched beyond the tiles (x splits), on CUs the tiles leave idle;
-    // they read the weight through the caches (see warm_weight)
+    // they read the weight through the caches (warm_caches in gemm_tiles.hpp)
     int warm_blocks;
 };
 
@@ -230,30 +230,6 @@ __device__ __forceinline__ void epilogue(const Args &a, v16i32 (&acc)[TN][TM], i
     }
 }
 
-// Few tiles: the launch is a chain of K / 128 steps, each as long as a CU needs to pull the
-// step's operands, and the weight comes from DRAM in 128-byte pieces of 64..128 rows per tile --
-// a third slower than from the memory-side cache (Infinity Cache, 256 MiB, shared by all CUs).
-// The CUs that have no tile therefore read the weight front to back, in whole rows, at memory
-// speed, and drop it: after a few microseconds the tiles' requests are answered by that cache.
-// Workgroup `part` of `parts`, eight 16-byte requests in flight per thread.
-__device__ __forceinline__ void warm_weight(const Args &a, int part, int parts) {
-    const uint4 *p = reinterpret_cast<const uint4 *>(a.wq);
-    const size_t n = (size_t)a.N * a.K / 16;
-    const size_t stride = (size_t)parts * THREADS;
-    size_t i = (size_t)part * THREADS + threadIdx.x;
-    for (; i + 7 * stride < n; i += 8 * stride) {
-        uint4 v[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = p[i + u * stride];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) asm volatile("" ::"v"(v[u].x), "v"(v[u].y), "v"(v[u].z), "v"(v[u].w));
-    }
-    for (; i < n; i += stride) {
-        const uint4 v = p[i];
-        asm volatile("" ::"v"(v.x), "v"(v.y), "v"(v.z), "v"(v.w));
-    }
-}
-
 // SPLIT: a.splits workgroups share a tile, each walking a contiguous part of K; they leave their
 // int32 accumulators in a.partials and the last to arrive (a.arrivals, cleared before the launch)
 // adds the others' to its own -- integer sums, exact in any order -- and runs the epilogue: the
@@ -272,7 +248,7 @@ gemm_w8a8_pipe_kernel(const Args a) {
     const int tiles = a.tiles_m * a.tiles_n;
     const int work = SPLIT ? tiles * a.splits : tiles;
     if ((int)blockIdx.x >= work) {  // uniform: no tile, and before any barrier
-        warm_weight(a, blockIdx.x - work, a.warm_blocks);
+        warm_caches(a.wq, (size_t)a.N * a.K, blockIdx.x - work, a.warm_blocks);
         return;
     }
     const int tile = SPLIT ? blockIdx.x % tiles : blockIdx.x, split = SPLIT ? blockIdx.x / tiles : 0;
@@ -469,15 +445,6 @@ gemm_w8a8_pipe_kernel(const Args a) {
                      scales + C::BN + wm * 32 * TM);
 }
 
-// How many workgroups beyond `work` read the weight through the caches: one per CU that would
-// otherwise idle, where at least a quarter of the chip would, the weight is at most 64 MiB and
-// its 16-byte vectors are whole.  (With every CU busy, 32 or 64 such workgroups on top measured
-// faster on some shapes and up to 30 % slower on others: not done.)
-int warm_blocks(const Args &a, int work) {
-    if (work > 192 || (size_t)a.N * a.K > ((size_t)64 << 20) || !aligned(a.wq, 16) || ((size_t)a.N * a.K) % 16 != 0) return 0;
-    return 256 - work;
-}
-
 template <int TN, int TM, int NST>
 int launch(Args &a, hipStream_t st) {
     using C = Cfg<TN, TM, NST>;
@@ -487,7 +454,7 @@ int launch(Args &a, hipStream_t st) {
     if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_pipe_kernel<TN, TM, NST>),
                                    C::LDS_BYTES, devices, "cmi_gemm_w8a8"))
         return rc;
-    a.warm_blocks = warm_blocks(a, a.tiles_m * a.tiles_n);
+    a.warm_blocks = warm_workgroups(a.wq, (size_t)a.N * a.K, a.tiles_m * a.tiles_n);
     gemm_w8a8_pipe_kernel<TN, TM, NST><<<dim3(a.tiles_m * a.tiles_n + a.warm_blocks), dim3(THREADS), C::LDS_BYTES, st>>>(a);
     return check_launch("cmi_gemm_w8a8");
 }
@@ -503,7 +470,7 @@ int launch_split(Args &a, hipStream_t st) {
     if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_pipe_kernel<TN, TM, NST, true>),
                                    C::LDS_BYTES, devices, "cmi_gemm_w8a8"))
         return rc;
-    a.warm_blocks = warm_blocks(a, a.tiles_m * a.tiles_n * a.splits);
+    a.warm_blocks = warm_workgroups(a.wq, (size_t)a.N * a.K, a.tiles_m * a.tiles_n * a.splits);
     gemm_w8a8_pipe_kernel<TN, TM, NST, true><<<dim3(a.tiles_m * a.tiles_n * a.splits + a.warm_blocks), dim3(THREADS), C::LDS_BYTES, st>>>(a);
     return check_launch("cmi_gemm_w8a8");
 }
@@ -899,9 +866,12 @@ int cmi::gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, co
         const double tiles_h = (double)((M + 63) / 64) * ((N + 63) / 64);
         const double tiles_g = (double)((M + 127) / 128) * ((N + 63) / 64);
         const double tiles_t = (double)((M + 127) / 128) * ((N + 127) / 128);
-        const double t_h = 2.5 + steps * (0.22 + N * 1.6e-5) * (1.0 + 0.50 * (rounds(tiles_h) - 1));
-        const double t_g = 2.5 + steps * (0.36 + N * 1.2e-5) * (1.0 + 0.75 * (rounds(tiles_g) - 1));
-        const double t_t = 2.5 + steps * (0.50 + N * 1.5e-5) * (1.0 + 0.65 * (rounds(tiles_t) - 1));
+        // up to 192 tiles the idle CUs read the weight through the caches meanwhile (warm_caches):
+        // steps measured 13 % (64 x 64) and 20-25 % (the larger tiles) shorter
+        auto warmed = [&](double tiles, double f) { return tiles <= 192 && wbytes <= 64.0 * 1048576.0 ? f : 1.0; };
+        const double t_h = 2.5 + steps * (0.22 + N * 1.6e-5) * warmed(tiles_h, 0.87) * (1.0 + 0.50 * (rounds(tiles_h) - 1));
+        const double t_g = 2.5 + steps * (0.36 + N * 1.2e-5) * warmed(tiles_g, 0.78) * (1.0 + 0.75 * (rounds(tiles_g) - 1));
+        const double t_t = 2.5 + steps * (0.50 + N * 1.5e-5) * warmed(tiles_t, 0.78) * (1.0 + 0.65 * (rounds(tiles_t) - 1));
         double t_rows = 1e30;
         if (K <= 10240) {
             const double per_chunk = 0.5 + wbytes / (gemm_w8a8_rows_tiles(N) * 2.0e7);
@@ -996,7 +966,9 @@ int cmi::gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, co
         const double steps = K / 128.0;
         auto cost = [&](int bm, int bn, double a0, double b0, double c0) {
             const double tiles = (double)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
-            return 2.5 + steps * (a0 + b0 * N) * (1.0 + c0 * (ceil(tiles / 256.0) - 1.0));
+            // the 4-wavefront tiles on up to 192 CUs: the idle CUs warm the caches (see above)
+            const double warmed = bm <= 192 && tiles <= 192 && (double)N * K <= 64.0 * 1048576.0 ? 0.8 : 1.0;
+            return 2.5 + steps * (a0 + b0 * N) * warmed * (1.0 + c0 * (ceil(tiles / 256.0) - 1.0));
         };
         const struct { int pick; double us; } candidates[] = {
             {64, N > 64 ? cost(128, 64, 0.407, 5.54e-6, 0.796) : 1e30},
