@@ -73,11 +73,12 @@ __device__ __forceinline__ void warm_caches(const void *p, size_t bytes, int par
 }
 
 // How many workgroups beyond the `work` that hold tiles read `bytes` of weight through the caches:
-// one per CU that would otherwise idle, where at least a quarter of the chip would, the weight is
-// at most 64 MiB and its 16-byte vectors are whole.  (With every CU busy, 32 or 64 such workgroups
-// on top measured faster on some shapes and up to 30 % slower on others: not done.)
+// one per CU that would otherwise idle, where at least an eighth of the chip would (32 of them still
+// gain 3-7 % at 216..224 tiles, 8..16 nothing), the weight is at most 64 MiB and its 16-byte
+// vectors are whole.  (With every CU busy, 32 or 64 such workgroups on top measured faster on some
+// shapes and up to 30 % slower on others: not done.)
 inline int warm_workgroups(const void *p, size_t bytes, int work) {
-    if (work > 192 || bytes > ((size_t)64 << 20) || (reinterpret_cast<uintptr_t>(p) & 15) != 0 || bytes % 16 != 0) return 0;
+    if (work > 224 || bytes > ((size_t)64 << 20) || (reinterpret_cast<uintptr_t>(p) & 15) != 0 || bytes % 16 != 0) return 0;
     return 256 - work;
 }
 
