@@ -14,7 +14,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libcoffin_mi355.so"
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 OK, E_ARG, E_UNSUPPORTED, E_HIP = 0, 1, 2, 3
 
@@ -27,6 +27,7 @@ SIGNATURES: dict[str, list] = {
     "cmi_quant_act_i8": [_vp, _vp, _vp, _ci, _ci, _vp],
     "cmi_gemv_w8a16": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp],
     "cmi_gemv_w8a16_mfma": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp],
+    "cmi_linear_w8a16": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cmi_w4_repack": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp],
     "cmi_gemv_w4a8": [_vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp],
     "cmi_gemv_w4a16": [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _vp],
@@ -45,7 +46,8 @@ SIGNATURES: dict[str, list] = {
 
 #: Entry points that do not return a status.
 OTHER_RESTYPES = {"cmi_linear_workspace_bytes": ([_ci, _ci], _sz),
-                  "cmi_linear_w8a8_workspace_bytes": ([_ci, _ci, _ci], _sz)}
+                  "cmi_linear_w8a8_workspace_bytes": ([_ci, _ci, _ci], _sz),
+                  "cmi_stream_capture_id": ([_vp], ctypes.c_longlong)}
 
 
 class NativeError(RuntimeError):

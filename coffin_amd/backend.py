@@ -82,6 +82,50 @@ W4A16 = os.environ.get("COFFIN_AMD_W4A16", "0").strip() == "1"
 W4A16_MAX_ROWS = 4
 #: Rows from which the matrix-pipe GEMV beats the dot-product one (measured on every layer shape).
 MFMA_MIN_ROWS = 3
+#: ``rms_norm`` / ``add_rms_norm`` / ``silu_mul`` also leave their output rows quantised (int8 +
+#: scale) in private scratch, and a ``linear*`` call on that very output -- W4A8 at any row count,
+#: W8A8 prefill -- takes them from there instead of quantising the bf16 rows again: the
+#: reference's own call sequence (``ops/norm.py:87`` then ``ops/gemv.py:75``;
+#: ``models/qwen35/blocks.py:69``) then runs the projection kernels on quantised rows, as a caller
+#: of ``rms_norm_i8`` + ``linear_quantized`` would.  Same bits (the producers quantise the stored
+#: bf16 values with the quantiser's arithmetic).  ``COFFIN_AMD_HANDOVER=0`` or
+#: ``configure(handover=False)`` switches it off.
+HANDOVER = os.environ.get("COFFIN_AMD_HANDOVER", "1").strip() != "0"
+#: Largest block of rows (bytes of int8) a producer leaves behind.
+HANDOVER_MAX_BYTES = 128 << 20
+
+_FAMILIES = {"dot": 0, "mfma": 1}
+
+
+def configure(*, batch_family: str | None = None, w8a8_verify: bool | None = None,
+              w4a16: bool | None = None, handover: bool | None = None) -> dict:
+    """Process-wide switches of this backend, settable after import (the environment variables
+    above give the initial values).  Returns the settings in force.
+
+    ``batch_family``: ``"dot"`` -- ``linear`` / ``linear_m`` on int8 weights run the dot-product
+    GEMV (fastest single row; 4-16 rows are vector-ALU bound) -- or ``"mfma"`` -- every int8
+    weight-only call, single rows included, runs the matrix-pipe GEMV (4-16 rows 1.05-2.8 times
+    faster, a single row slower).  Either way row r of a batch carries the bits of the single-row
+    call (models/qwen35/batch.py:19-22): the rule needs one family per weight, not a particular
+    one.  A weight object may carry its own choice in an attribute ``batch_family`` (read when the
+    weight is first used), e.g. ``"mfma"`` for the projections of a model served in static batches.
+    """
+    global BATCH_MFMA, W8A8_VERIFY, W4A16, HANDOVER
+    if batch_family is not None:
+        if batch_family not in _FAMILIES:
+            raise ValueError(f"batch_family must be 'dot' or 'mfma', got {batch_family!r}")
+        BATCH_MFMA = batch_family == "mfma"
+    if w8a8_verify is not None:
+        W8A8_VERIFY = bool(w8a8_verify)
+    if w4a16 is not None:
+        W4A16 = bool(w4a16)
+    if handover is not None:
+        HANDOVER = bool(handover)
+        _drop_handed()
+    return {"batch_family": "mfma" if BATCH_MFMA else "dot", "w8a8_verify": W8A8_VERIFY, "w4a16": W4A16,
+            "handover": HANDOVER}
+
+
 def _vp(address: int) -> int:
     """Pointer argument: the entry points declare ``void *`` (``argtypes``), so a plain int passes."""
     return address
@@ -124,28 +168,61 @@ def _on_gpu(t: torch.Tensor) -> bool:
 
 # --------------------------------------------------------------- private state
 
-#: (rows, k, device, n) -> uint8 workspace of cmi_linear_workspace_bytes(rows, k) bytes (the
-#: quantised rows and their scales of one projection); single-threaded caller by contract
-#: (backends/corex/__init__.py:654-690 keeps the same kind of pool).
-_SCRATCH: OrderedDict = OrderedDict()
-_SCRATCH_MAX = 32
+class _Arena:
+    """One grow-only block of device memory per (purpose, device) that is never handed back.
+
+    A captured HIP graph holds raw addresses of whatever scratch its kernels were launched with
+    (quantised rows, split-K arrival counters and partial tiles), so scratch that a later call
+    could free -- a pool that evicts by shape, say -- would be rewritten under a replay once the
+    allocator reuses it.  Here a request larger than the block allocates a new block of at least
+    twice the size and *retires* the old one: it stays allocated until the process ends, so every
+    address ever handed out stays valid, and the memory held is at most twice the largest request.
+    Calls are serialised on one stream by contract (backends/corex/__init__.py:656-658), so one
+    block serves every shape: a projection's scratch is dead when the next projection starts.
+    Growth allocates, which a stream capture must not do: the warm-up step that precedes a capture
+    (engine/llm_engine.py:116) sizes the block, and growth under capture raises."""
+
+    _ROUND = 1 << 20
+
+    def __init__(self, purpose: str) -> None:
+        self.purpose = purpose
+        self.blocks: dict = {}      # device index -> uint8 tensor
+        self.retired: list = []     # outgrown blocks, kept alive for graphs that captured them
+
+    def take(self, nbytes: int, device: torch.device) -> int:
+        """Address of at least ``nbytes`` bytes (256-byte aligned) on ``device``."""
+        block = self.blocks.get(device.index)
+        if block is None or block.numel() < nbytes:
+            if device.type == "cuda" and torch.cuda.is_current_stream_capturing():
+                raise RuntimeError(f"coffin_amd: {self.purpose} scratch must grow to {nbytes} bytes inside a "
+                                   "graph capture; run one eager step over the same shapes before capturing")
+            size = max(nbytes, 2 * block.numel() if block is not None else 0)
+            size = (size + self._ROUND - 1) // self._ROUND * self._ROUND
+            if block is not None:
+                self.retired.append(block)
+            block = torch.empty(size, dtype=torch.uint8, device=device)
+            self.blocks[device.index] = block
+        return block.data_ptr()
 
 
-def _scratch(rows: int, k: int, device: torch.device, n: int = 0) -> torch.Tensor:
-    """Workspace of the fused quantiser + projection entries; with ``n`` (int8 weights) sized so
+#: Workspace of the fused quantiser + projection entries (quantised rows, scales, split-K room).
+_WORKSPACE = _Arena("projection")
+#: (rows, n, k) -> bytes the library asks for; a few integers per distinct shape.
+_WORKSPACE_BYTES: dict = {}
+
+
+def _scratch(rows: int, k: int, device: torch.device, n: int = 0):
+    """``(address, bytes)`` of the workspace for one projection; with ``n`` (int8 weights) sized so
     that the W8A8 entry may split K where that pays."""
-    key = (rows, k, device, n)
-    hit = _SCRATCH.get(key)
-    if hit is None:
-        while len(_SCRATCH) >= _SCRATCH_MAX:
-            _SCRATCH.popitem(last=False)          # least recently used shape goes first
+    key = (rows, n, k)
+    nbytes = _WORKSPACE_BYTES.get(key)
+    if nbytes is None:
         lib = _native.load()
         nbytes = int(lib.cmi_linear_w8a8_workspace_bytes(rows, n, k) if n else lib.cmi_linear_workspace_bytes(rows, k))
-        hit = torch.empty(nbytes, dtype=torch.uint8, device=device)
-        _SCRATCH[key] = hit
-    else:
-        _SCRATCH.move_to_end(key)
-    return hit
+        if len(_WORKSPACE_BYTES) >= 65536:
+            _WORKSPACE_BYTES.clear()
+        _WORKSPACE_BYTES[key] = nbytes
+    return _WORKSPACE.take(nbytes, device), nbytes
 
 
 #: id(source tensor) -> device-layout copy, dropped when the source dies
@@ -231,6 +308,85 @@ def _w4_operands(w):
     return _memo(w.packed, make)
 
 
+# ------------------------------------------------- quantised rows handed forward
+
+class _Handed:
+    """The latest producer output and where its quantised rows are.  ``tensor`` is a strong
+    reference on purpose: while it lives no other allocation can have its address, so an
+    activation with the same address, layout and version counter *is* this tensor's memory."""
+
+    __slots__ = ("tensor", "version", "ptr", "rows", "k", "ld", "dev", "xq", "xs", "capture")
+
+
+_HANDED: _Handed | None = None
+_HANDOVER_ARENA = _Arena("quantised-row hand-over")
+#: Producers start leaving quantised rows behind once a projection has quantised activations in
+#: this process (a model of plain or weight-only int8 decode never pays for rows nobody reads).
+_QUANT_CONSUMER_SEEN = False
+
+
+def _round256(v: int) -> int:
+    return (v + 255) // 256 * 256
+
+
+def _drop_handed() -> None:
+    global _HANDED
+    _HANDED = None
+
+
+def _drop_handed_if_written(*written) -> None:
+    """Forget the handed rows when one of this backend's own ops writes into their tensor (torch
+    ops announce their writes through the version counter; these kernels do not)."""
+    h = _HANDED
+    if h is None:
+        return
+    home = h.tensor.untyped_storage().data_ptr()
+    for t in written:
+        if t is not None and t.device == h.dev and t.untyped_storage().data_ptr() == home:
+            _drop_handed()
+            return
+
+
+def _capture_id(stream: int) -> int:
+    return int(_native.load().cmi_stream_capture_id(stream))
+
+
+def _hand_target(rows: int, k: int, device: torch.device):
+    """``(xq address, xs address)`` for a producer of ``rows x k`` outputs, or ``None`` when it
+    should not leave quantised rows behind."""
+    if not (HANDOVER and _QUANT_CONSUMER_SEEN) or rows <= 0 or rows * k > HANDOVER_MAX_BYTES:
+        return None
+    try:
+        base = _HANDOVER_ARENA.take(_round256(rows * k) + _round256(4 * rows), device)
+    except RuntimeError:
+        return None                      # would have to grow inside a capture: this call goes without
+    return base, base + _round256(rows * k)
+
+
+def _hand_over(t: torch.Tensor, rows: int, k: int, ld: int, target, stream: int) -> None:
+    global _HANDED
+    h = _Handed()
+    h.tensor, h.version, h.ptr, h.rows, h.k, h.ld, h.dev = t, t._version, t.data_ptr(), rows, k, ld, t.device
+    h.xq, h.xs = target
+    # a graph must not read rows that a kernel outside it wrote (nor the other way round): the
+    # consumer has to be recorded into the same capture as the producer, or both run eagerly
+    h.capture = _capture_id(stream)
+    _HANDED = h
+
+
+def _handed_rows(x: torch.Tensor, rows: int, k: int, stream: int):
+    """The quantised copy of ``x`` left by the producer that wrote it, or ``None``."""
+    h = _HANDED
+    if h is None or x.data_ptr() != h.ptr or rows != h.rows or k != h.k or x._version != h.version \
+            or x.device != h.dev:
+        return None
+    if x.stride(-1) != 1 or (x.dim() == 2 and rows > 1 and x.stride(0) != h.ld):
+        return None
+    if _capture_id(stream) != h.capture:
+        return None
+    return h.xq, h.xs
+
+
 # ------------------------------------------------------------------- kernels
 
 def _quantize_rows(act: torch.Tensor, xq: torch.Tensor, xs: torch.Tensor, rows: int, k: int) -> None:
@@ -243,7 +399,7 @@ class _Record:
     """What the adapters need of one quantized weight, resolved once: operand addresses in
     device layout, shape, device.  Holds no strong reference to the caller's tensors."""
 
-    __slots__ = ("kind", "src", "src2", "a", "b", "n", "k", "gs", "dev")
+    __slots__ = ("kind", "src", "src2", "a", "b", "n", "k", "gs", "dev", "family")
 
 
 #: id(weight object) -> _Record; an entry is trusted only while the tensors it was
@@ -284,6 +440,10 @@ def _make_record(w) -> _Record:
         wq, scale = _q8_operands(w)
         rec.kind, rec.src, rec.a, rec.b = 8, weakref.ref(w.wq), wq.data_ptr(), scale.data_ptr()
         rec.n, rec.k, rec.gs, rec.dev = int(wq.shape[0]), int(wq.shape[1]), 0, w.wq.device
+    family = getattr(w, "batch_family", None)
+    if family is not None and family not in _FAMILIES:
+        raise ValueError(f"batch_family of a weight must be 'dot' or 'mfma', got {family!r}")
+    rec.family = family
     rec.src2 = weakref.ref(w.scale)
     _RECORDS.pop(id(w), None)                     # a stale entry under a reused id
     while len(_RECORDS) >= _RECORDS_MAX:
@@ -293,29 +453,25 @@ def _make_record(w) -> _Record:
 
 
 def _gemv_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor, mfma: bool = False) -> None:
+    """Weight-only projection, one native call for any number of rows.  ``mfma``: the call site may
+    use the matrix-pipe family (verify, short prefill chunks: from ``MFMA_MIN_ROWS`` rows); a weight
+    or a process whose family is "mfma" uses it for every call, single rows included."""
     n, k = rec.n, rec.k
-    lib = _native.load()
-    exact = lib.cmi_gemv_w8a16
-    fast = (lib.cmi_gemv_w8a16_mfma
-            if mfma and (BATCH_MFMA or rows >= MFMA_MIN_ROWS) and k % 128 == 0 and k <= 10240 else None)
-    stream = _stream()
-    x0, y0 = act.data_ptr(), out.data_ptr()
-    step = GEMV_MFMA_MAX_ROWS if fast is not None else GEMV_MAX_ROWS
-    for lo in range(0, rows, step):
-        m = min(step, rows - lo)
-        # every chunk of a fast call takes the fast kernel, also a short last one: a row's bits
-        # must not depend on where the batch happened to be cut
-        fn = fast if fast is not None else exact
-        rc = fn(rec.a, rec.b, x0 + lo * k * 2, y0 + lo * n * 2, m, n, k, stream)
-        if rc:
-            _native.check(rc, "gemv_w8a16")
+    whole = rec.family == "mfma" if rec.family is not None else BATCH_MFMA
+    fast = (whole or (mfma and rows >= MFMA_MIN_ROWS)) and k % 128 == 0 and k <= 10240
+    rc = _native.load().cmi_linear_w8a16(rec.a, rec.b, act.data_ptr(), out.data_ptr(), rows, n, k,
+                                         1 if fast else 0, _stream())
+    if rc:
+        _native.check(rc, "linear_w8a16")
 
 
 def _gemm_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> None:
+    global _QUANT_CONSUMER_SEEN
+    _QUANT_CONSUMER_SEEN = True
     n, k = rec.n, rec.k
-    work = _scratch(rows, k, act.device, n)
+    work, nbytes = _scratch(rows, k, act.device, n)
     rc = _native.load().cmi_linear_w8a8_bf16(act.data_ptr(), rec.a, rec.b, out.data_ptr(), rows, n, k, n,
-                                             work.data_ptr(), work.numel(), _stream())
+                                             work, nbytes, _stream())
     if rc:
         _native.check(rc, "linear_w8a8_bf16")
 
@@ -323,12 +479,32 @@ def _gemm_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> N
 def _rows_w4(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> None:
     """Quantiser + W4A8 GEMV or GEMM in one native call; the library picks the route (one launch
     with the quantiser folded into the GEMV for one or two rows, else two launches)."""
+    global _QUANT_CONSUMER_SEEN
+    _QUANT_CONSUMER_SEEN = True
     n, k = rec.n, rec.k
-    work = _scratch(rows, k, act.device)
+    work, nbytes = _scratch(rows, k, act.device)
     rc = _native.load().cmi_linear_w4a8_bf16(rec.a, rec.b, act.data_ptr(), out.data_ptr(), rows, n, k, rec.gs,
-                                             work.data_ptr(), work.numel(), _stream())
+                                             work, nbytes, _stream())
     if rc:
         _native.check(rc, "linear_w4a8_bf16")
+
+
+def _rows_quantised(rec: _Record, xq: int, xs: int, rows: int, out: torch.Tensor, stream: int) -> None:
+    """Projection of rows that are already int8 + scale (addresses): W4A8 GEMV / GEMM or the W8A8 GEMM."""
+    lib = _native.load()
+    if rec.kind == 4:
+        fn = lib.cmi_gemv_w4a8 if rows <= 16 else lib.cmi_gemm_w4a8
+        rc = fn(rec.a, rec.b, xq, xs, out.data_ptr(), None, rows, rec.n, rec.k, rec.gs, stream)
+    else:
+        rc = lib.cmi_gemm_w8a8(xq, rec.a, xs, rec.b, out.data_ptr(), None, rows, rec.n, rec.k, rec.n, stream)
+    if rc:
+        _native.check(rc, "projection of quantised rows")
+
+
+def _splits_k(rows: int, n: int, k: int, device: torch.device) -> bool:
+    """Whether the W8A8 entry would be given room to split K for this shape (it then needs the
+    quantiser's launch in front of it, which clears the arrival counters)."""
+    return _scratch(rows, k, device, n)[1] != _scratch(rows, k, device)[1]
 
 
 def _rows_w4a16(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> None:
@@ -387,12 +563,21 @@ def _project(w, x: torch.Tensor, prefill: bool, min_rows: int = PREFILL_MIN_ROWS
             return _project(w, x, prefill, min_rows, mfma)
     if rec is None:
         rec = _make_record(w)
-    act = x if x.is_contiguous() else x.contiguous()
     rows = 1 if nd == 1 else x.shape[0]
     # a [K] activation is one row answered as [N]: no view juggling on the decode path
     out = torch.empty((rec.n,) if nd == 1 else (rows, rec.n), dtype=torch.bfloat16, device=dev)
     if rows == 0:
         return out
+    quantising = (rec.kind == 4 and not (W4A16 and rows <= W4A16_MAX_ROWS and rec.k <= 10240)) or \
+                 (rec.kind == 8 and prefill and rows >= min_rows)
+    if quantising and _HANDED is not None:
+        # the rows a producer of this backend left behind for exactly this tensor
+        stream = _stream()
+        handed = _handed_rows(x, rows, rec.k, stream)
+        if handed is not None and (rec.kind == 4 or not _splits_k(rows, rec.n, rec.k, dev)):
+            _rows_quantised(rec, handed[0], handed[1], rows, out, stream)
+            return out
+    act = x if x.is_contiguous() else x.contiguous()
     if rec.kind == 4:
         if W4A16 and rows <= W4A16_MAX_ROWS and rec.k <= 10240:
             _rows_w4a16(rec, act, rows, out)
@@ -407,13 +592,13 @@ def _project(w, x: torch.Tensor, prefill: bool, min_rows: int = PREFILL_MIN_ROWS
 
 def linear(w, x: torch.Tensor) -> torch.Tensor:
     """``linear(w, x) -> y``: ``x`` ``[K]`` or ``[C, K]``, ``y`` ``[N]`` or ``[C, N]``, dtype of ``x``."""
-    return _project(w, x, prefill=False, mfma=BATCH_MFMA)
+    return _project(w, x, prefill=False)
 
 
 def linear_m(w, x: torch.Tensor) -> torch.Tensor:
     """``linear_m(w, x[M, K]) -> [M, N]``: one weight read serves all rows; row r carries the bits
-    of ``linear(w, x[r])`` (in either setting of ``BATCH_MFMA``: both entries switch together)."""
-    return _project(w, x, prefill=False, mfma=BATCH_MFMA)
+    of ``linear(w, x[r])`` (in either kernel family: both entries switch together, see :func:`configure`)."""
+    return _project(w, x, prefill=False)
 
 
 def linear_m_verify(w, x: torch.Tensor) -> torch.Tensor:
@@ -474,15 +659,7 @@ def linear_quantized(w, xq: torch.Tensor, xs: torch.Tensor) -> torch.Tensor:
     out = torch.empty((rows, rec.n), dtype=torch.bfloat16, device=xq.device)
     if rows == 0:
         return out
-    lib = _native.load()
-    if rec.kind == 4:
-        fn = lib.cmi_gemv_w4a8 if rows <= 16 else lib.cmi_gemm_w4a8
-        rc = fn(rec.a, rec.b, xq.data_ptr(), xs.data_ptr(), out.data_ptr(), None, rows, rec.n, k, rec.gs, _stream())
-    else:
-        rc = lib.cmi_gemm_w8a8(xq.data_ptr(), rec.a, xs.data_ptr(), rec.b, out.data_ptr(), None, rows, rec.n, k,
-                               rec.n, _stream())
-    if rc:
-        _native.check(rc, "linear_quantized")
+    _rows_quantised(rec, xq.data_ptr(), xs.data_ptr(), rows, out, _stream())
     return out
 
 
@@ -505,23 +682,32 @@ def kv_quant(x: torch.Tensor, out_q: torch.Tensor, out_s: torch.Tensor) -> torch
         out_s.copy_(s.reshape(out_s.shape))
         out_q.copy_(torch.round(xf / s.unsqueeze(-1)).clamp_(-127, 127).to(torch.int8))
         return out_q
+    _drop_handed_if_written(out_q, out_s)
     with torch.cuda.device(x.device):
         _quantize_rows(x, out_q, out_s, x.shape[0], x.shape[1])
     return out_q
 
 
-def _rows_view(t: torch.Tensor, what: str):
-    """``(rows, width, row pitch)`` of a 1-D row or a 2-D block whose innermost stride is 1."""
+def _rows_view(t: torch.Tensor):
+    """``(rows, width, row pitch)`` of ``[K]``, ``[rows, K]`` or ``[..., K]`` whose rows are
+    ``K`` contiguous elements at one pitch; ``None`` for any other layout."""
     if t.dim() == 1:
-        return 1, t.shape[0], t.shape[0]
+        return (1, t.shape[0], t.shape[0]) if t.stride(0) == 1 or t.shape[0] <= 1 else None
+    if t.dim() > 2:
+        try:
+            t = t.view(-1, t.shape[-1])          # leading axes that collapse without a copy
+        except RuntimeError:
+            return None
     if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
-        raise ValueError(f"{what} must be [K] or [rows, K] with a unit innermost stride, "
-                         f"got shape {tuple(t.shape)} strides {t.stride()}")
+        return None
     return t.shape[0], t.shape[1], (t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1]))
 
 
-def _silu_mul_native(gate, up, out, out_q, out_s) -> bool:
-    """Run the fused kernel when every tensor is one it takes; False leaves the call to torch."""
+def _silu_mul_native(gate, up, out, out_q, out_s, hand: bool = False) -> bool:
+    """Run the fused kernel when every tensor is one it takes; False leaves the call to torch
+    (other dtypes or devices, rows that are not ``K`` contiguous elements at one pitch).  ``hand``:
+    with no ``out_q`` of the caller's, leave the quantised rows behind for the projection that
+    follows (see ``HANDOVER``)."""
     tensors = [t for t in (gate, up, out, out_q, out_s) if t is not None]
     if not all(_on_gpu(t) and t.device == gate.device for t in tensors):
         return False
@@ -530,24 +716,36 @@ def _silu_mul_native(gate, up, out, out_q, out_s) -> bool:
     if out_q is not None and not (out_q.dtype == torch.int8 and out_q.is_contiguous()
                                   and out_s.dtype == torch.float32 and out_s.is_contiguous()):
         return False
-    rows, k, ldg = _rows_view(gate, "gate")
-    _, _, ldu = _rows_view(up, "up")
-    _, _, ldo = _rows_view(out, "out")
+    views = [_rows_view(t) for t in (gate, up, out)]
+    if any(v is None for v in views):
+        return False
+    (rows, k, ldg), (_, _, ldu), (_, _, ldo) = views
+    if rows == 0 or k == 0:
+        return True
+    q_ptr, s_ptr = _ptr(out_q), _ptr(out_s)
     with torch.cuda.device(gate.device):
-        rc = _native.load().cmi_silu_mul_quant(gate.data_ptr(), up.data_ptr(), out.data_ptr(), _ptr(out_q),
-                                               _ptr(out_s), rows, k, ldg, ldu, ldo, _stream())
-    if rc:
-        _native.check(rc, "silu_mul_quant")
+        stream = _stream()
+        target = _hand_target(rows, k, gate.device) if hand and out_q is None and out.dim() <= 2 else None
+        if target is not None:
+            q_ptr, s_ptr = target
+        rc = _native.load().cmi_silu_mul_quant(gate.data_ptr(), up.data_ptr(), out.data_ptr(), q_ptr, s_ptr,
+                                               rows, k, ldg, ldu, ldo, stream)
+        if rc:
+            _native.check(rc, "silu_mul_quant")
+        if target is not None:
+            _hand_over(out, rows, k, ldo, target, stream)
     return True
 
 
 def silu_mul(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     """``silu_mul(gate, up, out) -> out``: ``out = silu(gate) * up`` into a caller-owned buffer
     that may alias ``up`` (backends/protocol.py:265-273, backends/reference/__init__.py:253-268).
-    Registered together with :func:`silu_mul_quant` so that the two share one arithmetic."""
+    Registered together with :func:`silu_mul_quant` so that the two share one arithmetic.  Any
+    leading shape (``[...]`` in the contract): layouts the kernel does not take go to torch."""
     if gate.shape != up.shape or out.shape != gate.shape:
         raise ValueError("silu_mul needs gate, up and out of one shape")
-    if not _silu_mul_native(gate, up, out, None, None):
+    _drop_handed()
+    if not _silu_mul_native(gate, up, out, None, None, hand=True):
         out.copy_(F.silu(gate) * up)
     return out
 
@@ -563,6 +761,7 @@ def silu_mul_quant(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor, out_
     if tuple(out.shape) != tuple(gate.shape) or tuple(out_q.shape) != tuple(gate.shape) \
             or out_s.numel() != gate.shape[0]:
         raise ValueError("silu_mul_quant expects out [rows, K], out_q [rows, K], out_s [rows]")
+    _drop_handed()
     if not _silu_mul_native(gate, up, out, out_q, out_s):
         out.copy_(F.silu(gate) * up)
         kv_quant(out if out.is_contiguous() else out.contiguous(), out_q, out_s)
@@ -591,6 +790,7 @@ def rms_norm_i8(x: torch.Tensor, w: torch.Tensor, out_q: torch.Tensor, out_s: to
         raise ValueError("rms_norm_i8: out_q must be contiguous int8 and out_s contiguous fp32 on x's device")
     ldx = x.stride(0) if m > 1 else max(x.stride(0), n)
     lib = _native.load()
+    _drop_handed()
     y_ptr, ldy = 0, n
     if out is not None:
         if tuple(out.shape) != (m, n) or out.dtype != torch.bfloat16 or out.stride(1) != 1 or out.device != x.device:
@@ -634,14 +834,20 @@ def rms_norm(x: torch.Tensor, w: torch.Tensor, stride: int = 0, eps: float = 1e-
         return (xf * scale).to(x.dtype) * w.to(x.dtype)
     m, n = x.shape
     y = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
+    _drop_handed()
     if m == 0:
         return y
     gain = _gain_bf16(w)
     with torch.cuda.device(x.device):
-        rc = _native.load().cmi_rms_norm_i8(x.data_ptr(), gain.data_ptr(), y.data_ptr(), 0, 0, m, n,
-                                            x.stride(0) if m > 1 else max(x.stride(0), n), n, float(eps), _stream())
-    if rc:
-        _native.check(rc, "rms_norm")
+        stream = _stream()
+        target = _hand_target(m, n, x.device)
+        q_ptr, s_ptr = target if target is not None else (0, 0)
+        rc = _native.load().cmi_rms_norm_i8(x.data_ptr(), gain.data_ptr(), y.data_ptr(), q_ptr, s_ptr, m, n,
+                                            x.stride(0) if m > 1 else max(x.stride(0), n), n, float(eps), stream)
+        if rc:
+            _native.check(rc, "rms_norm")
+        if target is not None:
+            _hand_over(y, m, n, n, target, stream)
     return y
 
 
@@ -658,15 +864,21 @@ def add_rms_norm(x: torch.Tensor, add: torch.Tensor, w: torch.Tensor, out: torch
         out.copy_(rms_norm(x, w, 0, eps))
         return out
     m, n = x.shape
+    _drop_handed()
     if m == 0:
         return out
     gain = _gain_bf16(w)
     pitch = lambda t: t.stride(0) if m > 1 else max(t.stride(0), n)
     with torch.cuda.device(x.device):
-        rc = _native.load().cmi_add_rms_norm_i8(x.data_ptr(), add.data_ptr(), gain.data_ptr(), out.data_ptr(), 0, 0, m, n,
-                                                pitch(x), pitch(add), pitch(out), float(eps), _stream())
-    if rc:
-        _native.check(rc, "add_rms_norm")
+        stream = _stream()
+        target = _hand_target(m, n, x.device)
+        q_ptr, s_ptr = target if target is not None else (0, 0)
+        rc = _native.load().cmi_add_rms_norm_i8(x.data_ptr(), add.data_ptr(), gain.data_ptr(), out.data_ptr(), q_ptr,
+                                                s_ptr, m, n, pitch(x), pitch(add), pitch(out), float(eps), stream)
+        if rc:
+            _native.check(rc, "add_rms_norm")
+        if target is not None:
+            _hand_over(out, m, n, pitch(out), target, stream)
     return out
 
 

@@ -53,7 +53,7 @@ int gemv_w4a8_decode(const uint8_t *w4, const float *ws, const void *x, const in
                      void *y, int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,
                      void *stream);
 // gemv_w4a8_chain.hip: the same for 1..2 rows with the fp32 chain in registers; `variant` = lanes per
-// weight row (8, 16) + 100 * wavefronts sharing a row (1, 2, 4) + 10000 * wavefronts per workgroup
+// weight row (8, 16) + 100 * wavefronts sharing a row (1, 2, 4, 8) + 10000 * wavefronts per workgroup
 // (4, 8, 16); CMI_E_UNSUPPORTED (no error text) outside the variant's range.
 int gemv_w4a8_chain(const uint8_t *w4, const float *ws, const void *x, const int8_t *xq, const float *xs,
                     void *y, int32_t *group_acc, int8_t *xq_out, float *xs_out, int M, int N, int K,

@@ -22,7 +22,7 @@ using namespace cmi;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int GS = 128;  // group size the kernels are built for
+constexpr int GS = 128;  // group size the fast kernels are built for; the general kernel below also takes 64 and 256
 constexpr int FUSED_MAX_ROWS = 4;  // activation rows the fused-quantiser variant takes
 
 struct W4Args {
@@ -36,7 +36,7 @@ struct W4Args {
     uint16_t *y;
     int32_t *group_acc;
     int M, N, K;
-    int G;        // K / 128
+    int G;        // K / group size
     int nchunks;  // K / 32: 16-byte chunks per row
     int KW, teams, iters;
 };
@@ -46,10 +46,14 @@ struct W4Args {
 // 16-byte vectors per thread and row -- with the arithmetic of the stand-alone
 // quantiser; the bf16 loads are issued before anything else and the weight
 // stream hides the work.  Saves a launch and the int8 round trip through memory.
-template <int M, int R2, int CH, int XV>
+// LG: log2(group size / 32) -- 1, 2, 3 for groups of 64, 128, 256: a lane's 16-byte load is 32 k,
+// so 2, 4 or 8 adjacent lanes own a group and their partial sums meet in one, two or three DPP steps.
+template <int M, int R2, int CH, int XV, int LG = 2>
 __global__ void __launch_bounds__(256)
 gemv_w4a8_kernel(const W4Args a) {
     constexpr int ROWS = 2 * R2;
+    constexpr int GPH = 32 >> LG;  // groups per half-wavefront load (32 chunks of 32 k)
+    static_assert(LG >= 1 && LG <= 3 && (LG == 2 || XV == 0), "group sizes 64, 128, 256; the fused quantiser only with 128");
     extern __shared__ int32_t sums_base[];  // [fused: M*K int8, M scales, M*4 partial maxima] [teams][groups][ROWS*M]
     int8_t *xq_lds = reinterpret_cast<int8_t *>(sums_base);
     float *xs_lds = reinterpret_cast<float *>(xq_lds + (XV ? (size_t)M * a.K : 0));
@@ -104,7 +108,7 @@ gemv_w4a8_kernel(const W4Args a) {
     const int team = wave / a.KW;
     const int kw = wave - team * a.KW;
     const int n0 = (blockIdx.x * a.teams + team) * ROWS;
-    int32_t *team_sums = sums + (size_t)team * (a.iters * a.KW * CH * 8) * (ROWS * M);
+    int32_t *team_sums = sums + (size_t)team * (a.iters * a.KW * CH * GPH) * (ROWS * M);
     const int row_bytes = a.K / 2;
 
     const u32x4 *wrow[R2];
@@ -170,7 +174,7 @@ gemv_w4a8_kernel(const W4Args a) {
                     op[2 * i] = w[i] & 0x0F0F0F0Fu;
                     op[2 * i + 1] = (w[i] >> 4) & 0x0F0F0F0Fu;
                 }
-                const int group = chunk[j] >> 2;
+                const int group = chunk[j] >> LG;
 #pragma unroll
                 for (int m = 0; m < M; ++m) {
                     const uint32_t xv[8] = {xr[m][j][0].x, xr[m][j][0].y, xr[m][j][0].z,
@@ -180,9 +184,10 @@ gemv_w4a8_kernel(const W4Args a) {
 #pragma unroll
                     for (int i = 0; i < 8; ++i)
                         acc = __builtin_amdgcn_sdot4((int)op[i], (int)xv[i], acc, false);
-                    acc += dpp_i32<0xB1, 0xf>(acc);  // quad_perm [1,0,3,2]
-                    acc += dpp_i32<0x4E, 0xf>(acc);  // quad_perm [2,3,0,1]
-                    if ((hl & 3) == 0 && live[j])
+                    acc += dpp_i32<0xB1, 0xf>(acc);                           // quad_perm [1,0,3,2]
+                    if constexpr (LG >= 2) acc += dpp_i32<0x4E, 0xf>(acc);    // quad_perm [2,3,0,1]
+                    if constexpr (LG >= 3) acc += dpp_i32<0x141, 0xf>(acc);   // row_half_mirror: the other quad of 8 lanes
+                    if ((hl & ((1 << LG) - 1)) == 0 && live[j])
                         team_sums[group * (ROWS * M) + (2 * rr + half) * M + m] = acc;
                 }
             }
@@ -210,10 +215,14 @@ struct Plan {
     int mt, r2, ch, kw, teams, iters;
 };
 
-Plan make_plan(int M, int N, int K) {
+// lg: log2(group size / 32).  Group sizes other than 128 are served by fewer instantiations (one
+// row pair per wavefront, at most two chunks per trip).
+Plan make_plan(int M, int N, int K, int lg) {
     Plan p;
     p.mt = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
-    const int chmax = p.mt <= 4 ? 4 : p.mt <= 8 ? 2 : 1;
+    const int gph = 32 >> lg;
+    int chmax = p.mt <= 4 ? 4 : p.mt <= 8 ? 2 : 1;
+    if (lg != 2 && chmax > 2) chmax = 2;
     const int nhseg = (K / 32 + 31) / 32;
     // Up to a quarter of padding is accepted for fewer trips (more loads in
     // flight); then least padding, then fewest wavefronts per team.
@@ -237,27 +246,35 @@ Plan make_plan(int M, int N, int K) {
     const long target_waves = 256L * 8;
     while (r2 > 1 && (long)((N + 2 * r2 - 1) / (2 * r2)) * p.kw < target_waves) r2 >>= 1;
     while (2 * r2 * p.mt > 64) r2 >>= 1;
-    p.r2 = r2 < 1 ? 1 : r2;
+    p.r2 = r2 < 1 || lg != 2 ? 1 : r2;
     // Group sums of a whole team live in LDS; shrink the team count, then the
     // row block, until they fit comfortably.
     auto lds_bytes = [&]() {
-        return (size_t)4 * p.teams * (p.iters * p.kw * p.ch * 8) * (2 * p.r2 * p.mt);
+        return (size_t)4 * p.teams * (p.iters * p.kw * p.ch * gph) * (2 * p.r2 * p.mt);
     };
     while (lds_bytes() > 48 * 1024 && p.teams > 1) p.teams >>= 1;
     while (lds_bytes() > 48 * 1024 && p.r2 > 1) p.r2 >>= 1;
     return p;
 }
 
-template <int M, int R2, int CH, int XV>
+template <int M, int R2, int CH, int XV, int LG = 2>
 int launch_xv(const W4Args &a, hipStream_t st) {
     const int rows_per_block = 2 * R2 * a.teams;
     const dim3 grid((a.N + rows_per_block - 1) / rows_per_block);
-    const size_t lds = sizeof(int32_t) * a.teams * (a.iters * a.KW * CH * 8) * (2 * R2 * M) +
+    const size_t lds = sizeof(int32_t) * a.teams * (a.iters * a.KW * CH * (32 >> LG)) * (2 * R2 * M) +
                        (XV ? (size_t)M * a.K + sizeof(float) * M * 5 : 0);
     if (lds > 64 * 1024)
         return fail(CMI_E_UNSUPPORTED, "cmi_gemv_w4a8: K=%d needs %zu bytes of LDS", a.K, lds);
-    gemv_w4a8_kernel<M, R2, CH, XV><<<grid, dim3(64 * a.KW * a.teams), lds, st>>>(a);
+    gemv_w4a8_kernel<M, R2, CH, XV, LG><<<grid, dim3(64 * a.KW * a.teams), lds, st>>>(a);
     return check_launch("cmi_gemv_w4a8");
+}
+
+// Groups of 64 or 256: quantised activations only, one row pair per wavefront, one or two chunks per trip.
+template <int M>
+int launch_other_group(const W4Args &a, int ch, int lg, hipStream_t st) {
+    if (lg == 1) return ch == 1 ? launch_xv<M, 1, 1, 0, 1>(a, st) : launch_xv<M, 1, 2, 0, 1>(a, st);
+    if constexpr (M <= 8) return ch == 1 ? launch_xv<M, 1, 1, 0, 3>(a, st) : launch_xv<M, 1, 2, 0, 3>(a, st);
+    else return launch_xv<M, 1, 1, 0, 3>(a, st);
 }
 
 template <int M, int R2, int CH>

@@ -129,6 +129,6 @@ extern "C" int cmi_set_option(const char *name, int value) {
     return fail(CMI_E_ARG, "cmi_set_option: unknown option '%s'", name);
 }
 
-extern "C" int cmi_abi_version(void) { return 2; }
+extern "C" int cmi_abi_version(void) { return 3; }
 
 extern "C" const char *cmi_last_error(void) { return g_error; }

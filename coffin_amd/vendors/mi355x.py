@@ -47,6 +47,15 @@ def build_ops() -> "Ops":
         return Ops()
 
 
+def configure(**settings) -> dict:
+    """Process-wide switches of the native entries, e.g. ``configure(batch_family="mfma")`` for a
+    deployment that decodes static batches (see ``coffin_amd.backend.configure``).  The contract's
+    ``VendorSpec`` has no field for backend options, so the door is this module-level function of
+    the vendor file; environment variables (``COFFIN_AMD_BATCH_MFMA`` ...) give the initial values."""
+    from coffin_amd import backend
+    return backend.configure(**settings)
+
+
 SPEC = VendorSpec(
     name="mi355x",
     detection=Detection(

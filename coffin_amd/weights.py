@@ -24,12 +24,16 @@ _CHUNK_ROWS = 16384
 class QWeight:
     """int8 ``[N, K]`` weight with one fp32 absmax scale per output row."""
 
-    __slots__ = ("wq", "scale", "n", "k")
+    __slots__ = ("wq", "scale", "n", "k", "batch_family")
 
-    def __init__(self, wq: torch.Tensor, scale: torch.Tensor) -> None:
+    def __init__(self, wq: torch.Tensor, scale: torch.Tensor, batch_family: str | None = None) -> None:
         self.wq = wq
         self.scale = scale
         self.n, self.k = (int(d) for d in wq.shape)
+        #: ``None`` (the process-wide setting), ``"dot"`` or ``"mfma"``: the kernel family every
+        #: weight-only call on this weight uses (``coffin_amd.backend.configure``); read by the
+        #: adapter when the weight is first used.  Not an attribute of the reference's class.
+        self.batch_family = batch_family
 
     @classmethod
     def quantize(cls, w: torch.Tensor, chunk_rows: int = _CHUNK_ROWS) -> "QWeight":

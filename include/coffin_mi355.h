@@ -46,8 +46,10 @@ int cmi_abi_version(void);
  *                   decode GEMV (one bf16 or quantised row);
  *   "w4_decode_chain" 0 (the library chooses) | 1 (never) | lanes + 100 * split + 10000 * waves: the
  *                   W4A8 decode kernel that keeps the fp32 chain in registers, with `lanes` (8, 16)
- *                   lanes per weight row, `split` (1, 2, 4) wavefronts sharing a row and `waves`
- *                   (4, 8, 16) wavefronts per workgroup, wherever the shape fits that arrangement.
+ *                   lanes per weight row, `split` (1, 2, 4, 8) wavefronts sharing a row and `waves`
+ *                   (4, 8, 16) wavefronts per workgroup, wherever the shape fits that arrangement
+ *                   (a combination that is not built, or a shape it does not fit, leaves the
+ *                   choice to the library).
  * The environment variables CMI_GEMM_TILE and CMI_GEMV_WHOLEROW give the initial values; they are
  * read once, at the first call that needs them.  Unknown names or values: CMI_E_ARG.  Every choice
  * gives the same bits. */
@@ -89,6 +91,27 @@ int cmi_gemv_w8a16(const int8_t *wq, const float *ws, const void *x, void *y,
  * (backends/corex/__init__.py:495-546). */
 int cmi_gemv_w8a16_mfma(const int8_t *wq, const float *ws, const void *x, void *y,
                         int M, int N, int K, void *stream);
+
+/* int8 weight-only projection of any number of rows, with the kernel family named by the caller:
+ *   CMI_FAMILY_DOT   cmi_gemv_w8a16, 16 rows per launch: row m carries the bits of the single-row call
+ *                    (what static-batch decode owes its users, models/qwen35/batch.py:19-22);
+ *   CMI_FAMILY_MFMA  cmi_gemv_w8a16_mfma, 64 rows per launch (K % 128 == 0, K <= 10240, else
+ *                    CMI_E_UNSUPPORTED and nothing is launched): 1.5-2.8 times faster at 4-16 rows,
+ *                    slower at one row; a row's bits depend on K only.
+ * The rule holds inside either family as long as every call on a weight -- single rows included --
+ * names the same one, so the family is a property of a weight (or of a deployment), not of a call
+ * site.  Stands where linear / linear_m / linear_m_verify reach gemv_nk_i8 / gemv_nk_i8_m
+ * (backends/corex/__init__.py:396-425,495-546). */
+#define CMI_FAMILY_DOT 0
+#define CMI_FAMILY_MFMA 1
+int cmi_linear_w8a16(const int8_t *wq, const float *ws, const void *x, void *y, int M, int N, int K,
+                     int family, void *stream);
+
+/* Identity of the capture `stream` is recording into: 0 when it is not capturing, a positive
+ * number that differs between captures while it is, -1 when the runtime cannot say.  No
+ * counterpart in the reference; the adapter uses it to keep decisions taken at capture time
+ * (which scratch a captured kernel reads) from leaking between graphs. */
+long long cmi_stream_capture_id(void *stream);
 
 /* One-time re-layout of a W4A8Weight for the device kernels.
  *   in : packed u8 [ceil(K/2), N] (low nibble = even k, code = q+8) and

@@ -446,3 +446,238 @@ def test_pre_quantised_directory_feeds_the_kernels(tmp_path, orc):
     ref = QWeight(q.wq.to(G.DEV), q.scale.to(G.DEV))
     assert (backend.linear_m(w, x).view(torch.int16) == backend.linear_m(ref, x).view(torch.int16)).all()
     assert (backend.linear(w, x[0]).view(torch.int16) == backend.linear(ref, x[0]).view(torch.int16)).all()
+
+
+# ------------------------------------------------ quantised rows handed forward by the producers
+
+def _count_quantised_routes(monkeypatch):
+    calls = []
+    real = backend._rows_quantised
+
+    def spy(rec, xq, xs, rows, out, stream):
+        calls.append((rec.kind, rows))
+        return real(rec, xq, xs, rows, out, stream)
+
+    monkeypatch.setattr(backend, "_rows_quantised", spy)
+    return calls
+
+
+@pytest.mark.parametrize("rows", [1, 2, 16, 70, 300, 1100])
+def test_table_entry_sequence_hands_quantised_rows_to_the_projection(monkeypatch, rows):
+    """The reference's own call sequence -- ``rms_norm`` then ``linear``, ``add_rms_norm`` then
+    ``linear``, ``silu_mul`` then ``linear`` (ops/norm.py:87,135, models/qwen35/blocks.py:69) -- runs
+    the integer kernels on the rows the producer quantised, with the bits of the route that
+    quantises the bf16 rows again."""
+    g = synth.generator(5)
+    k, n = 2560, 1536
+    w4, q8 = _w4(n, k, g), _q8(n, k, g)
+    wd = _w4(k, 2 * k, g)                      # a "down" projection for the SwiGLU product
+    x = synth.activations(rows, k, g).to(G.DEV)
+    gain = synth.activations(1, k, g)[0].to(G.DEV).contiguous()
+    add = synth.activations(rows, k, g).to(G.DEV)
+    gu = synth.activations(rows, 4 * k, g).to(G.DEV)
+
+    def sequence():
+        outs = []
+        h = backend.rms_norm(x, gain)
+        hv = h.view(-1) if rows == 1 else h.view(rows, k)          # ops/norm.py:87 hands out a view
+        outs.append(backend.linear(w4, hv))
+        outs.append(backend.linear_prefill(w4, h))                 # a second consumer of the same rows
+        outs.append(backend.linear_prefill(q8, h))                 # W8A8 from 64 rows, weight-only below
+        res = x.clone()
+        nxt = torch.empty_like(res)
+        backend.add_rms_norm(res, add, gain, nxt)
+        outs.append(backend.linear_m(w4, nxt) if rows > 1 else backend.linear(w4, nxt[0]))
+        gate, up = gu[:, :2 * k], gu[:, 2 * k:]                    # halves of a fused gate_up output
+        prod = backend.silu_mul(gate, up, up)
+        outs.append(backend.linear_prefill(wd, prod))
+        return outs
+
+    gu0 = gu.clone()                           # silu_mul overwrites the `up` half in place
+    monkeypatch.setattr(backend, "HANDOVER", False)
+    want = sequence()
+    monkeypatch.setattr(backend, "HANDOVER", True)
+    calls = _count_quantised_routes(monkeypatch)
+    gu.copy_(gu0)
+    got = sequence()
+    for i, (a, b) in enumerate(zip(got, want)):
+        assert (a.view(torch.int16) == b.view(torch.int16)).all(), i
+    kinds = [c[0] for c in calls]
+    assert kinds.count(4) == 4                                     # every int4 projection took the handed rows
+    assert kinds.count(8) == (1 if rows >= 64 and not backend._splits_k(rows, n, k, x.device) else 0)
+
+
+def test_handed_rows_are_not_trusted_after_the_tensor_changed(monkeypatch):
+    g = synth.generator(6)
+    k, n = 2560, 1024
+    w4 = _w4(n, k, g)
+    x = synth.activations(4, k, g).to(G.DEV)
+    gain = synth.activations(1, k, g)[0].to(G.DEV).contiguous()
+    backend.linear(w4, x)                                          # a quantising consumer has been seen
+    calls = _count_quantised_routes(monkeypatch)
+
+    def fresh(t):                                                  # the same values in memory of their own
+        return backend.linear_m(w4, t.clone())
+
+    h = backend.rms_norm(x, gain)
+    assert (backend.linear_m(w4, h).view(torch.int16) == fresh(h).view(torch.int16)).all()
+    assert len(calls) == 1
+    h.mul_(2)                                                      # torch writes announce themselves
+    assert (backend.linear_m(w4, h).view(torch.int16) == fresh(h).view(torch.int16)).all()
+    assert len(calls) == 1
+    h = backend.rms_norm(x, gain)
+    other = h.clone()                                              # same values, other memory: not the handed tensor
+    backend.linear_m(w4, other)
+    assert len(calls) == 1
+    backend.linear_m(w4, h[:2])                                    # fewer rows than were handed
+    assert len(calls) == 1
+    backend.linear_m(w4, h)
+    assert len(calls) == 2
+    # one of this backend's own kernels writes into the tensor: the entry goes
+    gate = synth.activations(4, k, g).to(G.DEV)
+    q = torch.empty((4, k), dtype=torch.int8, device=G.DEV)
+    s = torch.empty(4, dtype=torch.float32, device=G.DEV)
+    h = backend.rms_norm(x, gain)
+    backend.silu_mul_quant(gate, x, h, q, s)
+    assert (backend.linear_m(w4, h).view(torch.int16) == fresh(h).view(torch.int16)).all()
+    assert len(calls) == 2
+    # switched off, nothing is handed
+    backend.configure(handover=False)
+    try:
+        h = backend.rms_norm(x, gain)
+        backend.linear_m(w4, h)
+        assert len(calls) == 2 and backend._HANDED is None
+    finally:
+        backend.configure(handover=True)
+
+
+def test_handed_rows_inside_a_captured_graph_and_not_across_its_edge(monkeypatch):
+    """Producer and consumer recorded into one capture replay together (fresh inputs, same bits as
+    eager); a consumer recorded into a capture does not read rows an eager producer left."""
+    g = synth.generator(8)
+    k, n = 2560, 1024
+    w4 = _w4(n, k, g)
+    gain = synth.activations(1, k, g)[0].to(G.DEV).contiguous()
+    x = synth.activations(2, k, g).to(G.DEV)
+    gu = synth.activations(2, 2 * k, g).to(G.DEV)
+
+    def step():
+        a = backend.linear_m(w4, backend.rms_norm(x, gain))
+        up = gu[:, k:].clone()
+        b = backend.linear_m(w4, backend.silu_mul(gu[:, :k], up, up))
+        return a, b
+
+    step()
+    torch.cuda.synchronize()
+    calls = _count_quantised_routes(monkeypatch)
+    eager_h = backend.rms_norm(x, gain)                            # handed eagerly, consumed under capture: refused
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            crossing = backend.linear_m(w4, eager_h)
+            assert len(calls) == 0
+            outs = step()
+            assert len(calls) == 2
+    torch.cuda.current_stream().wait_stream(side)
+    for seed in (1, 2, 3):
+        gg = synth.generator(seed)
+        x.copy_(synth.activations(2, k, gg))
+        gu.copy_(synth.activations(2, 2 * k, gg))
+        junk = torch.randn(1 << 20, device=G.DEV)                  # eager work between the replays
+        del junk
+        graph.replay()
+        torch.cuda.synchronize()
+        backend.configure(handover=False)
+        try:
+            want = step()
+        finally:
+            backend.configure(handover=True)
+        for a, b in zip(outs, want):
+            assert (a.view(torch.int16) == b.view(torch.int16)).all()
+    assert crossing.shape == (2, n)
+
+
+def test_scratch_captured_by_a_graph_survives_forty_other_shapes():
+    """A captured step holds raw addresses of the adapter's scratch; calls with many other shapes
+    (which once evicted and freed it) must leave the replay's bits alone."""
+    g = synth.generator(9)
+    k, n = 2560, 1024
+    w4, q8 = _w4(n, k, g), _q8(n, k, g)
+    x4 = synth.activations(4, k, g).to(G.DEV)
+    x80 = synth.activations(80, k, g).to(G.DEV)
+
+    def step():
+        return backend.linear_m(w4, x4), backend.linear_prefill(q8, x80), backend.linear_prefill(w4, x80)
+
+    step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            outs = step()
+    torch.cuda.current_stream().wait_stream(side)
+    hold = []
+    for rows in range(65, 65 + 44):                                 # other prefill lengths, growing scratch
+        xs = synth.activations(rows * 8, k, synth.generator(rows)).to(G.DEV)
+        backend.linear_prefill(q8, xs)
+        backend.linear_prefill(w4, xs)
+        hold.append(torch.full((1 << 18,), float(rows), device=G.DEV))   # memory a freed block would be reused for
+    torch.cuda.synchronize()
+    gg = synth.generator(77)
+    x4.copy_(synth.activations(4, k, gg))
+    x80.copy_(synth.activations(80, k, gg))
+    graph.replay()
+    torch.cuda.synchronize()
+    for a, b in zip(outs, step()):
+        assert (a.view(torch.int16) == b.view(torch.int16)).all()
+    for rows, t in zip(range(65, 65 + 44), hold):
+        assert bool((t == float(rows)).all())
+
+
+def test_family_is_a_property_of_the_weight_or_the_process():
+    """Static-batch decode is owed "row r == single-row call" (models/qwen35/batch.py:19-22).  It
+    holds in the dot-product family (default) and in the matrix-pipe family, chosen per weight
+    (attribute ``batch_family``) or per process (``configure``) -- every entry switches together."""
+    g = synth.generator(10)
+    k, n = 2560, 1536
+    x = synth.activations(16, k, g).to(G.DEV)
+    plain = _q8(n, k, g)
+    fast = QWeight(plain.wq, plain.scale, batch_family="mfma")
+    y_dot, y_mfma = backend.linear_m(plain, x), backend.linear_m(fast, x)
+    assert _rel(y_mfma, y_dot.float()) < 1e-2
+    assert not (y_mfma.view(torch.int16) == y_dot.view(torch.int16)).all()      # two summation orders
+    for w, y in ((plain, y_dot), (fast, y_mfma)):
+        for r in (0, 5, 15):
+            assert (backend.linear(w, x[r]).view(torch.int16) == y[r].view(torch.int16)).all()
+        for m in (2, 4, 8):
+            assert (backend.linear_m(w, x[:m].contiguous()).view(torch.int16) == y[:m].view(torch.int16)).all()
+    # mfma family: verify and short prefill chunks are the same kernel, so the same bits
+    assert (backend.linear_m_verify(fast, x).view(torch.int16) == y_mfma.view(torch.int16)).all()
+    assert (backend.linear_prefill(fast, x).view(torch.int16) == y_mfma.view(torch.int16)).all()
+    # the process-wide switch does the same for weights that do not say
+    try:
+        assert backend.configure(batch_family="mfma")["batch_family"] == "mfma"
+        assert (backend.linear_m(plain, x).view(torch.int16) == y_mfma.view(torch.int16)).all()
+        assert (backend.linear(plain, x[3]).view(torch.int16) == y_mfma[3].view(torch.int16)).all()
+    finally:
+        backend.configure(batch_family="dot")
+    assert (backend.linear_m(plain, x).view(torch.int16) == y_dot.view(torch.int16)).all()
+    with pytest.raises(ValueError):
+        backend.configure(batch_family="tensor")
+    # the C entry that takes the family as an argument: any number of rows in one call
+    lib = backend._native.load()
+    x100 = synth.activations(100, k, g).to(G.DEV)
+    for family, mfma in ((0, False), (1, True)):
+        y = torch.empty((100, n), dtype=torch.bfloat16, device=G.DEV)
+        backend._native.check(lib.cmi_linear_w8a16(G.ptr(plain.wq), G.ptr(plain.scale), G.ptr(x100), G.ptr(y),
+                                                   100, n, k, family, G.stream()), "linear_w8a16")
+        step = 64 if mfma else 16
+        for lo in range(0, 100, step):
+            piece = G.gemv_w8a16(plain.wq, plain.scale, x100[lo:lo + step].contiguous(), mfma=mfma)
+            assert (y[lo:lo + step].view(torch.int16) == piece.view(torch.int16)).all()
+    assert lib.cmi_linear_w8a16(G.ptr(plain.wq), G.ptr(plain.scale), G.ptr(x100), G.ptr(y), 100, n, k, 2,
+                                G.stream()) == backend._native.E_ARG

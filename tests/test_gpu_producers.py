@@ -104,6 +104,17 @@ def test_silu_mul_table_entries(orc):
     assert (G.bits(one) == out_ref[3]).all()
     with pytest.raises(ValueError):
         backend.silu_mul_quant(gate, up[:, :100], out, out_q, out_s)
+    # any leading shape (the contract writes [...]): collapsible axes run the kernel, other layouts torch
+    g3, u3, o3 = gate.view(3, 3, 512), up.view(3, 3, 512), torch.empty((3, 3, 512), dtype=torch.bfloat16, device=G.DEV)
+    assert backend.silu_mul(g3, u3, o3) is o3 and (G.bits(o3).reshape(9, 512) == out_ref).all()
+    gt = gate.t().contiguous().t()                                         # innermost stride is not 1
+    ot = torch.empty_like(gate)
+    backend.silu_mul(gt, up, ot)
+    assert torch.allclose(ot.float(), (torch.nn.functional.silu(gt) * up).float())
+    gs3 = gate.view(3, 3, 512)[:, :2]                                      # leading axes that do not collapse
+    os3 = torch.empty((3, 2, 512), dtype=torch.bfloat16, device=G.DEV)
+    backend.silu_mul(gs3, up.view(3, 3, 512)[:, :2], os3)
+    assert torch.allclose(os3.float(), out.view(3, 3, 512)[:, :2].float(), rtol=2e-2, atol=1e-3)
     # fp32 inputs are answered by the torch statement of the op
     f = torch.empty((9, 512), device=G.DEV)
     backend.silu_mul(gate.float(), up.float(), f)

@@ -271,18 +271,24 @@ def test_w4_operands_are_checked_before_any_address_reaches_a_kernel():
     assert not backend._kernels_take(NS(wq=torch.zeros((4, 24), dtype=torch.int8), scale=torch.ones(4)))
 
 
-def test_scratch_and_record_pools_evict_the_least_recently_used_entry(monkeypatch):
-    monkeypatch.setattr(backend, "_SCRATCH_MAX", 3)
-    backend._SCRATCH.clear()
+def test_scratch_never_moves_under_a_caller_and_the_record_pool_evicts_the_oldest(monkeypatch):
+    """Scratch addresses may sit inside captured graphs: a block is outgrown, never freed or moved."""
+    arena = backend._Arena("test")
+    monkeypatch.setattr(backend, "_WORKSPACE", arena)
+    backend._WORKSPACE_BYTES.clear()
     cpu = torch.device("cpu")
-    a = backend._scratch(1, 16, cpu)
-    assert a.dtype == torch.uint8 and a.numel() == 512     # 16 B of rows + 4 B of scale, 256 each
-    backend._scratch(2, 16, cpu)
-    backend._scratch(3, 16, cpu)
-    assert backend._scratch(1, 16, cpu) is a               # refreshed: now the most recent
-    backend._scratch(4, 16, cpu)                           # evicts (2, 16), the oldest
-    assert list(k[0] for k in backend._SCRATCH) == [3, 1, 4]
-    backend._SCRATCH.clear()
+    a, nbytes = backend._scratch(1, 16, cpu)
+    assert nbytes == 512                                   # 16 B of rows + 4 B of scale, 256 each
+    first = arena.blocks[None]
+    assert a == first.data_ptr() and first.numel() >= nbytes
+    for rows in range(2, 40):                              # forty other shapes: same block, same address
+        assert backend._scratch(rows, 16, cpu)[0] == a
+    assert not arena.retired
+    big, big_bytes = backend._scratch(4096, 4096, cpu)     # outgrows the block
+    assert arena.retired == [first] and arena.blocks[None].numel() >= big_bytes
+    assert first.data_ptr() == a                           # the outgrown block is still allocated
+    assert backend._scratch(1, 16, cpu)[0] == big          # one block serves every shape
+    backend._WORKSPACE_BYTES.clear()
     monkeypatch.setattr(backend, "_RECORDS_MAX", 2)
     backend._RECORDS.clear()
     g = synth.generator()

@@ -57,6 +57,37 @@ def test_static_workspace_entry_matches_the_workspace_entry_on_consecutive_calls
     assert (_static(w42, ws2, x3, n2, k2).view(torch.int16) == _with_workspace(w42, ws2, x3, n2, k2).view(torch.int16)).all()
 
 
+def test_static_workspace_entry_replays_inside_a_captured_graph():
+    """What the entry exists for: after one eager call per shape (the first call on a device takes
+    the array's address and raises the kernels' LDS limits, which a capture cannot record), the call
+    is recorded into a graph -- a hipMalloc or an attribute change inside it would fail the capture --
+    and replayed on new activations in the same buffer, bit for bit the eager result."""
+    g = synth.generator(4321, G.DEV)
+    n, k = 1536, 2560
+    w = synth.int4_weight(n, k, g)
+    w4, ws = G.w4_repack(w.packed, w.scale, k)
+    xs = {m: synth.activations(m, k, g) for m in (1, 6, 40)}
+    for x in xs.values():
+        _static(w4, ws, x, n, k)                             # warm-up, eager
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            outs = {m: _static(w4, ws, x, n, k) for m, x in xs.items()}
+    torch.cuda.current_stream().wait_stream(side)
+    for seed in (1, 2, 3):
+        gg = synth.generator(seed, G.DEV)
+        for m, x in xs.items():
+            x.copy_(synth.activations(m, k, gg))
+        graph.replay()
+        torch.cuda.synchronize()
+        for m, x in xs.items():
+            want = _with_workspace(w4, ws, x, n, k)
+            assert (outs[m].view(torch.int16) == want.view(torch.int16)).all(), (seed, m)
+
+
 def test_static_workspace_entry_refuses_what_does_not_fit():
     lib = _native.load()
     one = ctypes.c_void_p(256)
