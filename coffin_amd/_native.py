@@ -47,7 +47,8 @@ SIGNATURES: dict[str, list] = {
 #: Entry points that do not return a status.
 OTHER_RESTYPES = {"cmi_linear_workspace_bytes": ([_ci, _ci], _sz),
                   "cmi_linear_w8a8_workspace_bytes": ([_ci, _ci, _ci], _sz),
-                  "cmi_stream_capture_id": ([_vp], ctypes.c_longlong)}
+                  "cmi_stream_capture_id": ([_vp], ctypes.c_longlong),
+                  "cmi_w4_device_k": ([_ci, _ci], _ci)}
 
 
 class NativeError(RuntimeError):

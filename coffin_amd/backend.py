@@ -268,7 +268,7 @@ def _w4_check(w) -> None:
     if packed.dtype != torch.uint8 or packed.dim() != 2 or not packed.is_contiguous():
         raise ValueError(f"int4 weight: packed must be contiguous 2-D uint8, got "
                          f"{tuple(packed.shape)} {packed.dtype}")
-    if packed.shape[1] != n or packed.shape[0] * 2 < k:
+    if packed.shape[1] != n or gs < 1 or packed.shape[0] * 2 < -(-k // gs) * gs:
         raise ValueError(f"int4 weight: packed {tuple(packed.shape)} does not hold K={k} x N={n} codes")
     if scale.dtype != torch.float32 or scale.dim() != 2 or not scale.is_contiguous():
         raise ValueError(f"int4 weight: scale must be contiguous 2-D fp32, got "
@@ -284,23 +284,28 @@ def _w4_check(w) -> None:
 def _kernels_take(w) -> bool:
     """Whether the native kernels are built for this quantized weight's shape.
 
-    int4: group size 128 and K a multiple of 128; int8: K a multiple of 16.  Other shapes are
-    answered by the torch statement of the op (the reference's corex adapter likewise falls back
-    for group sizes its GEMM does not take, backends/corex/__init__.py:633).
+    int4: group sizes 64, 128 and 256, any K (rows are padded to whole groups on the device);
+    int8: K a multiple of 16.  Other shapes are answered by the torch statement of the op (the
+    reference's corex adapter likewise falls back for group sizes its GEMM does not take,
+    backends/corex/__init__.py:633).
     """
     if _is_w4(w):
-        return int(w.group_size) == 128 and int(w.k) % 128 == 0
+        gs, k = int(w.group_size), int(w.k)
+        # whole groups in storage, as the encoder writes them (tools/quant_disk_w4a8.py:60-66)
+        return gs in (64, 128, 256) and k >= 1 and int(w.packed.shape[0]) * 2 >= -(-k // gs) * gs
     return int(w.wq.shape[-1]) % 16 == 0
 
 
 def _w4_operands(w):
-    """Device layout ``(w4 uint8 [N,K/2], ws fp32 [N,G])`` of a W4A8Weight-like, built once."""
+    """Device layout ``(w4 uint8 [N,Kd/2], ws fp32 [N,Kd/gs])`` of a W4A8Weight-like, built once
+    (``Kd``: K rounded up to whole groups and whole 128-element steps, ``cmi_w4_device_k``)."""
     def make():
         _w4_check(w)
         n, k, gs = int(w.n), int(w.k), int(w.group_size)
-        w4 = torch.empty((n, k // 2), dtype=torch.uint8, device=w.packed.device)
-        ws = torch.empty((n, k // gs), dtype=torch.float32, device=w.packed.device)
         lib = _native.load()
+        kd = int(lib.cmi_w4_device_k(k, gs))
+        w4 = torch.empty((n, kd // 2), dtype=torch.uint8, device=w.packed.device)
+        ws = torch.empty((n, kd // gs), dtype=torch.float32, device=w.packed.device)
         with torch.cuda.device(w.packed.device):
             _native.check(lib.cmi_w4_repack(_ptr(w.packed), _ptr(w.scale), _ptr(w4), _ptr(ws),
                                             n, k, gs, _stream()), "w4 re-layout")
@@ -399,7 +404,7 @@ class _Record:
     """What the adapters need of one quantized weight, resolved once: operand addresses in
     device layout, shape, device.  Holds no strong reference to the caller's tensors."""
 
-    __slots__ = ("kind", "src", "src2", "a", "b", "n", "k", "gs", "dev", "family")
+    __slots__ = ("kind", "src", "src2", "a", "b", "n", "k", "kd", "gs", "dev", "family")
 
 
 #: id(weight object) -> _Record; an entry is trusted only while the tensors it was
@@ -436,10 +441,12 @@ def _make_record(w) -> _Record:
         w4, ws = _w4_operands(w)
         rec.kind, rec.src, rec.a, rec.b = 4, weakref.ref(w.packed), w4.data_ptr(), ws.data_ptr()
         rec.n, rec.k, rec.gs, rec.dev = int(w.n), int(w.k), int(w.group_size), w.packed.device
+        rec.kd = 2 * int(w4.shape[1])
     else:
         wq, scale = _q8_operands(w)
         rec.kind, rec.src, rec.a, rec.b = 8, weakref.ref(w.wq), wq.data_ptr(), scale.data_ptr()
         rec.n, rec.k, rec.gs, rec.dev = int(wq.shape[0]), int(wq.shape[1]), 0, w.wq.device
+        rec.kd = rec.k
     family = getattr(w, "batch_family", None)
     if family is not None and family not in _FAMILIES:
         raise ValueError(f"batch_family of a weight must be 'dot' or 'mfma', got {family!r}")
@@ -482,7 +489,7 @@ def _rows_w4(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor) -> N
     global _QUANT_CONSUMER_SEEN
     _QUANT_CONSUMER_SEEN = True
     n, k = rec.n, rec.k
-    work, nbytes = _scratch(rows, k, act.device)
+    work, nbytes = _scratch(rows, rec.kd, act.device)
     rc = _native.load().cmi_linear_w4a8_bf16(rec.a, rec.b, act.data_ptr(), out.data_ptr(), rows, n, k, rec.gs,
                                              work, nbytes, _stream())
     if rc:
@@ -568,9 +575,9 @@ def _project(w, x: torch.Tensor, prefill: bool, min_rows: int = PREFILL_MIN_ROWS
     out = torch.empty((rec.n,) if nd == 1 else (rows, rec.n), dtype=torch.bfloat16, device=dev)
     if rows == 0:
         return out
-    quantising = (rec.kind == 4 and not (W4A16 and rows <= W4A16_MAX_ROWS and rec.k <= 10240)) or \
-                 (rec.kind == 8 and prefill and rows >= min_rows)
-    if quantising and _HANDED is not None:
+    w4a16 = rec.kind == 4 and W4A16 and rows <= W4A16_MAX_ROWS and rec.k <= 10240 and rec.gs == 128 and rec.kd == rec.k
+    quantising = (rec.kind == 4 and not w4a16) or (rec.kind == 8 and prefill and rows >= min_rows)
+    if quantising and _HANDED is not None and rec.kd == rec.k:
         # the rows a producer of this backend left behind for exactly this tensor
         stream = _stream()
         handed = _handed_rows(x, rows, rec.k, stream)
@@ -579,7 +586,7 @@ def _project(w, x: torch.Tensor, prefill: bool, min_rows: int = PREFILL_MIN_ROWS
             return out
     act = x if x.is_contiguous() else x.contiguous()
     if rec.kind == 4:
-        if W4A16 and rows <= W4A16_MAX_ROWS and rec.k <= 10240:
+        if w4a16:
             _rows_w4a16(rec, act, rows, out)
         else:
             _rows_w4(rec, act, rows, out)
@@ -656,6 +663,9 @@ def linear_quantized(w, xq: torch.Tensor, xs: torch.Tensor) -> torch.Tensor:
     rows, k = xq.shape
     if k != rec.k:
         raise ValueError(f"linear_quantized expects K={rec.k}, got {k}")
+    if rec.kd != rec.k:
+        raise ValueError(f"linear_quantized: this weight's rows are padded to {rec.kd} on the device; "
+                         "pass bf16 rows to linear*, which pads the quantised rows itself")
     out = torch.empty((rows, rec.n), dtype=torch.bfloat16, device=xq.device)
     if rows == 0:
         return out
@@ -891,7 +901,7 @@ def embed_rows(w, ids: torch.Tensor) -> torch.Tensor:
         if not (_is_w4(w) or _is_q8(w)):
             raise ValueError("embed_rows expects a QWeight or W4A8Weight")
         if _is_w4(w) and not _kernels_take(w):
-            raise ValueError("embed_rows: int4 rows are gathered for group size 128 and K % 128 == 0")
+            raise ValueError("embed_rows: int4 rows are gathered for group sizes 64, 128 and 256")
         rec = _make_record(w)
     if rec.dev.type != "cuda":
         raise ValueError(f"coffin_amd: a quantized embedding is gathered on the GPU, weight is on {rec.dev}")

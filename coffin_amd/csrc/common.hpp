@@ -44,6 +44,9 @@ int gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, const f
 size_t gemm_w8a8_split_bytes(int M, int N, int K);
 // quant_act_i8.hip: cmi_quant_act_i8 that also clears n_zero ints at `zero` (null / 0: none).
 int quant_act_i8_and_clear(const void *x, int8_t *q, float *s, int M, int K, int *zero, int n_zero, void *stream);
+// quant_act_i8.hip: the quantiser writing rows of pitch ldq >= K, the tail K .. ldq-1 cleared (rows
+// of an int4 weight whose K is padded to whole groups on the device).
+int quant_act_i8_padded(const void *x, int8_t *q, float *s, int M, int K, int ldq, void *stream);
 // 16-row weight tiles per workgroup (1 or 2) that gemm_w8a8_rows16 uses for 17..128 rows.
 int gemm_w8a8_rows_tiles(int N);
 

@@ -99,6 +99,32 @@ embed_rows_w4_kernel(const uint8_t *__restrict__ w4, const float *__restrict__ w
     }
 }
 
+// Any group size the device layout takes and any K: a thread expands one 32-bit word (8 codes);
+// rows are Kd / 2 bytes apart (Kd: K padded to whole groups and steps), the output has K columns.
+__global__ void __launch_bounds__(THREADS)
+embed_rows_w4_general(const uint8_t *__restrict__ w4, const float *__restrict__ ws, const int64_t *__restrict__ ids,
+                      uint16_t *__restrict__ out, int N, int K, int Kd, int gs) {
+    const int t = blockIdx.x;
+    const int64_t id = ids[t];
+    uint16_t *orow = out + (size_t)t * K;
+    if (id < 0 || id >= N) {
+        for (int k = threadIdx.x; k < K; k += THREADS) orow[k] = 0x7fc0;
+        return;
+    }
+    const uint32_t *wrow = reinterpret_cast<const uint32_t *>(w4 + (size_t)id * (Kd / 2));
+    const float *srow = ws + (size_t)id * (Kd / gs);
+    for (int i = threadIdx.x; i * 8 < K; i += THREADS) {
+        const uint32_t w = wrow[i];
+        const float sc = srow[(8 * i) / gs];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int lo = 8 * i + b, hi = lo + 4;
+            if (lo < K) orow[lo] = (uint16_t)f32_to_bf16_bits(__fmul_rn((float)((int)((w >> (8 * b)) & 15) - 8), sc));
+            if (hi < K) orow[hi] = (uint16_t)f32_to_bf16_bits(__fmul_rn((float)((int)((w >> (8 * b + 4)) & 15) - 8), sc));
+        }
+    }
+}
+
 }  // namespace
 
 extern "C" int cmi_embed_rows_i8(const int8_t *wq, const float *ws, const int64_t *ids, void *out, int T, int N,
@@ -120,11 +146,14 @@ extern "C" int cmi_embed_rows_w4(const uint8_t *w4, const float *ws, const int64
     CMI_REQUIRE(T >= 0 && N >= 1 && K >= 1, CMI_E_ARG, "cmi_embed_rows_w4: bad shape T=%d N=%d K=%d", T, N, K);
     if (T == 0) return CMI_OK;
     CMI_REQUIRE(w4 && ws && ids && out, CMI_E_ARG, "cmi_embed_rows_w4: null pointer");
-    CMI_REQUIRE(gs == 128 && K % 128 == 0, CMI_E_UNSUPPORTED,
-                "cmi_embed_rows_w4: group size %d, K=%d; built for group size 128 and K %% 128 == 0", gs, K);
-    CMI_REQUIRE(aligned(w4, 16) && aligned(out, 16) && aligned(ids, 8), CMI_E_ARG,
-                "cmi_embed_rows_w4: w4 and out must be 16-byte aligned, ids 8-byte aligned int64");
+    const int Kd = cmi_w4_device_k(K, gs);
+    CMI_REQUIRE(Kd > 0, CMI_E_UNSUPPORTED, "cmi_embed_rows_w4: group size %d, the device layout is built for 64, 128 and 256", gs);
+    CMI_REQUIRE(aligned(w4, 16) && aligned(out, 2) && aligned(ids, 8), CMI_E_ARG,
+                "cmi_embed_rows_w4: w4 must be 16-byte aligned, ids 8-byte aligned int64");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    embed_rows_w4_kernel<<<dim3(T), dim3(THREADS), 0, st>>>(w4, ws, ids, static_cast<uint16_t *>(out), N, K);
+    if (gs == 128 && Kd == K && aligned(out, 16))
+        embed_rows_w4_kernel<<<dim3(T), dim3(THREADS), 0, st>>>(w4, ws, ids, static_cast<uint16_t *>(out), N, K);
+    else
+        embed_rows_w4_general<<<dim3(T), dim3(THREADS), 0, st>>>(w4, ws, ids, static_cast<uint16_t *>(out), N, K, Kd, gs);
     return check_launch("cmi_embed_rows_w4");
 }

@@ -54,9 +54,13 @@ typedef __attribute__((address_space(3))) void *lds_ptr_t;
 
 // DUMP: also write the int32 group sums (parity checks); a separate instantiation, the
 // 64 extra store addresses per lane would otherwise be carried through the hot loop.
-template <bool DUMP>
+// LG: log2(group size / 32).  2: a K step is a group (what the kernel is tuned for).  3: a group is
+// two steps, the integer accumulators run on over the odd step and flush behind it.  1: a step holds
+// two groups, flushed behind the second and the fourth k quarter.
+template <bool DUMP, int LG = 2>
 __global__ void __launch_bounds__(THREADS, 2)
 gemm_w4a8_kernel(const Args a) {
+    static_assert(LG >= 1 && LG <= 3, "group sizes 64, 128, 256");
     extern __shared__ __align__(16) int8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -166,9 +170,33 @@ gemm_w4a8_kernel(const Args a) {
     Frag f0, f1;
     uint4 wreg[2];
     float sc[2];
+    float sc_b[2] = {0.f, 0.f};  // LG == 1: scales of the step's second group
+    auto dump = [&](int group) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int n = nb + j * 32 + (lane & 31);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int m = mb + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                    if (m < a.M && n < a.N) a.group_acc[((size_t)m * a.G + group) * a.N + n] = acc[i][j][v];
+                }
+            }
+    };
+    auto flush = [&](const float (&scale)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) total[i][j][v] = fmaf((float)acc[i][j][v], scale[j], total[i][j][v]);
+    };
     auto step = [&](auto more_tag, int ks) {
         constexpr bool MORE = decltype(more_tag)::value;  // a step ks+2 exists
         const int cur = ks & 1;
+        const bool opens = LG == 3 ? (ks & 1) == 0 : true;   // this step starts a group
+        const bool closes = LG == 3 ? (ks & 1) == 1 || ks + 1 == ksteps : true;
         // four MFMAs with the four fragment reads of the next quarter spread between them
         auto pace_quarter = [&]() {
 #pragma unroll
@@ -178,27 +206,37 @@ gemm_w4a8_kernel(const Args a) {
             }
         };
         read_q(cur, 1, f1);
-        mma_q(f0, true);
+        mma_q(f0, opens);
         pace_quarter();
         read_q(cur, 2, f0);
         mma_q(f1, false);
         pace_quarter();
+        if constexpr (LG == 1) {  // the step's first group is complete
+            if constexpr (DUMP) dump(2 * ks);
+            flush(sc);
+        }
         read_q(cur, 3, f1);
-        mma_q(f0, false);
+        mma_q(f0, LG == 1);
         pace_quarter();
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         if (ks + 1 < ksteps) stash_w(cur ^ 1, wreg);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        float sc_next[2] = {0.f, 0.f};
+        float sc_next[2] = {0.f, 0.f}, sc_next_b[2] = {0.f, 0.f};
         if constexpr (MORE) {
             issue_x(cur, ks + 2);
             fetch_w(wreg, ks + 2);
         }
         if (ks + 1 < ksteps) {
-            sc_next[0] = wsp[0][ks + 1];
-            sc_next[1] = wsp[1][ks + 1];
+            // scales of the group(s) the next step meets: group = step (LG 2), step / 2 (LG 3), 2 step and 2 step + 1 (LG 1)
+            const int g = LG == 3 ? (ks + 1) >> 1 : LG == 1 ? 2 * (ks + 1) : ks + 1;
+            sc_next[0] = wsp[0][g];
+            sc_next[1] = wsp[1][g];
+            if constexpr (LG == 1) {
+                sc_next_b[0] = wsp[0][g + 1];
+                sc_next_b[1] = wsp[1][g + 1];
+            }
         }
         read_q(cur ^ 1, 0, f0);  // past the last step: a stale stage nobody uses
         mma_q(f1, false);
@@ -208,27 +246,17 @@ gemm_w4a8_kernel(const Args a) {
             if (MORE) __builtin_amdgcn_sched_group_barrier(0x010, 2, 0);  // requests for step ks+2
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
-        if constexpr (DUMP) {
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const int n = nb + j * 32 + (lane & 31);
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int m = mb + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                        if (m < a.M && n < a.N) a.group_acc[((size_t)m * a.G + ks) * a.N + n] = acc[i][j][v];
-                    }
-                }
+        if (closes) {
+            if constexpr (DUMP) dump(LG == 3 ? ks >> 1 : LG == 1 ? 2 * ks + 1 : ks);
+            if constexpr (LG == 1) flush(sc_b);
+            else flush(sc);
         }
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-            for (int j = 0; j < 2; ++j)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) total[i][j][v] = fmaf((float)acc[i][j][v], sc[j], total[i][j][v]);
         sc[0] = sc_next[0];
         sc[1] = sc_next[1];
+        if constexpr (LG == 1) {
+            sc_b[0] = sc_next_b[0];
+            sc_b[1] = sc_next_b[1];
+        }
     };
     using more_t = std::integral_constant<bool, true>;
     using last_t = std::integral_constant<bool, false>;
@@ -238,6 +266,10 @@ gemm_w4a8_kernel(const Args a) {
     fetch_w(wreg, 0);
     sc[0] = wsp[0][0];
     sc[1] = wsp[1][0];
+    if constexpr (LG == 1) {
+        sc_b[0] = wsp[0][1];
+        sc_b[1] = wsp[1][1];
+    }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     stash_w(0, wreg);
     if (ksteps > 1) {
@@ -278,8 +310,10 @@ extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     CMI_REQUIRE(M >= 0 && N >= 1 && K >= BK, CMI_E_ARG, "cmi_gemm_w4a8: bad shape M=%d N=%d K=%d", M, N, K);
     if (M == 0) return CMI_OK;  // an empty batch has no storage to point at
     CMI_REQUIRE(w4 && ws && xq && xs && y, CMI_E_ARG, "cmi_gemm_w4a8: null pointer");
-    CMI_REQUIRE(gs == BK, CMI_E_UNSUPPORTED, "cmi_gemm_w4a8: group size %d, kernels are built for %d", gs, BK);
-    CMI_REQUIRE(K % BK == 0, CMI_E_UNSUPPORTED, "cmi_gemm_w4a8: K=%d is not a multiple of %d", K, BK);
+    CMI_REQUIRE(gs == 64 || gs == BK || gs == 256, CMI_E_UNSUPPORTED,
+                "cmi_gemm_w4a8: group size %d, kernels are built for 64, 128 and 256", gs);
+    CMI_REQUIRE(K % BK == 0 && K % gs == 0, CMI_E_UNSUPPORTED,
+                "cmi_gemm_w4a8: K=%d is not a multiple of 128 and of the group size %d (pad the rows with zeros)", K, gs);
     CMI_REQUIRE(aligned(xq, 16) && aligned(w4, 16), CMI_E_ARG,
                 "cmi_gemm_w4a8: xq and w4 must be 16-byte aligned");
     // Which kernel: with few tiles a launch is a chain of K/128 dependent steps and the kernels differ
@@ -290,8 +324,10 @@ extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     // bits from all of them.  Cost models (us) fitted to cold-weight measurements on ten layer
     // shapes x eleven batch sizes.  The ring kernels do not write the group sums.
     const int forced = option_gemm_tile();
-    int ring = !group_acc && (forced == 64 || forced == 6464) ? forced : 0;
-    if (!forced) {
+    int ring = !group_acc && gs == BK && (forced == 64 || forced == 6464) ? forced : 0;
+    // groups of 64 and 256: the two-stage tile kernel (and, up to 16 rows, the general GEMV)
+    if (gs != BK && M <= 16 && !forced) return cmi_gemv_w4a8(w4, ws, xq, xs, y, group_acc, M, N, K, gs, stream);
+    if (!forced && gs == BK) {
         const double steps = K / 128.0, wn = (double)N * K;
         const double tiles = (double)a_ceil(M, BM) * a_ceil(N, BN);
         const double t_tiled = 3.0 + steps * (tiles <= 512 ? 1.15 + 0.0013 * tiles : 1.6 * ceil(tiles / 512.0));
@@ -337,19 +373,19 @@ extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     a.M = M;
     a.N = N;
     a.K = K;
-    a.G = K / BK;
+    a.G = K / gs;
     a.tiles_m = (M + BM - 1) / BM;
     a.tiles_n = (N + BN - 1) / BN;
-    static std::atomic<uint64_t> devices[2];
-    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w4a8_kernel<false>),
-                                   LDS_BYTES, devices[0], "cmi_gemm_w4a8"))
-        return rc;
-    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w4a8_kernel<true>),
-                                   LDS_BYTES, devices[1], "cmi_gemm_w4a8"))
-        return rc;
     const dim3 grid(a.tiles_m * a.tiles_n), block(THREADS);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (group_acc) gemm_w4a8_kernel<true><<<grid, block, LDS_BYTES, st>>>(a);
-    else gemm_w4a8_kernel<false><<<grid, block, LDS_BYTES, st>>>(a);
-    return check_launch("cmi_gemm_w4a8");
+    static std::atomic<uint64_t> devices[6];
+    auto run = [&](auto kernel, int slot) {
+        if (const int rc = reserve_lds(reinterpret_cast<const void *>(kernel), LDS_BYTES, devices[slot], "cmi_gemm_w4a8"))
+            return rc;
+        kernel<<<grid, block, LDS_BYTES, st>>>(a);
+        return check_launch("cmi_gemm_w4a8");
+    };
+    if (gs == 64) return group_acc ? run(gemm_w4a8_kernel<true, 1>, 0) : run(gemm_w4a8_kernel<false, 1>, 1);
+    if (gs == 256) return group_acc ? run(gemm_w4a8_kernel<true, 3>, 2) : run(gemm_w4a8_kernel<false, 3>, 3);
+    return group_acc ? run(gemm_w4a8_kernel<true, 2>, 4) : run(gemm_w4a8_kernel<false, 2>, 5);
 }

@@ -272,9 +272,10 @@ int launch_xv(const W4Args &a, hipStream_t st) {
 // Groups of 64 or 256: quantised activations only, one row pair per wavefront, one or two chunks per trip.
 template <int M>
 int launch_other_group(const W4Args &a, int ch, int lg, hipStream_t st) {
-    if (lg == 1) return ch == 1 ? launch_xv<M, 1, 1, 0, 1>(a, st) : launch_xv<M, 1, 2, 0, 1>(a, st);
-    if constexpr (M <= 8) return ch == 1 ? launch_xv<M, 1, 1, 0, 3>(a, st) : launch_xv<M, 1, 2, 0, 3>(a, st);
-    else return launch_xv<M, 1, 1, 0, 3>(a, st);
+    if constexpr (M <= 8) {
+        if (ch == 2) return lg == 1 ? launch_xv<M, 1, 2, 0, 1>(a, st) : launch_xv<M, 1, 2, 0, 3>(a, st);
+    }
+    return lg == 1 ? launch_xv<M, 1, 1, 0, 1>(a, st) : launch_xv<M, 1, 1, 0, 3>(a, st);
 }
 
 template <int M, int R2, int CH>
@@ -320,10 +321,12 @@ int run_gemv_w4a8(const char *who, const uint8_t *w4, const float *ws, const int
                   const void *xb, int8_t *xq_out, float *xs_out, void *y, int32_t *group_acc, int M, int N,
                   int K, int gs, void *stream) {
     CMI_REQUIRE(M >= 1 && M <= 16, CMI_E_UNSUPPORTED, "%s: M=%d outside 1..16", who, M);
-    CMI_REQUIRE(N >= 1 && K >= GS, CMI_E_ARG, "%s: bad shape N=%d K=%d", who, N, K);
-    CMI_REQUIRE(gs == GS, CMI_E_UNSUPPORTED, "%s: group size %d, kernels are built for %d", who, gs, GS);
-    CMI_REQUIRE(K % GS == 0, CMI_E_UNSUPPORTED, "%s: K=%d is not a multiple of %d", who, K, GS);
-    const Plan p = make_plan(M, N, K);
+    CMI_REQUIRE(gs == 64 || gs == 128 || gs == 256, CMI_E_UNSUPPORTED, "%s: group size %d, kernels are built for 64, 128 and 256", who, gs);
+    CMI_REQUIRE(N >= 1 && K >= gs, CMI_E_ARG, "%s: bad shape N=%d K=%d", who, N, K);
+    CMI_REQUIRE(K % gs == 0, CMI_E_UNSUPPORTED, "%s: K=%d is not a multiple of the group size %d (pad the rows with zeros)", who, K, gs);
+    CMI_REQUIRE(gs == GS || !xb, CMI_E_UNSUPPORTED, "%s: group size %d takes quantised rows only", who, gs);
+    const int lg = gs == 64 ? 1 : gs == 128 ? 2 : 3;
+    const Plan p = make_plan(M, N, K, lg);
     W4Args a;
     a.w4 = w4;
     a.ws = ws;
@@ -337,12 +340,21 @@ int run_gemv_w4a8(const char *who, const uint8_t *w4, const float *ws, const int
     a.M = M;
     a.N = N;
     a.K = K;
-    a.G = K / GS;
+    a.G = K / gs;
     a.nchunks = K / 32;
     a.KW = p.kw;
     a.teams = p.teams;
     a.iters = p.iters;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (lg != 2) {
+        switch (p.mt) {
+            case 1: return launch_other_group<1>(a, p.ch, lg, st);
+            case 2: return launch_other_group<2>(a, p.ch, lg, st);
+            case 4: return launch_other_group<4>(a, p.ch, lg, st);
+            case 8: return launch_other_group<8>(a, p.ch, lg, st);
+            default: return launch_other_group<16>(a, p.ch, lg, st);
+        }
+    }
     switch (p.mt) {
         case 1: return dispatch_r<1>(a, p, st);
         case 2: return dispatch_r<2>(a, p, st);
@@ -395,7 +407,7 @@ extern "C" int cmi_gemv_w4a8_bf16(const uint8_t *w4, const float *ws, const void
                 "cmi_gemv_w4a8_bf16: M=%d outside 1..%d (quantise with cmi_quant_act_i8 and call cmi_gemv_w4a8)",
                 M, FUSED_MAX_ROWS);
     CMI_REQUIRE(N >= 1 && K >= GS, CMI_E_ARG, "cmi_gemv_w4a8_bf16: bad shape N=%d K=%d", N, K);
-    CMI_REQUIRE(gs == GS, CMI_E_UNSUPPORTED, "cmi_gemv_w4a8_bf16: group size %d, kernels are built for %d", gs, GS);
+    CMI_REQUIRE(gs == GS, CMI_E_UNSUPPORTED, "cmi_gemv_w4a8_bf16: group size %d, the fused kernels are built for %d (quantise and call cmi_gemv_w4a8)", gs, GS);
     CMI_REQUIRE(K % GS == 0, CMI_E_UNSUPPORTED, "cmi_gemv_w4a8_bf16: K=%d is not a multiple of %d", K, GS);
     // long rows: the matrix-pipe kernel with the quantiser folded in (the dot-product kernel shares
     // such rows among wavefronts and its fp32 chain serialises: 10.5 us at 9728 -> 2560; or holds

@@ -29,15 +29,19 @@ bool w4_fused_route(int rows, int N, int K) {
 
 int cmi::linear_w4a8_rows(const uint8_t *w4, const float *ws, const void *x, void *y, int M, int N, int K,
                           int gs, int8_t *xq, float *xs, void *stream) {
-    if (w4_fused_route(M, N, K)) {
+    // the device copy of the weight has rows of Kd >= K codes (whole groups, whole 128-element
+    // steps, cmi_w4_device_k); the quantised rows are padded with zeros to match
+    const int Kd = cmi_w4_device_k(K, gs);
+    CMI_REQUIRE(Kd > 0, CMI_E_UNSUPPORTED, "cmi_linear_w4a8_bf16: group size %d, the kernels are built for 64, 128 and 256", gs);
+    if (gs == 128 && Kd == K && w4_fused_route(M, N, K)) {
         const int rc = cmi_gemv_w4a8_bf16(w4, ws, x, y, nullptr, nullptr, nullptr, M, N, K, gs, stream);
         if (rc != CMI_E_UNSUPPORTED) return rc;
     }
-    if (const int rc = cmi_quant_act_i8(x, xq, xs, M, K, stream)) return rc;
+    if (const int rc = quant_act_i8_padded(x, xq, xs, M, K, Kd, stream)) return rc;
     // up to 16 rows the GEMV entry; beyond, the GEMM entry (which itself goes through the
     // read-once kernels while they are cheaper than the tile pipeline)
-    if (M <= 16) return cmi_gemv_w4a8(w4, ws, xq, xs, y, nullptr, M, N, K, gs, stream);
-    return cmi_gemm_w4a8(w4, ws, xq, xs, y, nullptr, M, N, K, gs, stream);
+    if (M <= 16) return cmi_gemv_w4a8(w4, ws, xq, xs, y, nullptr, M, N, Kd, gs, stream);
+    return cmi_gemm_w4a8(w4, ws, xq, xs, y, nullptr, M, N, Kd, gs, stream);
 }
 
 namespace {
@@ -93,11 +97,13 @@ extern "C" int cmi_linear_w8a8_bf16(const void *x, const int8_t *wq, const float
 
 extern "C" int cmi_linear_w4a8_bf16(const uint8_t *w4, const float *ws, const void *x, void *y, int M, int N, int K,
                                     int gs, void *workspace, size_t workspace_bytes, void *stream) {
-    CMI_REQUIRE(M >= 0 && N >= 1 && K >= 128, CMI_E_ARG, "cmi_linear_w4a8_bf16: bad shape M=%d N=%d K=%d", M, N, K);
+    CMI_REQUIRE(M >= 0 && N >= 1 && K >= 1, CMI_E_ARG, "cmi_linear_w4a8_bf16: bad shape M=%d N=%d K=%d", M, N, K);
     if (M == 0) return CMI_OK;
     CMI_REQUIRE(w4 && ws && x && y, CMI_E_ARG, "cmi_linear_w4a8_bf16: null pointer");
+    const int Kd = cmi_w4_device_k(K, gs);
+    CMI_REQUIRE(Kd > 0, CMI_E_UNSUPPORTED, "cmi_linear_w4a8_bf16: group size %d, the kernels are built for 64, 128 and 256", gs);
     int8_t *xq;
     float *xs;
-    if (const int rc = split_workspace("cmi_linear_w4a8_bf16", workspace, workspace_bytes, M, K, &xq, &xs)) return rc;
+    if (const int rc = split_workspace("cmi_linear_w4a8_bf16", workspace, workspace_bytes, M, Kd, &xq, &xs)) return rc;
     return linear_w4a8_rows(w4, ws, x, y, M, N, K, gs, xq, xs, stream);
 }

@@ -48,11 +48,13 @@ int static_workspace(unsigned char **out) {
 
 extern "C" int cmi_linear_w4a8_bf16_static(const uint8_t *w4, const float *ws, const void *x, void *y, int M, int N,
                                            int K, int gs, void *stream) {
-    CMI_REQUIRE(M >= 0 && N >= 1 && K >= 128, CMI_E_ARG, "cmi_linear_w4a8_bf16_static: bad shape M=%d N=%d K=%d", M,
+    CMI_REQUIRE(M >= 0 && N >= 1 && K >= 1, CMI_E_ARG, "cmi_linear_w4a8_bf16_static: bad shape M=%d N=%d K=%d", M,
                 N, K);
     if (M == 0) return CMI_OK;
     CMI_REQUIRE(w4 && ws && x && y, CMI_E_ARG, "cmi_linear_w4a8_bf16_static: null pointer");
-    CMI_REQUIRE(M <= STATIC_MAX_ROWS && (size_t)M * K <= STATIC_XQ_BYTES, CMI_E_UNSUPPORTED,
+    const int Kd = cmi_w4_device_k(K, gs);
+    CMI_REQUIRE(Kd > 0, CMI_E_UNSUPPORTED, "cmi_linear_w4a8_bf16_static: group size %d, the kernels are built for 64, 128 and 256", gs);
+    CMI_REQUIRE(M <= STATIC_MAX_ROWS && (size_t)M * Kd <= STATIC_XQ_BYTES, CMI_E_UNSUPPORTED,
                 "cmi_linear_w4a8_bf16_static: M=%d x K=%d exceeds the fixed workspace (M <= %d, M*K <= %zu); "
                 "use cmi_linear_w4a8_bf16 with a workspace of cmi_linear_workspace_bytes(M, K)",
                 M, K, STATIC_MAX_ROWS, STATIC_XQ_BYTES);

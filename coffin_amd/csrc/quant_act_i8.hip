@@ -68,16 +68,17 @@ quant_act_i8_vec(const uint4 *__restrict__ x, uint2 *__restrict__ q, float *__re
     }
 }
 
-// Any K, any alignment.
+// Any K, any alignment; q rows have pitch ldq >= K and the tail K .. ldq-1 is cleared.
 __global__ void __launch_bounds__(QUANT_THREADS)
 quant_act_i8_scalar(const uint16_t *__restrict__ x, int8_t *__restrict__ q,
-                    float *__restrict__ s, int K, int *__restrict__ zero, int n_zero) {
+                    float *__restrict__ s, int K, int ldq, int *__restrict__ zero, int n_zero) {
     __shared__ float smem[QUANT_THREADS / 64];
     const int row = blockIdx.x;
     if (row == 0)
         for (int i = threadIdx.x; i < n_zero; i += QUANT_THREADS) zero[i] = 0;
     const uint16_t *xr = x + (size_t)row * K;
-    int8_t *qr = q + (size_t)row * K;
+    int8_t *qr = q + (size_t)row * ldq;
+    for (int k = K + threadIdx.x; k < ldq; k += QUANT_THREADS) qr[k] = 0;
     float amax = 0.f;
     for (int k = threadIdx.x; k < K; k += QUANT_THREADS)
         amax = fmaxf(amax, fabsf(bf16_bits_to_f32(xr[k])));
@@ -110,8 +111,18 @@ int cmi::quant_act_i8_and_clear(const void *x, int8_t *q, float *s, int M, int K
         else if (vpt <= 16) quant_act_i8_vec<16><<<grid, block, 0, st>>>(xv, qv, s, nvec, zero, n_zero);
         else quant_act_i8_vec<0><<<grid, block, 0, st>>>(xv, qv, s, nvec, zero, n_zero);
     } else {
-        quant_act_i8_scalar<<<grid, block, 0, st>>>(static_cast<const uint16_t *>(x), q, s, K, zero, n_zero);
+        quant_act_i8_scalar<<<grid, block, 0, st>>>(static_cast<const uint16_t *>(x), q, s, K, K, zero, n_zero);
     }
+    return check_launch("cmi_quant_act_i8");
+}
+
+int cmi::quant_act_i8_padded(const void *x, int8_t *q, float *s, int M, int K, int ldq, void *stream) {
+    if (ldq == K) return quant_act_i8_and_clear(x, q, s, M, K, nullptr, 0, stream);
+    CMI_REQUIRE(M >= 0 && K > 0 && ldq > K, CMI_E_ARG, "cmi_quant_act_i8: bad shape M=%d K=%d pitch=%d", M, K, ldq);
+    if (M == 0) return CMI_OK;
+    CMI_REQUIRE(x && q && s, CMI_E_ARG, "cmi_quant_act_i8: null pointer");
+    quant_act_i8_scalar<<<dim3(M), dim3(QUANT_THREADS), 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const uint16_t *>(x), q, s, K, ldq, nullptr, 0);
     return check_launch("cmi_quant_act_i8");
 }
 

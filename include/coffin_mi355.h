@@ -114,18 +114,23 @@ int cmi_linear_w8a16(const int8_t *wq, const float *ws, const void *x, void *y, 
 long long cmi_stream_capture_id(void *stream);
 
 /* One-time re-layout of a W4A8Weight for the device kernels.
- *   in : packed u8 [ceil(K/2), N] (low nibble = even k, code = q+8) and
- *        scale fp32 [K/gs, N]      (w4a8_weights.py:14-20,28-53)
- *   out: w4 u8 [N, K/2] with, inside every 32-bit word, nibble 2i = code of
+ *   in : packed u8 [ceil(Kp/2), N] (low nibble = even k, code = q+8; Kp = K rounded up to whole
+ *        groups, pad code 8) and scale fp32 [ceil(K/gs), N]   (w4a8_weights.py:14-20,28-53)
+ *   out: w4 u8 [N, Kd/2] with, inside every 32-bit word, nibble 2i = code of
  *        k0+i and nibble 2i+1 = code of k0+4+i (k0 = 8*word index), and
- *        ws fp32 [N, K/gs].
- * K % 32 == 0, gs % 32 == 0, K % gs == 0.  Plays the role of the load-time
+ *        ws fp32 [N, Kd/gs];  Kd = cmi_w4_device_k(K, gs) >= K: K rounded up to whole groups and
+ *        whole 128-element steps, the padding holding code 8 and scale 0.
+ * gs in {64, 128, 256} (else CMI_E_UNSUPPORTED), any K >= 1.  Plays the role of the load-time
  * repack a backend may do at its own cost (backends/protocol.py:118-126,
- * backends/corex/pack.py:323-359). */
+ * backends/corex/pack.py:323-359).  The kernels below that take quantised rows (cmi_gemv_w4a8,
+ * cmi_gemm_w4a8) are called with K = Kd and rows padded with zeros to Kd; the entries that take bf16
+ * rows (cmi_linear_w4a8_bf16*, cmi_embed_rows_w4) take the logical K and do that themselves. */
+int cmi_w4_device_k(int K, int gs);  /* 0 when the group size is not one the kernels take */
 int cmi_w4_repack(const uint8_t *packed, const float *scale, uint8_t *w4, float *ws,
                   int N, int K, int gs, void *stream);
 
-/* W4A8 GEMV, 1 <= M <= 16 (up to 128 when K <= 10240), on the re-laid-out weight:
+/* W4A8 GEMV, 1 <= M <= 16 (up to 128 when K <= 10240 and gs == 128), on the re-laid-out weight;
+ * K % gs == 0, gs in {64, 128, 256} (the fast kernels are built for 128, the others take a general one):
  *   sum_g = sum_{k in g} xq[m,k]*(code-8)           (int32, exact)
  *   total = fma((float)sum_g, ws[n,g], total)        (g ascending, from 0)
  *   y[m,n] = bf16(total * xs[m])
@@ -172,7 +177,8 @@ int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs, const flo
                   void *y, int32_t *acc_out, int M, int N, int K, int ldy, void *stream);
 
 /* W4A8 GEMM on the re-laid-out weight; same arithmetic as cmi_gemv_w4a8 for
- * any M.  K % 128 == 0, gs == 128.  Replaces w4a8_gemm_tcu
+ * any M.  K % 128 == 0 and K % gs == 0, gs in {64, 128, 256} (the tile-count and few-row routes
+ * are built for 128; other group sizes take the two-stage tile kernel).  Replaces w4a8_gemm_tcu
  * (backends/corex/kernels/w8a8_tcu.cu:453-574, called from
  * backends/corex/__init__.py:647). group_acc as in cmi_gemv_w4a8. */
 int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs,
@@ -188,7 +194,9 @@ int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const fl
  *   cmi_linear_w4a8_bf16: what _w4_rows issues (backends/corex/__init__.py:576-651: quant_act_i8
  *     into private scratch, then w4a8_gemv or w4a8_gemm_tcu by row count); the GEMV that
  *     quantises by itself (cmi_gemv_w4a8_bf16) is taken where it is the faster route, the GEMV
- *     entry up to 16 rows, the GEMM entry beyond. */
+ *     entry up to 16 rows, the GEMM entry beyond.  K is the logical row length (any K >= 1, gs in
+ *     {64, 128, 256}); the workspace is sized for the padded one,
+ *     cmi_linear_workspace_bytes(M, cmi_w4_device_k(K, gs)). */
 size_t cmi_linear_workspace_bytes(int M, int K);
 /* A workspace of cmi_linear_w8a8_workspace_bytes(M, N, K) bytes -- the above plus, for 17..256 rows,
  * 256 arrival counters and 8 MiB of partial tiles (16 MiB for 257..1024 rows of a projection of at
@@ -244,7 +252,7 @@ int cmi_add_rms_norm_i8(void *x, const void *add, const void *w, void *y, int8_t
 /* Embedding lookup on a quantized weight: rows `ids` (int64 [T]) dequantised to bf16 [T,K].
  *   int8: out[t,k] = bf16(float(wq[id,k]) * ws[id])         (ops/embed.py:64-81, int8_weights.py:359)
  *   int4: out[t,k] = bf16(float(code-8) * ws[id,k/gs])      (w4a8_weights.py:84-94), on the
- *         re-laid-out weight of cmi_w4_repack (gs == 128, K % 128 == 0)
+ *         re-laid-out weight of cmi_w4_repack (any K; gs in {64, 128, 256})
  * An id outside [0, N) gives a row of bf16 NaN (a device-side range error cannot be returned
  * without synchronising). */
 int cmi_embed_rows_i8(const int8_t *wq, const float *ws, const int64_t *ids, void *out, int T,

@@ -67,9 +67,11 @@ def gemm_w8a8(xq, wq, xs, ws, want_acc=True, ldy=None):
 
 
 def w4_repack(packed, scale, k, gs=128):
+    """Device layout of an int4 weight: rows of cmi_w4_device_k(k, gs) codes."""
     n = packed.shape[1]
-    w4 = torch.empty((n, k // 2), dtype=torch.uint8, device=DEV)
-    ws = torch.empty((n, k // gs), dtype=torch.float32, device=DEV)
+    kd = int(_native.load().cmi_w4_device_k(k, gs))
+    w4 = torch.empty((n, kd // 2), dtype=torch.uint8, device=DEV)
+    ws = torch.empty((n, kd // gs), dtype=torch.float32, device=DEV)
     _native.check(_native.load().cmi_w4_repack(ptr(packed), ptr(scale), ptr(w4), ptr(ws), n, k, gs,
                                                stream()), "w4_repack")
     return w4, ws

@@ -265,8 +265,9 @@ def test_w4_operands_are_checked_before_any_address_reaches_a_kernel():
             backend._w4_check(NS(**{**good, **patch}))
     # shapes the kernels are not built for are answered by the torch statement of the op
     assert backend._kernels_take(NS(**good))
-    assert not backend._kernels_take(NS(**{**good, "group_size": 64}))
-    assert not backend._kernels_take(NS(**{**good, "k": 192}))
+    assert backend._kernels_take(NS(**{**good, "group_size": 64})) and backend._kernels_take(NS(**{**good, "k": 192}))
+    assert not backend._kernels_take(NS(**{**good, "group_size": 96}))
+    assert not backend._kernels_take(NS(**{**good, "group_size": 32}))
     assert backend._kernels_take(NS(wq=torch.zeros((4, 32), dtype=torch.int8), scale=torch.ones(4)))
     assert not backend._kernels_take(NS(wq=torch.zeros((4, 24), dtype=torch.int8), scale=torch.ones(4)))
 
@@ -381,11 +382,16 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     assert "outside 1..16" in _native.last_error()
     assert lib.cmi_gemv_w8a16(one, one, one, one, 1, 8, 24, null) == _native.E_UNSUPPORTED
     assert lib.cmi_gemv_w8a16(ctypes.c_void_p(8), one, one, one, 1, 8, 16, null) == _native.E_ARG
-    assert lib.cmi_gemv_w4a8(one, one, one, one, one, null, 1, 8, 256, 64, null) == _native.E_UNSUPPORTED
+    assert lib.cmi_gemv_w4a8(one, one, one, one, one, null, 1, 8, 256, 96, null) == _native.E_UNSUPPORTED
+    assert "64, 128 and 256" in _native.last_error()
     assert lib.cmi_gemv_w4a8(one, one, one, one, one, null, 1, 8, 192, 128, null) == _native.E_UNSUPPORTED
+    assert lib.cmi_gemv_w4a8(one, one, one, one, one, null, 1, 8, 320, 256, null) == _native.E_UNSUPPORTED
     assert lib.cmi_gemm_w8a8(one, one, one, one, one, null, 4, 8, 64, 4, null) == _native.E_ARG
     assert "ldy" in _native.last_error()
     assert lib.cmi_gemm_w4a8(one, one, one, one, one, null, 4, 8, 200, 128, null) == _native.E_UNSUPPORTED
-    assert lib.cmi_w4_repack(one, one, one, one, 8, 100, 128, null) == _native.E_UNSUPPORTED
+    assert lib.cmi_gemm_w4a8(one, one, one, one, one, null, 4, 8, 256, 32, null) == _native.E_UNSUPPORTED
+    assert lib.cmi_w4_repack(one, one, one, one, 8, 100, 96, null) == _native.E_UNSUPPORTED
+    assert [lib.cmi_w4_device_k(k, gs) for k, gs in ((200, 128), (200, 64), (200, 256), (2560, 128), (2561, 64),
+                                                      (300, 256), (128, 32), (0, 128))] == [256, 256, 256, 2560, 2688, 512, 0, 0]
     with pytest.raises(ValueError, match="cmi_gemv_w8a16"):
         _native.check(lib.cmi_gemv_w8a16(one, one, one, one, 0, 8, 16, null), "gemv")
