@@ -157,6 +157,10 @@ def parse_args():
                          "for that kernel; prints its own JSON line")
     ap.add_argument("--prequantised", action="store_true",
                     help="with --w4a8-decode-only: activations arrive as int8 rows + scales")
+    ap.add_argument("--table-entries", action="store_true",
+                    help="with --w4a8-decode-only: drive the step through the table entries of the backend "
+                         "(rms_norm / add_rms_norm / silu_mul in front of linear), with and without the "
+                         "producers handing over their quantised rows")
     ap.add_argument("--w4a8-decode-only", action="store_true",
                     help="time only the W4A8 decode step (32 layers + lm_head at one row, one "
                          "cmi_linear_w4a8_bf16 call per projection): the profiling target for the W4A8 decode "
@@ -321,6 +325,79 @@ def main() -> int:
                              "avg_projection_us": round(t / len(proj) * 1e6, 3),
                              "algorithmic_bytes_per_projection": round(alg / len(proj))}}
 
+    def w4a8_step_through_table_entries(rows: int, iters: int):
+        """The W4A8 decode step driven the way the reference drives it, through the table entries of
+        coffin_amd.backend: per layer rms_norm -> linear(qkv), linear(o) on plain bf16 rows (the
+        attention output: no producer of this backend in front of it), add_rms_norm -> linear(gate_up),
+        silu_mul -> linear(down); rms_norm -> linear(lm_head) at the end (ops/norm.py:87,135,
+        models/qwen35/blocks.py:69,97, ops/gemv.py:75,93).  Captured in a graph.  Measured with the
+        producers handing their quantised rows to the projection behind them and without, and the
+        producers alone (97 launches), so that "projections only" = sequence - producers."""
+        from coffin_amd import backend as B
+        from coffin_amd.weights import W4A8Weight as W4
+        layers = []
+        for _ in range(LAYERS):
+            ws = []
+            for _, n_, k_ in synth.DECODE_LAYER_FUSED:
+                w = synth.int4_weight(n_, k_, gen)
+                ws.append(W4(w.packed, w.scale, k=k_))
+            layers.append(ws)
+        _, n_, k_ = synth.LM_HEAD
+        w = synth.int4_weight(n_, k_, gen)
+        head = W4(w.packed, w.scale, k=k_)
+        hidden, inter = 2560, 9728
+        gain = (1.0 + 0.1 * torch.randn(hidden, generator=gen, device=dev)).to(torch.bfloat16)
+        resid = synth.activations(rows, hidden, gen)
+        attn = synth.activations(rows, 4096, gen)
+        mix = synth.activations(rows, hidden, gen)
+        normed = torch.empty((rows, hidden), dtype=torch.bfloat16, device=dev)
+        gu_fixed = synth.activations(rows, 2 * inter, gen)
+        one = rows == 1
+        proj = B.linear if one else B.linear_m
+
+        def row(t):                                   # a single sequence hands [K] to linear, as ops/gemv.py:75 does
+            return t.view(-1) if one else t
+
+        def sequence(projections: bool = True):
+            x = resid.clone()
+            for qkv, o, gate_up, down in layers:
+                h = B.rms_norm(x, gain)
+                if projections:
+                    proj(qkv, row(h))
+                    proj(o, row(attn))
+                B.add_rms_norm(x, mix, gain, normed)
+                gu = proj(gate_up, row(normed)) if projections else row(gu_fixed)
+                gate, up = (gu[:inter], gu[inter:]) if one else (gu[:, :inter], gu[:, inter:])
+                act = B.silu_mul(gate, up, up)
+                if projections:
+                    proj(down, act)
+            h = B.rms_norm(x, gain)
+            if projections:
+                proj(head, row(h))
+
+        out = {"rows": rows}
+        alg = sum(synth.w4_gemv_bytes(rows, w_.n, w_.k) for ws in layers for w_ in ws) + synth.w4_gemv_bytes(rows, head.n, head.k)
+        for label, handover, projections in (("handed_rows", True, True), ("bf16_rows", False, True),
+                                             ("producers_only", False, False)):
+            B.configure(handover=handover)
+            sequence(projections)                     # warm-up: re-layouts, scratch, the consumer-seen flag
+            sequence(projections)
+            torch.cuda.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr):
+                sequence(projections)
+            t = timed(gr.replay, iters, warm=2)
+            out[label + "_ms"] = round(t * 1e3, 4)
+            del gr
+        B.configure(handover=True)
+        for label in ("handed_rows", "bf16_rows"):
+            t = (out[label + "_ms"] - out["producers_only_ms"]) * 1e-3
+            out[label + "_projections_only_ms"] = round(t * 1e3, 4)
+            out[label + "_projections_only_GBps"] = round(alg / t / 1e9, 1)
+        out["launches"] = {"projections": 4 * LAYERS + 1, "producers": 3 * LAYERS + 1}
+        out["algorithmic_bytes_of_the_projections"] = alg
+        return out
+
     if args.quant_only:
         out = {}
         for m, k_ in ((8192, 2560), (2048, 9728), (16, 9728), (1, 2560)):
@@ -334,6 +411,11 @@ def main() -> int:
         print(json.dumps({"metric": "per-token int8 quantiser HBM GB/s", "unit": "GB/s", "quant_act_i8": out}))
         return 0
 
+    if args.w4a8_decode_only and args.table_entries:
+        print(json.dumps({"metric": "W4A8 decode step through the table entries", "unit": "ms",
+                          "w4a8_decode_step": {f"M{args.rows}_through_table_entries":
+                                               w4a8_step_through_table_entries(args.rows, args.steps)}}))
+        return 0
     if args.w4a8_decode_only:
         key = f"M{args.rows}" + ("_prequantised" if args.prequantised else "")
         out = {key: w4a8_decode_step(args.rows, not args.no_graph, args.steps, args.prequantised)}
@@ -460,10 +542,22 @@ def main() -> int:
             t = timed(r, max(3, args.steps // 2), warm=2)
             extra[f"decode_gemv_int8_M{m}_GBps"] = round(step_bytes(m) / t / 1e9, 1)
         # the same step through the matrix-pipe GEMV (linear_m_verify, short linear_prefill chunks)
-        for m in (4, 8, 16):
+        family = {"dot": {}, "mfma": {}}
+        for m in (1, 4, 8, 16):
             r, _ = make_runner(m, True)
             t = timed(r, max(3, args.steps // 2), warm=2)
-            extra[f"verify_gemv_int8_mfma_M{m}_GBps"] = round(step_bytes(m) / t / 1e9, 1)
+            if m > 1:
+                extra[f"verify_gemv_int8_mfma_M{m}_GBps"] = round(step_bytes(m) / t / 1e9, 1)
+            family["mfma"][f"M{m}"] = {"ms_per_step": round(t * 1e3, 4), "GBps": round(step_bytes(m) / t / 1e9, 1),
+                                       "frac_of_hbm_peak": round(step_bytes(m) / t / 1e9 / HBM_PEAK_GBPS, 4)}
+            g_ = extra[f"decode_gemv_int8_M{m}_GBps"]
+            family["dot"][f"M{m}"] = {"ms_per_step": round(step_bytes(m) / g_ / 1e6, 4), "GBps": g_,
+                                      "frac_of_hbm_peak": round(g_ / HBM_PEAK_GBPS, 4)}
+        # Static-batch decode owes "row r of a batch == the single-row call" (models/qwen35/batch.py:19-22),
+        # which holds inside either kernel family as long as every call on a weight uses the same one
+        # (coffin_amd.backend.configure(batch_family=...), or the weight's batch_family attribute): the
+        # whole decode step at 1 / 4 / 8 / 16 rows in both, so the trade is a measured table.
+        extra["static_batch_decode_by_family"] = family
         # per-shape kernel time, weights rotated through > 1 GB so HBM serves them
         per_shape = {}
         for name, n_, k_ in shapes + [synth.LM_HEAD]:
@@ -476,6 +570,40 @@ def main() -> int:
             per_shape[name] = {"us": round(t * 1e6, 2),
                                "GBps": round(synth.gemv_bytes(1, n_, k_) / t / 1e9, 1)}
         extra["decode_gemv_int8_M1_per_shape_eager"] = per_shape
+
+        # What each projection costs the replayed step: per shape, the same launches as a dependent
+        # chain of their own in a captured graph (the 32 layers' weights of that shape, cold; four
+        # copies of lm_head), time / launches = start-to-start interval of that shape in steady
+        # state.  A kernel trace cannot show this: the profiler serialises dispatches and adds about
+        # 3 us between them (the traced step takes 1.2 ms).  The intervals, weighted by how often
+        # each shape occurs, must add up to ms_per_step.
+        if M == 1 and not args.no_graph and not args.mfma:
+            chain = {}
+            total = 0.0
+            for name, n_, k_ in shapes + [synth.LM_HEAD]:
+                group = [l for l in launches if (l[4], l[5]) == (n_, k_)]
+                count = len(group)
+                extra_w = []
+                if count < 4:   # lm_head: one weight in the model; three more so that none is answered from cache
+                    extra_w = [synth.int8_weight(n_, k_, gen) for _ in range(3)]
+                    group = group + [(q_.wq, q_.scale, group[0][2], group[0][3], n_, k_) for q_ in extra_w]
+                def one(group=group):
+                    st = cur_stream()
+                    for wq, sc, x, y, nn, kk in group:
+                        lib.cmi_gemv_w8a16(ptr(wq), ptr(sc), ptr(x), ptr(y), 1, nn, kk, st)
+                one()
+                torch.cuda.synchronize()
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr):
+                    one()
+                t = timed(gr.replay, 10, warm=3) / len(group)
+                chain[name] = {"interval_us": round(t * 1e6, 3), "per_step": count,
+                               "GBps": round(synth.gemv_bytes(1, n_, k_) / t / 1e9, 1)}
+                total += count * t
+                del gr, extra_w
+            chain["sum_of_intervals_ms"] = round(total * 1e3, 4)
+            chain["ms_per_step"] = round(step_s * 1e3, 4)
+            extra["decode_gemv_int8_M1_per_shape_hipgraph_chain"] = chain
 
         # the same 129 projections through the table entry (backend.linear: Python adapter + ctypes +
         # a fresh output tensor per call), eager and as a captured graph: what the host side costs
@@ -532,6 +660,9 @@ def main() -> int:
         torch.cuda.empty_cache()
         extra["w4a8_decode_step"]["M16_prequantised"] = w4a8_decode_step(16, True, max(3, args.steps // 2), True)
         torch.cuda.empty_cache()
+        for m in (1, 16):
+            extra["w4a8_decode_step"][f"M{m}_through_table_entries"] = w4a8_step_through_table_entries(m, max(3, args.steps // 2))
+            torch.cuda.empty_cache()
 
         # W4A8 decode GEMV (quantiser + GEMV, as the adapter issues them)
         w4 = {}

@@ -93,6 +93,13 @@ MFMA_MIN_ROWS = 3
 HANDOVER = os.environ.get("COFFIN_AMD_HANDOVER", "1").strip() != "0"
 #: Largest block of rows (bytes of int8) a producer leaves behind.
 HANDOVER_MAX_BYTES = 128 << 20
+#: Fewest rows a producer hands over.  A single row is not worth it: at one row every kernel here
+#: runs at its launch floor, quantising costs about 1 us wherever it is done (a second
+#: workgroup-wide reduction in the producer: rms_norm 2.6 -> 3.6 us, silu_mul 2.9 -> 4.6 us), and the
+#: one-row GEMVs that quantise for themselves lose only 0.4 / 1.1 / 1.9 us to it (qkv / gate_up /
+#: down): the 129-projection step measured 1.042 ms handed against 1.058 ms not.  From two rows up
+#: the projection would otherwise launch the quantiser in front of its kernel (2.5 .. 4 us).
+HANDOVER_MIN_ROWS = 2
 
 _FAMILIES = {"dot": 0, "mfma": 1}
 
@@ -359,7 +366,7 @@ def _capture_id(stream: int) -> int:
 def _hand_target(rows: int, k: int, device: torch.device):
     """``(xq address, xs address)`` for a producer of ``rows x k`` outputs, or ``None`` when it
     should not leave quantised rows behind."""
-    if not (HANDOVER and _QUANT_CONSUMER_SEEN) or rows <= 0 or rows * k > HANDOVER_MAX_BYTES:
+    if not (HANDOVER and _QUANT_CONSUMER_SEEN) or rows < HANDOVER_MIN_ROWS or rows * k > HANDOVER_MAX_BYTES:
         return None
     try:
         base = _HANDOVER_ARENA.take(_round256(rows * k) + _round256(4 * rows), device)

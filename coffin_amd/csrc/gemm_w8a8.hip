@@ -87,6 +87,7 @@ struct Cfg {
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     if constexpr (N == 0) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    else if constexpr (N == 3) asm volatile("s_waitcnt vmcnt(3) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 4) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 6) asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)" ::: "memory");
     else if constexpr (N == 8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
@@ -818,6 +819,288 @@ int launch_wide(Args &a, hipStream_t st) {
     return check_launch("cmi_gemm_w8a8");
 }
 
+// ---------------------------------------------------------------------------
+// The same 256(m) x 320(n) tile walked weight tile by weight tile inside a K step, so that a
+// stage is handed back in pieces and its next contents are in flight for about a step and a half
+// instead of one step.  The two-stage kernel above reads every row of a stage in each of the
+// four k quarters, so nothing of a stage is free before the step's last quarter and a stage's 72 KiB
+// are requested one step (about 1.2 us of MFMAs) before they are needed.  Here a wavefront keeps the
+// step's activation fragments in registers (8 x 16 bytes, all four quarters) and goes through its
+// five 32-row weight tiles one after the other, in ten "half groups" of 4 MFMAs (weight tile I,
+// k quarters 2H and 2H+1, against both activation tiles): the activation rows of a stage and weight
+// tiles 0, 1 are free three tenths into the step, tiles 2..4 nine tenths.  Two barriers per step
+// (A in half group 3, B in half group 9) hand the freed rows to the requests of step ks+2:
+//     A(ks): X(ks+2), W tiles 0, 1 (ks+2)      B(ks): W tiles 2..4 (ks+2)
+// and certify what the next reads need: at B(ks) every wavefront's share of X(ks+1) and W 0, 1
+// (ks+1) has landed (requested at A(ks-1)), at A(ks) W 2..4 (ks) (requested at B(ks-2)); a
+// wavefront requests 6 + 3 loads per step, so both waits are vmcnt(9).
+//
+// Fragment reads are issued where the compiler does not see them (inline ds_read_b128) and
+// waited for with exact counts: left to itself the compiler drains the LDS queue (lgkmcnt(0)) in
+// front of every use, so a read never has more than the few MFMAs between it and its use to
+// land -- measured 12 us of a 50 us launch.  Here the fragments of half group k+2 are read during
+// half group k into one of three fragment buffers (LDS returns in order, so the wait in front of
+// half group k is "all but the reads issued since": lgkmcnt(2)), except where the data is
+// certified only at a barrier (half groups 4 and 5 are read together behind A, 0 and 1 of the next
+// step behind B).  Which buffer a half group uses is a fixed table per step parity, chosen so that
+// a read never lands in a buffer that a pending half group still needs.
+// Requests are buffer loads (buffer_load_dwordx4 ... lds): one 32-bit lane offset per operand, the
+// tile / step / row-group offset in a scalar register, rows past the matrix read as zeros.
+// Same MFMAs on the same operands per accumulator, in the same k order: the accumulators, and so
+// the bits, are those of the two-stage kernel.
+namespace tilewise {
+// fragment buffer of half group k in a step of parity P
+constexpr int BUF[2][10] = {{0, 2, 1, 0, 2, 1, 0, 2, 1, 0}, {1, 2, 0, 1, 2, 0, 1, 2, 0, 1}};
+__device__ __forceinline__ uint32_t lds_offset(const void *p) { return (uint32_t)(uintptr_t)(lds_ptr_t)p; }
+template <int IMM>
+__device__ __forceinline__ void read16(v4i32 &d, uint32_t base) {
+    static_assert(IMM >= 0 && IMM < 65536, "LDS immediate offset");
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(d) : "v"(base), "n"(IMM) : "memory");
+}
+// the registers named are not used before the LDS queue is down to N reads
+template <int N>
+__device__ __forceinline__ void lds_wait(v4i32 &f0, v4i32 &f1) {
+    if constexpr (N == 0) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f0), "+v"(f1)::"memory");
+    else if constexpr (N == 2) asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(f0), "+v"(f1)::"memory");
+    else static_assert(N < 0, "add the lgkmcnt literal");
+}
+template <int N>
+__device__ __forceinline__ void lds_wait(v4i32 &f0, v4i32 &f1, v4i32 &x0, v4i32 &x1, v4i32 &x2, v4i32 &x3) {
+    if constexpr (N == 2)
+        asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(f0), "+v"(f1), "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3)::"memory");
+    else if constexpr (N == 6)
+        asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(f0), "+v"(f1), "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3)::"memory");
+    else static_assert(N < 0, "add the lgkmcnt literal");
+}
+}  // namespace tilewise
+
+__global__ void __launch_bounds__(512, 2)
+gemm_w8a8_wide_tilewise_kernel(const Args a) {
+    using namespace wide;
+    using namespace tilewise;
+    extern __shared__ __align__(16) int8_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wn = wave & 1, wm = wave >> 1;
+
+    int tm, tn;
+    tile_coords(a, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    float *scales = reinterpret_cast<float *>(lds + OPERAND_BYTES);
+    stage_scales<BN, BM>(a, scales, n0, m0);
+
+    // LDS: weights as [n half][stage][160 rows], activations behind them as [m quarter][stage][64 rows],
+    // so that both stages of a wavefront's rows are within the 64 KiB reach of an LDS instruction's
+    // immediate offset and one base register per k quarter serves a whole operand.
+    constexpr int W_HALF = 160 * BK, X_QUARTER = 64 * BK, X_BASE = 4 * W_HALF;
+    // Requests.  Weight tile i of n half h is rows 160 h + 32 i .. + 31; its 64 rows (both halves)
+    // are 8 loads of 8 rows, one per wavefront: wavefront w takes rows 160 (w & 1) + 32 i + 8 (w >> 1)
+    // .. + 7.  X rows 32 w + 8 g .. + 7, g = 0..3.  Lane i of a load lands in slot i of the 1 KiB:
+    // row i / 8, stored chunk i % 8, which holds k chunk (i % 8) ^ ((row / 2) % 8).
+    const int lrow = lane >> 3;
+    const int wrow = wn * 160 + wm * 8 + lrow;  // + 32 i: the swizzle does not depend on i
+    const uint32_t wvoff = (uint32_t)wrow * (uint32_t)a.K + (((lane & 7) ^ ((wrow >> 1) & 7)) * 16);
+    const int xrow = XL * wave * 8 + lrow;      // + 8 g: odd g flip bit 2 of the swizzle
+    uint32_t xvoff[2];
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+        xvoff[g] = (uint32_t)xrow * (uint32_t)a.K + (((lane & 7) ^ (((xrow + 8 * g) >> 1) & 7)) * 16);
+    const __amdgpu_buffer_rsrc_t wres =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(a.wq), 0, (int)((size_t)a.N * a.K), 0x00020000);
+    const __amdgpu_buffer_rsrc_t xres =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(a.xq), 0, (int)((size_t)a.M * a.K), 0x00020000);
+    const uint32_t wtile = (uint32_t)n0 * (uint32_t)a.K, xtile = (uint32_t)m0 * (uint32_t)a.K;
+    const uint32_t k32 = 32u * (uint32_t)a.K, k8 = 8u * (uint32_t)a.K;
+    int8_t *const wslot = lds + wn * 2 * W_HALF + wm * 8 * BK;                              // weight tile 0, stage 0
+    int8_t *const xslot = lds + X_BASE + (wave >> 1) * 2 * X_QUARTER + (wave & 1) * 4 * 1024;  // g = 0, stage 0
+    auto issue_w = [&](int stage, int ks, int i) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(wres, (lds_ptr_t)(wslot + stage * W_HALF + i * 32 * BK), 16, wvoff,
+                                                 wtile + i * k32 + ks * BK, 0, 0);
+    };
+    auto issue_a = [&](int stage, int ks) {
+#pragma unroll
+        for (int g = 0; g < XL; ++g)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(xres, (lds_ptr_t)(xslot + stage * X_QUARTER + g * 1024), 16,
+                                                     xvoff[g & 1], xtile + g * k8 + ks * BK, 0, 0);
+        issue_w(stage, ks, 0);
+        issue_w(stage, ks, 1);
+    };
+    auto issue_b = [&](int stage, int ks) {
+        issue_w(stage, ks, 2);
+        issue_w(stage, ks, 3);
+        issue_w(stage, ks, 4);
+    };
+
+    // Fragment reads: lane reads row (lane % 32) of a 32-row MFMA tile; for k quarter q its 16 bytes
+    // are k chunk 2q + lane / 32 (swizzled).  One base per quarter and operand, the rest immediates.
+    const int frow = lane & 31;
+    const int fsw = (frow >> 1) & 7;
+    uint32_t wbase[4], xbase[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int foff = frow * BK + ((2 * q + (lane >> 5)) ^ fsw) * 16;
+        wbase[q] = lds_offset(lds + wn * 2 * W_HALF) + foff;
+        xbase[q] = lds_offset(lds + X_BASE + wm * 2 * X_QUARTER) + foff;
+    }
+    v4i32 xf[TM][4];  // the step's activation fragments, all four k quarters
+    v4i32 wf[3][2];   // two k quarters of one weight tile, three buffers
+    using std::integral_constant;
+#define IC(v) integral_constant<int, (v)>{}
+    // fragments of half group K of a step of parity P (its operands are in stage P)
+    auto read_w = [&](auto parity_tag, auto hg_tag) {
+        constexpr int P = decltype(parity_tag)::value, K = decltype(hg_tag)::value, I = K / 2, H = K % 2;
+        read16<P * W_HALF + I * 32 * BK>(wf[BUF[P][K]][0], wbase[2 * H]);
+        read16<P * W_HALF + I * 32 * BK>(wf[BUF[P][K]][1], wbase[2 * H + 1]);
+    };
+    // activation quarters 2H, 2H+1 of a step of parity P
+    auto read_x = [&](auto parity_tag, auto half_tag) {
+        constexpr int P = decltype(parity_tag)::value, H = decltype(half_tag)::value;
+#pragma unroll
+        for (int q = 2 * H; q < 2 * H + 2; ++q) {
+            read16<P * X_QUARTER>(xf[0][q], xbase[q]);
+            read16<P * X_QUARTER + 32 * BK>(xf[1][q], xbase[q]);
+        }
+    };
+
+    v16i32 acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+    // the 4 MFMAs of half group K in a step of parity P
+    auto mma = [&](auto parity_tag, auto hg_tag) {
+        constexpr int P = decltype(parity_tag)::value, K = decltype(hg_tag)::value, I = K / 2, H = K % 2;
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+#pragma unroll
+            for (int j = 0; j < TM; ++j)
+                acc[I][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[BUF[P][K]][q], xf[j][2 * H + q], acc[I][j], 0, 0, 0);
+    };
+    // the wait in front of half group K: N reads were issued after its fragments
+    auto wait_w = [&](auto parity_tag, auto hg_tag, auto n_tag) {
+        constexpr int P = decltype(parity_tag)::value, K = decltype(hg_tag)::value, N = decltype(n_tag)::value;
+        lds_wait<N>(wf[BUF[P][K]][0], wf[BUF[P][K]][1]);
+    };
+    auto wait_wx = [&](auto parity_tag, auto hg_tag, auto n_tag) {
+        constexpr int P = decltype(parity_tag)::value, K = decltype(hg_tag)::value, N = decltype(n_tag)::value, H = K % 2;
+        lds_wait<N>(wf[BUF[P][K]][0], wf[BUF[P][K]][1], xf[0][2 * H], xf[1][2 * H], xf[0][2 * H + 1], xf[1][2 * H + 1]);
+    };
+    auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
+
+    const int ksteps = a.K / BK;
+    // One K step from stage P = ks & 1.  On entry the fragments of half groups 0 and 1 are on their
+    // way (12 reads, issued in that order).  The last two steps request the last step's operands once
+    // more instead of nothing (into rows that are free, nobody reads them): every step then issues the
+    // same 9 loads and both vmcnt waits are 9 throughout.
+    auto step = [&](auto p, int ks) {
+        constexpr int P = decltype(p)::value;
+        constexpr auto np = IC(P ^ 1);
+        const int ahead = min(ks + 2, ksteps - 1);
+        wait_wx(p, IC(0), IC(6));
+        mma(p, IC(0));
+        read_w(p, IC(2));
+        fence();
+        wait_wx(p, IC(1), IC(2));
+        mma(p, IC(1));
+        read_w(p, IC(3));
+        fence();
+        wait_w(p, IC(2), IC(2));
+        mma(p, IC(2));
+        fence();
+        // A: X and weight tiles 0, 1 of this stage are in registers everywhere; tiles 2..4 have landed
+        wait_w(p, IC(3), IC(0));
+        asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        issue_a(P, ahead);
+        read_w(p, IC(4));
+        read_w(p, IC(5));
+        mma(p, IC(3));
+        fence();
+        wait_w(p, IC(4), IC(2));
+        mma(p, IC(4));
+        read_w(p, IC(6));
+        fence();
+        wait_w(p, IC(5), IC(2));
+        mma(p, IC(5));
+        read_w(p, IC(7));
+        fence();
+        wait_w(p, IC(6), IC(2));
+        mma(p, IC(6));
+        read_w(p, IC(8));
+        fence();
+        wait_w(p, IC(7), IC(2));
+        mma(p, IC(7));
+        read_w(p, IC(9));
+        fence();
+        wait_w(p, IC(8), IC(2));
+        mma(p, IC(8));
+        fence();
+        // B: weight tiles 2..4 are in registers everywhere; X and tiles 0, 1 of the next step have landed
+        wait_w(p, IC(9), IC(0));
+        asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        issue_b(P, ahead);
+        // the next step's first fragments (past the last step: a stale stage, nobody uses them);
+        // its quarters 2, 3 of X replace the ones this half group still multiplies, so they follow it
+        read_w(np, IC(0));
+        read_x(np, IC(0));
+        fence();
+        mma(p, IC(9));
+        fence();
+        read_w(np, IC(1));
+        read_x(np, IC(1));
+        fence();
+    };
+
+    // Prologue: both stages requested in the order the steps request them (A then B).
+    issue_a(0, 0);
+    issue_b(0, 0);
+    issue_a(1, min(1, ksteps - 1));
+    issue_b(1, min(1, ksteps - 1));
+    asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    read_w(IC(0), IC(0));
+    read_x(IC(0), IC(0));
+    read_w(IC(0), IC(1));
+    read_x(IC(0), IC(1));
+    fence();
+    int ks = 0;
+    for (; ks + 1 < ksteps; ks += 2) {
+        step(IC(0), ks);
+        step(IC(1), ks + 1);
+    }
+    if (ks < ksteps) step(IC(0), ks);
+    // the stale fragment reads and the repeated requests of the last steps must be over before their
+    // registers and the stages are used for anything else
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    fence();
+#undef IC
+
+    epilogue<TN, TM, 1>(a, acc, lds, wave, lane, n0 + wn * 32 * TN, m0 + wm * 32 * TM, scales + wn * 32 * TN,
+                        scales + BN + wm * 32 * TM);
+}
+
+int launch_wide(Args &a, hipStream_t st);
+
+int launch_wide_tilewise(Args &a, hipStream_t st) {
+    // buffer offsets are 32 bits: matrices (and the tile rows past their end) must stay below 2 GiB
+    if ((size_t)(a.N + wide::BN) * a.K >= ((size_t)1 << 31) || (size_t)(a.M + wide::BM) * a.K >= ((size_t)1 << 31))
+        return launch_wide(a, st);
+    a.tiles_m = (a.M + wide::BM - 1) / wide::BM;
+    a.tiles_n = (a.N + wide::BN - 1) / wide::BN;
+    static std::atomic<uint64_t> devices{0};
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_wide_tilewise_kernel),
+                                   wide::LDS_BYTES, devices, "cmi_gemm_w8a8"))
+        return rc;
+    gemm_w8a8_wide_tilewise_kernel<<<dim3(a.tiles_m * a.tiles_n), dim3(512), wide::LDS_BYTES, st>>>(a);
+    return check_launch("cmi_gemm_w8a8");
+}
+
 }  // namespace
 
 extern "C" int cmi_gemm_w8a8(const int8_t *xq, const int8_t *wq, const float *xs, const float *ws,
@@ -1000,6 +1283,7 @@ int cmi::gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, co
             }
         }
     }
+    if (pick == 321) return launch_wide_tilewise(a, st);
     if (pick == 320) return launch_wide(a, st);
     if (pick == 256) return launch_big(a, st);
     if (pick == 192) return launch<3, 2, 3>(a, st);

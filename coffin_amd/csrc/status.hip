@@ -55,7 +55,7 @@ std::atomic<int> g_gemv_wholerow{UNREAD};  // -1 = the library chooses, 0 = neve
 std::atomic<int> g_w4_decode_waves{0};     // 0 = the library chooses, 4 or 16 wavefronts per workgroup
 std::atomic<int> g_w4_decode_chain{0};     // 0 = the library chooses, 1 = never, else a variant code
 
-bool valid_gemm_tile(int v) { return v == 0 || v == 64 || v == 128 || v == 256 || v == 192 || v == 320 || v == 6464 || v == 128192; }
+bool valid_gemm_tile(int v) { return v == 0 || v == 64 || v == 128 || v == 256 || v == 192 || v == 320 || v == 321 || v == 6464 || v == 128192; }
 bool valid_wholerow(int v) { return v >= -1 && v <= 1; }
 
 int from_env(const char *name, int fallback, bool (*valid)(int)) {

@@ -494,6 +494,7 @@ def test_table_entry_sequence_hands_quantised_rows_to_the_projection(monkeypatch
         return outs
 
     gu0 = gu.clone()                           # silu_mul overwrites the `up` half in place
+    monkeypatch.setattr(backend, "HANDOVER_MIN_ROWS", 1)   # the mechanism at every row count (default: from 2 rows)
     monkeypatch.setattr(backend, "HANDOVER", False)
     want = sequence()
     monkeypatch.setattr(backend, "HANDOVER", True)
@@ -541,6 +542,10 @@ def test_handed_rows_are_not_trusted_after_the_tensor_changed(monkeypatch):
     backend.silu_mul_quant(gate, x, h, q, s)
     assert (backend.linear_m(w4, h).view(torch.int16) == fresh(h).view(torch.int16)).all()
     assert len(calls) == 2
+    # a single row is not handed by default (quantising costs the producer what it saves the projection)
+    one = backend.rms_norm(x[:1], gain)
+    backend.linear(w4, one[0])
+    assert len(calls) == 2 and backend._HANDED is None
     # switched off, nothing is handed
     backend.configure(handover=False)
     try:

@@ -290,7 +290,7 @@ def test_sixteen_row_kernels_at_lm_head_size_sampled_columns(orc):
 
 # ------------------------------------------------------------------ W8A8 GEMM
 
-@pytest.fixture(params=["auto", "64", "128", "192", "128192", "256", "320", "6464"])
+@pytest.fixture(params=["auto", "64", "128", "192", "128192", "256", "320", "321", "6464"])
 def gemm_tile(request):
     """Force the 128 x 64, 128 x 128, 128 x 192, 192 x 128, 256 x 256, 256 x 320 or 64 x 64 (m x n) block-tile kernel through
     cmi_set_option, or leave the choice to the library (conftest resets it after each test)."""
@@ -614,7 +614,7 @@ def test_random_shapes_and_forced_tiles_against_the_oracle(orc):
         k = step * pick((1, 9), (9, 41), (41, 11008 // step + 1))
         while m * n * k > 2e9:
             m = max(1, m // 2)
-        tile = int(rnd.choice([0, 0, 0, 64, 128, 192, 128192, 256, 320, 6464]))
+        tile = int(rnd.choice([0, 0, 0, 64, 128, 192, 128192, 256, 320, 321, 6464]))
         want_acc = bool(rnd.randint(2))
         what = (case, kind, m, n, k, tile, want_acc)
         x = synth.activations(m, k, g, outliers=bool(rnd.randint(2)))
@@ -727,7 +727,7 @@ def test_entry_points_raise_on_unsupported_shapes():
     with pytest.raises(ValueError, match="group size"):
         G.w4a8(torch.zeros((8, 128), dtype=torch.uint8, device=G.DEV), torch.ones((8, 4), device=G.DEV),
                torch.zeros((1, 256), dtype=torch.int8, device=G.DEV), torch.ones(1, device=G.DEV),
-               256, gemm=False, gs=64)
+               256, gemm=False, gs=96)
 
 
 # ------------------------------------------------------ seeded random shape sweep
