@@ -168,6 +168,11 @@ def parse_args():
     ap.add_argument("--quant-only", action="store_true",
                     help="time only the per-token quantiser (8192 x 2560, 2048 x 9728, 16 x 9728 and 1 x 2560 rows): "
                          "the profiling target for quant_act_i8; prints its own JSON line")
+    ap.add_argument("--tile-choice-check", action="store_true",
+                    help="W8A8 GEMM: time the library's own kernel choice against every forced block tile on cold "
+                         "weights over a set of layer shapes and batch sizes; prints the regret per shape.  The "
+                         "choice is made by cost models fitted to this machine: run this after a driver, "
+                         "compiler or clock change to see whether they still hold")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one 256 MiB device-to-device copy (known traffic, for scaling HBM counters)")
     return ap.parse_args()
@@ -218,6 +223,47 @@ def main() -> int:
         dst.copy_(src)          # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
+
+    if args.tile_choice_check:
+        tiles = (64, 128, 192, 128192, 256, 320, 321, 6464)
+        shapes_ = [(m, n_, k_) for (n_, k_) in ((9728, 2560), (4096, 2560), (2560, 9728), (6144, 2560), (2560, 4096))
+                   for m in (64, 256, 512, 2048, 8192)]
+        rows_, worst, sum_auto, sum_best = {}, 0.0, 0.0, 0.0
+        for m, n_, k_ in shapes_:
+            x = synth.activations(m, k_, gen, outliers=True)
+            xq = torch.empty((m, k_), dtype=torch.int8, device=dev)
+            xs = torch.empty(m, dtype=torch.float32, device=dev)
+            y = torch.empty((m, n_), dtype=torch.bfloat16, device=dev)
+            lib.cmi_quant_act_i8(ptr(x), ptr(xq), ptr(xs), m, k_, cur_stream())
+            copies = min(24, -(-600_000_000 // (n_ * k_)))
+            cold_w = [synth.int8_weight(n_, k_, gen) for _ in range(copies)]
+            def cold():
+                st = cur_stream()
+                for c in cold_w:
+                    lib.cmi_gemm_w8a8(ptr(xq), ptr(c.wq), ptr(xs), ptr(c.scale), ptr(y), vp(0), m, n_, k_, n_, st)
+            t_by = {}
+            for tile in (0,) + tiles:
+                if lib.cmi_set_option(b"gemm_tile", tile):
+                    continue
+                cold()
+                torch.cuda.synchronize()
+                g_ = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g_):
+                    cold()
+                t_by[tile] = timed(g_.replay, 3, warm=1) / copies * 1e6
+                del g_
+            lib.cmi_set_option(b"gemm_tile", 0)
+            best = min((t, tl) for tl, t in t_by.items() if tl)
+            regret = t_by[0] / best[0] - 1.0
+            worst, sum_auto, sum_best = max(worst, regret), sum_auto + t_by[0], sum_best + best[0]
+            rows_[f"M{m}_N{n_}_K{k_}"] = {"auto_us": round(t_by[0], 2), "best_forced_us": round(best[0], 2),
+                                        "best_forced_tile": best[1], "regret": round(regret, 4)}
+            del cold_w
+        print(json.dumps({"metric": "W8A8 GEMM kernel choice against the best forced tile (cold weights)", "unit": "us",
+                          "total_auto_us": round(sum_auto, 1), "total_best_forced_us": round(sum_best, 1),
+                          "total_regret": round(sum_auto / sum_best - 1.0, 4), "worst_regret": round(worst, 4),
+                          "shapes": rows_}))
+        return 0
 
     if args.prefill_only:
         out = {}

@@ -69,7 +69,7 @@ int gemv_w4a8_rows16(const uint8_t *w4, const float *ws, const int8_t *xq, const
 // gemm_w4a8_ring.hip: W4A8 tile GEMM with a ring of LDS stages for launches of few tiles; tile =
 // 6464 (64 x 64) or 64 (128 m x 64 n); arguments already checked.
 int gemm_w4a8_ring(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs, void *y, int M, int N,
-                   int K, int tile, void *stream);
+                   int K, int tile, void *stream, int ldy = 0);  // ldy: row pitch of y (0: N)
 // linear_bf16.hip: quantiser + W4A8 GEMV / GEMM (or the GEMV that quantises by itself where that
 // is faster) on bf16 rows, with xq int8 [M,K] / xs fp32 [M] as staging; arguments already checked.
 int linear_w4a8_rows(const uint8_t *w4, const float *ws, const void *x, void *y, int M, int N, int K, int gs,

@@ -47,6 +47,7 @@ struct Args {
     uint16_t *y;
     int32_t *group_acc;  // [M, G, N], nullable
     int M, N, K, G;
+    int ldy;  // row pitch of y (elements), >= N
     int tiles_m, tiles_n;
 };
 
@@ -295,7 +296,7 @@ gemm_w4a8_kernel(const Args a) {
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const int n = nb + j * 32 + (lane & 31);
-                if (n < a.N) a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total[i][j][v] * xm);
+                if (n < a.N) a.y[(size_t)m * a.ldy + n] = (uint16_t)f32_to_bf16_bits(total[i][j][v] * xm);
             }
         }
 }
@@ -374,8 +375,31 @@ extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     a.N = N;
     a.K = K;
     a.G = K / gs;
+    a.ldy = N;
     a.tiles_m = (M + BM - 1) / BM;
     a.tiles_n = (N + BN - 1) / BN;
+    // Whole rounds.  Two workgroups share a CU, so a launch runs in rounds of 512 tiles and a last
+    // round that is nearly empty costs as much as a full one (1024 x 25600: 1600 tiles = 3.125
+    // rounds, 252 us against 211 us for the 3.000 rounds of N = 24576).  The n tiles of such a
+    // remainder (at most half a round) go to a second launch of 64 x 64 tiles with a ring of
+    // stages, whose step is 0.44 us instead of 1.15 us and which spreads them over all CUs:
+    // same arithmetic, same bits.  (Not when the group sums are asked for: the ring kernels do not
+    // write them.)
+    int ring_n = 0;  // columns handed to the second launch
+    if (!forced && gs == BK && !group_acc) {
+        const int slots = 512, tiles = a.tiles_m * a.tiles_n, rest = tiles % slots;
+        if (tiles > slots && rest > 0 && rest <= slots / 2 && rest % a.tiles_m == 0) {
+            const int rest_n = rest / a.tiles_m;             // n tiles of the remainder
+            const int cols = N - (a.tiles_n - rest_n) * BN;  // their columns (the last tile may be ragged)
+            const double steps = K / 128.0, tiles_h = (double)a_ceil(M, 64) * a_ceil(cols, 64);
+            const double s_h = tiles_h <= 256 ? 0.44 + 6e-6 * cols : tiles_h <= 512 ? 0.65 + 1e-5 * cols : 0.4 + 0.00137 * tiles_h;
+            if (2.5 + steps * s_h < steps * 1.15) {
+                ring_n = cols;
+                a.N = N - cols;
+                a.tiles_n -= rest_n;
+            }
+        }
+    }
     const dim3 grid(a.tiles_m * a.tiles_n), block(THREADS);
     hipStream_t st = static_cast<hipStream_t>(stream);
     static std::atomic<uint64_t> devices[6];
@@ -387,5 +411,9 @@ extern "C" int cmi_gemm_w4a8(const uint8_t *w4, const float *ws, const int8_t *x
     };
     if (gs == 64) return group_acc ? run(gemm_w4a8_kernel<true, 1>, 0) : run(gemm_w4a8_kernel<false, 1>, 1);
     if (gs == 256) return group_acc ? run(gemm_w4a8_kernel<true, 3>, 2) : run(gemm_w4a8_kernel<false, 3>, 3);
-    return group_acc ? run(gemm_w4a8_kernel<true, 2>, 4) : run(gemm_w4a8_kernel<false, 2>, 5);
+    if (const int rc = group_acc ? run(gemm_w4a8_kernel<true, 2>, 4) : run(gemm_w4a8_kernel<false, 2>, 5)) return rc;
+    if (!ring_n) return CMI_OK;
+    const int n1 = N - ring_n;
+    return gemm_w4a8_ring(w4 + (size_t)n1 * (K / 2), ws + (size_t)n1 * a.G, xq, xs, static_cast<uint16_t *>(y) + n1, M, ring_n,
+                          K, 6464, stream, N);
 }

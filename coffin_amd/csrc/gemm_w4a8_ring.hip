@@ -39,6 +39,7 @@ struct Args {
     const float *ws;  // [N, G]
     uint16_t *y;
     int M, N, K, G;
+    int ldy;  // row pitch of y (elements), >= N
     int tiles_m, tiles_n;
 };
 
@@ -301,7 +302,7 @@ gemm_w4a8_ring_kernel(const Args a) {
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
                 const int n = nb + j * 32 + (lane & 31);
-                if (n < a.N) a.y[(size_t)m * a.N + n] = (uint16_t)f32_to_bf16_bits(total[i][j][v] * xm);
+                if (n < a.N) a.y[(size_t)m * a.ldy + n] = (uint16_t)f32_to_bf16_bits(total[i][j][v] * xm);
             }
         }
 }
@@ -327,7 +328,7 @@ namespace cmi {
 // the two-stage kernel, two of whose workgroups share a CU.  Arguments already checked by the
 // caller (K % 128 == 0, group size 128, 16-byte aligned xq and w4).
 int gemm_w4a8_ring(const uint8_t *w4, const float *ws, const int8_t *xq, const float *xs, void *y, int M, int N,
-                   int K, int tile, void *stream) {
+                   int K, int tile, void *stream, int ldy) {
     Args a;
     a.xq = xq;
     a.w4 = w4;
@@ -338,6 +339,7 @@ int gemm_w4a8_ring(const uint8_t *w4, const float *ws, const int8_t *xq, const f
     a.N = N;
     a.K = K;
     a.G = K / BK;
+    a.ldy = ldy > 0 ? ldy : N;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (tile == 6464) return launch<1, 1, 4>(a, st);
     if (tile == 64) return launch<1, 2, 3>(a, st);

@@ -400,6 +400,19 @@ gemm_w8a8_pipe_kernel(const Args a) {
         // point), ordered by "all my stores acknowledged" (vmcnt 0) before the arrival.  A device-
         // scope fence would do the same by writing back and invalidating the whole L2 under the
         // other workgroups' operand streams (measured: +25 us per launch).
+        // What this relies on, all of it properties of gfx950 and not of the HIP memory model:
+        //   - a relaxed agent-scope atomic store is emitted as global_store_dword ... sc1, which
+        //     writes through the issuing XCD's L2 to memory (the point all XCDs agree on);
+        //   - stores are counted by vmcnt on this ISA (gfx9 has no separate store counter), and a
+        //     write-through store is acknowledged only once it has reached that point, so
+        //     "s_waitcnt vmcnt(0)" below means every partial of this wavefront is visible chip-wide;
+        //   - __syncthreads() then orders all wavefronts' acknowledged stores before thread 0's
+        //     arrival atomic (a device-scope RMW executed at the same coherence point);
+        //   - a relaxed agent-scope atomic load is global_load_dword ... sc1, which misses the local
+        //     L2 and reads that point, so the last arriver cannot see a stale line.
+        // A compiler that lowered these atomics differently, or a part whose vmcnt did not cover
+        // write-through acknowledgement, would break this; test_linear_w8a8_bf16_split_k_same_bits
+        // and the repeated-launch comparison against the unsplit kernel are the guard.
         constexpr int ELEMS = TN * TM * 16;
         int *mine = a.partials + ((size_t)split * tiles + tile) * (ELEMS * THREADS) + threadIdx.x;
 #pragma unroll
@@ -1283,7 +1296,9 @@ int cmi::gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, co
             }
         }
     }
-    if (pick == 321) return launch_wide_tilewise(a, st);
+    // the 256 x 320 tile: the tile-wise kernel (1..3 % faster than the two-stage one on every shape
+    // tried, 7 % at 2048 x 4096 x 2560); a forced 320 still names the two-stage kernel
+    if (pick == 321 || (pick == 320 && !force)) return launch_wide_tilewise(a, st);
     if (pick == 320) return launch_wide(a, st);
     if (pick == 256) return launch_big(a, st);
     if (pick == 192) return launch<3, 2, 3>(a, st);

@@ -99,7 +99,7 @@ extern "C" int cmi_set_option(const char *name, int value) {
     CMI_REQUIRE(name, CMI_E_ARG, "cmi_set_option: null name");
     if (!strcmp(name, "gemm_tile")) {
         CMI_REQUIRE(valid_gemm_tile(value), CMI_E_ARG,
-                    "cmi_set_option: gemm_tile=%d, expected 0 (library's choice), 64, 128, 192, 256, 320, 6464 or 128192", value);
+                    "cmi_set_option: gemm_tile=%d, expected 0 (library's choice), 64, 128, 192, 256, 320, 321, 6464 or 128192", value);
         g_gemm_tile.store(value, std::memory_order_relaxed);
         return CMI_OK;
     }
