@@ -225,7 +225,7 @@ def main() -> int:
         del src, dst
 
     if args.tile_choice_check:
-        tiles = (64, 128, 192, 128192, 256, 320, 321, 6464)
+        tiles = (64, 128, 192, 128192, 256, 320, 321, 322, 6464)
         shapes_ = [(m, n_, k_) for (n_, k_) in ((9728, 2560), (4096, 2560), (2560, 9728), (6144, 2560), (2560, 4096))
                    for m in (64, 256, 512, 2048, 8192)]
         rows_, worst, sum_auto, sum_best = {}, 0.0, 0.0, 0.0

@@ -17,6 +17,8 @@ int check_launch(const char *what);
 // Raise a kernel's dynamic-LDS limit to `bytes` on the current device, once per device
 // (`devices`: one bit per device ordinal, owned by the call site).  CMI_OK or CMI_E_HIP.
 int reserve_lds(const void *kernel, int bytes, std::atomic<uint64_t> &devices, const char *who);
+// CUs of the current device (0: it cannot be read); cached per device.
+int compute_units();
 
 // Kernel-selection overrides (cmi_set_option / CMI_GEMM_TILE, CMI_GEMV_WHOLEROW read once).
 int option_gemm_tile();      // 0 = the library chooses, else 64 / 128 / 192 / 256 / 320 / 6464 / 128192

@@ -885,8 +885,104 @@ __device__ __forceinline__ void lds_wait(v4i32 &f0, v4i32 &f1, v4i32 &x0, v4i32 
         asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(f0), "+v"(f1), "+v"(x0), "+v"(x1), "+v"(x2), "+v"(x3)::"memory");
     else static_assert(N < 0, "add the lgkmcnt literal");
 }
+template <int IMM>
+__device__ __forceinline__ void read4(uint32_t &d, uint32_t base) {
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(d) : "v"(base), "n"(IMM) : "memory");
+}
+// A step of the persistent kernel next to a tile boundary differs from the plain one: the first
+// step of a tile starts its accumulators from zero, requests the tile's scales and, like the A
+// barrier of the second, has nothing to wait for in memory (the epilogue, or the prologue, before it
+// ended with every request landed); the last step of a tile leaves the next step's fragment reads
+// to whoever comes after the epilogue, which needs the registers.
+enum { STEP_PLAIN = 0, STEP_FIRST = 1, STEP_SECOND = 2, STEP_LAST = 3 };
+constexpr int SCALE_SLOTS = 16;  // persistent kernel: 256-byte pieces of the scale area, one per request
 }  // namespace tilewise
 
+// Epilogue of the persistent kernel for one wavefront tile of 5 x 2 MFMA tiles (corner: column
+// n0 + 160 (wave & 1), row m0 + 64 (wave / 2) of the matrix): scale, narrow, and write from
+// registers, touching no operand stage.  A lane holds, per MFMA tile and q, 4 consecutive columns of
+// its row (8 bytes of bf16); v_permlane32_swap trades one of each pair of such pieces with the lane
+// 32 up, which holds the columns in between, so that each lane owns 8 consecutive columns per
+// store: 20 stores of 16 bytes per wavefront.  They are buffer stores -- rows past M fall outside
+// the resource and are dropped, columns past N get an offset that does; N % 8 == 0 -- so every
+// wavefront issues all 20 whatever the tile.  The scales come from LDS at `scales_lds` (320 column
+// scales, then 256 row scales) through reads the compiler does not see: it would otherwise wait
+// for every request in flight, which are LDS writes to it.  Before the first store every request of
+// the wavefront has landed (vmcnt(0): by then the loads for the next tile's first two steps are
+// some microseconds old), so the vmcnt waits of the steps that follow never depend on how stores
+// and loads are retired relative to each other.
+__device__ __forceinline__ void epilogue_direct(const Args &a, v16i32 (&acc)[5][2], __amdgpu_buffer_rsrc_t yres,
+                                                uint32_t scales_lds, int wave, int n0, int m0) {
+    using namespace tilewise;
+    // the lane number anew, where the compiler cannot move it (and what is derived from it) out of
+    // the tile loop: the K steps have no registers to spare for the epilogue's addresses
+    int lane;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=&v"(lane));
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    typedef unsigned u32x2_swap __attribute__((ext_vector_type(2)));
+    const int wn = wave & 1, wm = wave >> 1, h = lane >> 5, r = lane & 31;
+    const uint32_t ws_base = scales_lds + (wn * 160 + 4 * h) * 4;
+    const uint32_t xs_base = scales_lds + (wide::BN + wm * 64 + r) * 4;
+    uint32_t xm_bits[2];
+    read4<0>(xm_bits[0], xs_base);
+    read4<128>(xm_bits[1], xs_base);
+    u32x4 out[5][2][2];
+    using std::integral_constant;
+    auto tile_row = [&](auto i_tag) {
+        constexpr int I = decltype(i_tag)::value;
+        v4i32 wsv[4];
+        read16<(32 * I + 0) * 4>(wsv[0], ws_base);
+        read16<(32 * I + 8) * 4>(wsv[1], ws_base);
+        read16<(32 * I + 16) * 4>(wsv[2], ws_base);
+        read16<(32 * I + 24) * 4>(wsv[3], ws_base);
+        asm volatile("s_waitcnt lgkmcnt(0)"
+                     : "+v"(wsv[0]), "+v"(wsv[1]), "+v"(wsv[2]), "+v"(wsv[3]), "+v"(xm_bits[0]), "+v"(xm_bits[1])::"memory");
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const float xm = __uint_as_float(xm_bits[j]);
+            uint32_t d[4][2];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float t[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) t[e] = ((float)acc[I][j][4 * q + e] * xm) * __int_as_float(wsv[q][e]);
+                d[q][0] = pack_bf16(t[0], t[1]);
+                d[q][1] = pack_bf16(t[2], t[3]);
+            }
+            // pieces 2p and 2p+1 hold columns 16p + 4h .. and 16p + 8 + 4h ..: the lower lane hands
+            // its 2p+1 up and gets the upper lane's 2p, after which lane half h owns 16p + 8h .. + 7
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const u32x2_swap s0 = __builtin_amdgcn_permlane32_swap(d[2 * p][0], d[2 * p + 1][0], false, false);
+                const u32x2_swap s1 = __builtin_amdgcn_permlane32_swap(d[2 * p][1], d[2 * p + 1][1], false, false);
+                out[I][j][p] = u32x4{s0.x, s1.x, s0.y, s1.y};
+            }
+        }
+    };
+    tile_row(integral_constant<int, 0>{});
+    tile_row(integral_constant<int, 1>{});
+    tile_row(integral_constant<int, 2>{});
+    tile_row(integral_constant<int, 3>{});
+    tile_row(integral_constant<int, 4>{});
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    const int ncols = a.N - (n0 + wn * 160 + 8 * h);  // columns left from this lane's first
+    const uint32_t ytile = (uint32_t)(((size_t)m0 * a.ldy + n0) * 2);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t voff = (uint32_t)(((wm * 64 + 32 * j + r) * a.ldy + wn * 160 + 8 * h) * 2);
+#pragma unroll
+        for (int i = 0; i < 5; ++i)
+#pragma unroll
+            for (int p = 0; p < 2; ++p)
+                __builtin_amdgcn_raw_buffer_store_b128(out[i][j][p], yres,
+                                                       32 * i + 16 * p < ncols ? voff + (32 * i + 16 * p) * 2 : 0x80000000u,
+                                                       ytile, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+template <bool PERSIST>
 __global__ void __launch_bounds__(512, 2)
 gemm_w8a8_wide_tilewise_kernel(const Args a) {
     using namespace wide;
@@ -896,11 +992,12 @@ gemm_w8a8_wide_tilewise_kernel(const Args a) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int wn = wave & 1, wm = wave >> 1;
 
+    const int tiles = a.tiles_m * a.tiles_n;
     int tm, tn;
     tile_coords(a, tm, tn);
-    const int m0 = tm * BM, n0 = tn * BN;
+    int m0 = tm * BM, n0 = tn * BN;
     float *scales = reinterpret_cast<float *>(lds + OPERAND_BYTES);
-    stage_scales<BN, BM>(a, scales, n0, m0);
+    if constexpr (!PERSIST) stage_scales<BN, BM>(a, scales, n0, m0);
 
     // LDS: weights as [n half][stage][160 rows], activations behind them as [m quarter][stage][64 rows],
     // so that both stages of a wavefront's rows are within the 64 KiB reach of an LDS instruction's
@@ -910,6 +1007,9 @@ gemm_w8a8_wide_tilewise_kernel(const Args a) {
     // are 8 loads of 8 rows, one per wavefront: wavefront w takes rows 160 (w & 1) + 32 i + 8 (w >> 1)
     // .. + 7.  X rows 32 w + 8 g .. + 7, g = 0..3.  Lane i of a load lands in slot i of the 1 KiB:
     // row i / 8, stored chunk i % 8, which holds k chunk (i % 8) ^ ((row / 2) % 8).
+    // A buffer access is checked against the resource's size with the scalar offset included
+    // (measured on gfx950: lane offset 0 + scalar offset past the end reads 0), so the tile corner
+    // can live in the scalar offset and rows past the matrix still read as zeros.
     const int lrow = lane >> 3;
     const int wrow = wn * 160 + wm * 8 + lrow;  // + 32 i: the swizzle does not depend on i
     const uint32_t wvoff = (uint32_t)wrow * (uint32_t)a.K + (((lane & 7) ^ ((wrow >> 1) & 7)) * 16);
@@ -922,26 +1022,45 @@ gemm_w8a8_wide_tilewise_kernel(const Args a) {
         __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(a.wq), 0, (int)((size_t)a.N * a.K), 0x00020000);
     const __amdgpu_buffer_rsrc_t xres =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(a.xq), 0, (int)((size_t)a.M * a.K), 0x00020000);
-    const uint32_t wtile = (uint32_t)n0 * (uint32_t)a.K, xtile = (uint32_t)m0 * (uint32_t)a.K;
+    uint32_t wtile = (uint32_t)n0 * (uint32_t)a.K, xtile = (uint32_t)m0 * (uint32_t)a.K;
     const uint32_t k32 = 32u * (uint32_t)a.K, k8 = 8u * (uint32_t)a.K;
     int8_t *const wslot = lds + wn * 2 * W_HALF + wm * 8 * BK;                              // weight tile 0, stage 0
     int8_t *const xslot = lds + X_BASE + (wave >> 1) * 2 * X_QUARTER + (wave & 1) * 4 * 1024;  // g = 0, stage 0
-    auto issue_w = [&](int stage, int ks, int i) {
+    // step ks of the tile whose corner offsets are wt / xt
+    auto issue_w = [&](int stage, uint32_t wt, int ks, int i) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(wres, (lds_ptr_t)(wslot + stage * W_HALF + i * 32 * BK), 16, wvoff,
-                                                 wtile + i * k32 + ks * BK, 0, 0);
+                                                 wt + i * k32 + ks * BK, 0, 0);
     };
-    auto issue_a = [&](int stage, int ks) {
+    auto issue_a = [&](int stage, uint32_t wt, uint32_t xt, int ks) {
 #pragma unroll
         for (int g = 0; g < XL; ++g)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(xres, (lds_ptr_t)(xslot + stage * X_QUARTER + g * 1024), 16,
-                                                     xvoff[g & 1], xtile + g * k8 + ks * BK, 0, 0);
-        issue_w(stage, ks, 0);
-        issue_w(stage, ks, 1);
+                                                     xvoff[g & 1], xt + g * k8 + ks * BK, 0, 0);
+        issue_w(stage, wt, ks, 0);
+        issue_w(stage, wt, ks, 1);
     };
-    auto issue_b = [&](int stage, int ks) {
-        issue_w(stage, ks, 2);
-        issue_w(stage, ks, 3);
-        issue_w(stage, ks, 4);
+    auto issue_b = [&](int stage, uint32_t wt, int ks) {
+        issue_w(stage, wt, ks, 2);
+        issue_w(stage, wt, ks, 3);
+        issue_w(stage, wt, ks, 4);
+    };
+    // Persistent kernel: the scales of the tile whose corner is (n_, m_), two requests of 64 floats
+    // per wavefront (every wavefront issues the same number of loads: the vmcnt waits count them):
+    // pieces 0..4 the 320 column scales, 5..8 the 256 row scales, the rest unused; past the matrix zeros.
+    auto issue_scales = [&](int n_, int m_) {
+        const __amdgpu_buffer_rsrc_t wsres =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(a.ws), 0, a.N * 4, 0x00020000);
+        const __amdgpu_buffer_rsrc_t xsres =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(a.xs), 0, a.M * 4, 0x00020000);
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int q = 2 * wave + e;
+            const lds_ptr_t dst = (lds_ptr_t)(lds + OPERAND_BYTES + q * 256);
+            if (q >= 5 && q < 9)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(xsres, dst, 4, lane * 4, (m_ + 64 * (q - 5)) * 4, 0, 0);
+            else
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(wsres, dst, 4, lane * 4, (n_ + (q < 5 ? 64 * q : 0)) * 4, 0, 0);
+        }
     };
 
     // Fragment reads: lane reads row (lane % 32) of a 32-row MFMA tile; for k quarter q its 16 bytes
@@ -976,20 +1095,29 @@ gemm_w8a8_wide_tilewise_kernel(const Args a) {
     };
 
     v16i32 acc[TN][TM];
+    if constexpr (!PERSIST) {
 #pragma unroll
-    for (int i = 0; i < TN; ++i)
+        for (int i = 0; i < TN; ++i)
 #pragma unroll
-        for (int j = 0; j < TM; ++j)
+            for (int j = 0; j < TM; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
-    // the 4 MFMAs of half group K in a step of parity P
-    auto mma = [&](auto parity_tag, auto hg_tag) {
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+    }
+    // the 4 MFMAs of half group K in a step of parity P; FRESH: the accumulators start from zero
+    // (the first MFMA into each takes the constant as its addend)
+    auto mma = [&](auto parity_tag, auto hg_tag, auto fresh_tag) {
         constexpr int P = decltype(parity_tag)::value, K = decltype(hg_tag)::value, I = K / 2, H = K % 2;
+        constexpr bool FRESH = decltype(fresh_tag)::value != 0 && H == 0;
 #pragma unroll
         for (int q = 0; q < 2; ++q)
 #pragma unroll
-            for (int j = 0; j < TM; ++j)
-                acc[I][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[BUF[P][K]][q], xf[j][2 * H + q], acc[I][j], 0, 0, 0);
+            for (int j = 0; j < TM; ++j) {
+                v16i32 c = acc[I][j];
+                if (FRESH && q == 0)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) c[v] = 0;
+                acc[I][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[BUF[P][K]][q], xf[j][2 * H + q], c, 0, 0, 0);
+            }
     };
     // the wait in front of half group K: N reads were issued after its fragments
     auto wait_w = [&](auto parity_tag, auto hg_tag, auto n_tag) {
@@ -1001,104 +1129,153 @@ gemm_w8a8_wide_tilewise_kernel(const Args a) {
         lds_wait<N>(wf[BUF[P][K]][0], wf[BUF[P][K]][1], xf[0][2 * H], xf[1][2 * H], xf[0][2 * H + 1], xf[1][2 * H + 1]);
     };
     auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
-
-    const int ksteps = a.K / BK;
-    // One K step from stage P = ks & 1.  On entry the fragments of half groups 0 and 1 are on their
-    // way (12 reads, issued in that order).  The last two steps request the last step's operands once
-    // more instead of nothing (into rows that are free, nobody reads them): every step then issues the
-    // same 9 loads and both vmcnt waits are 9 throughout.
-    auto step = [&](auto p, int ks) {
-        constexpr int P = decltype(p)::value;
-        constexpr auto np = IC(P ^ 1);
-        const int ahead = min(ks + 2, ksteps - 1);
-        wait_wx(p, IC(0), IC(6));
-        mma(p, IC(0));
-        read_w(p, IC(2));
-        fence();
-        wait_wx(p, IC(1), IC(2));
-        mma(p, IC(1));
-        read_w(p, IC(3));
-        fence();
-        wait_w(p, IC(2), IC(2));
-        mma(p, IC(2));
-        fence();
-        // A: X and weight tiles 0, 1 of this stage are in registers everywhere; tiles 2..4 have landed
-        wait_w(p, IC(3), IC(0));
-        asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        issue_a(P, ahead);
-        read_w(p, IC(4));
-        read_w(p, IC(5));
-        mma(p, IC(3));
-        fence();
-        wait_w(p, IC(4), IC(2));
-        mma(p, IC(4));
-        read_w(p, IC(6));
-        fence();
-        wait_w(p, IC(5), IC(2));
-        mma(p, IC(5));
-        read_w(p, IC(7));
-        fence();
-        wait_w(p, IC(6), IC(2));
-        mma(p, IC(6));
-        read_w(p, IC(8));
-        fence();
-        wait_w(p, IC(7), IC(2));
-        mma(p, IC(7));
-        read_w(p, IC(9));
-        fence();
-        wait_w(p, IC(8), IC(2));
-        mma(p, IC(8));
-        fence();
-        // B: weight tiles 2..4 are in registers everywhere; X and tiles 0, 1 of the next step have landed
-        wait_w(p, IC(9), IC(0));
-        asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        issue_b(P, ahead);
-        // the next step's first fragments (past the last step: a stale stage, nobody uses them);
-        // its quarters 2, 3 of X replace the ones this half group still multiplies, so they follow it
-        read_w(np, IC(0));
-        read_x(np, IC(0));
-        fence();
-        mma(p, IC(9));
-        fence();
-        read_w(np, IC(1));
-        read_x(np, IC(1));
+    // the first fragments of a tile's first step (half groups 0 and 1 of a step of parity 0)
+    auto read_first = [&]() {
+        read_w(IC(0), IC(0));
+        read_x(IC(0), IC(0));
+        read_w(IC(0), IC(1));
+        read_x(IC(0), IC(1));
         fence();
     };
 
+    const int ksteps = a.K / BK;
+    // One K step from stage P.  On entry the fragments of half groups 0 and 1 are on their way (12
+    // reads, issued in that order).  Its requests are step `rks` of the tile at rw / rx: two steps
+    // ahead; past the end of the last tile the last step's operands once more instead of nothing
+    // (into rows that are free, nobody reads them), so that every step issues the same 9 loads and
+    // both vmcnt waits are 9 throughout.
+    auto step = [&](auto p, auto kind_tag, uint32_t rw, uint32_t rx, int rks) {
+        constexpr int P = decltype(p)::value, KIND = decltype(kind_tag)::value;
+        constexpr auto np = IC(P ^ 1);
+        constexpr auto fresh = IC(KIND == STEP_FIRST ? 1 : 0);
+        wait_wx(p, IC(0), IC(6));
+        mma(p, IC(0), fresh);
+        read_w(p, IC(2));
+        fence();
+        wait_wx(p, IC(1), IC(2));
+        mma(p, IC(1), fresh);
+        read_w(p, IC(3));
+        fence();
+        wait_w(p, IC(2), IC(2));
+        mma(p, IC(2), fresh);
+        fence();
+        // A: X and weight tiles 0, 1 of this stage are in registers everywhere; tiles 2..4 have landed
+        wait_w(p, IC(3), IC(0));
+        if constexpr (KIND != STEP_FIRST && KIND != STEP_SECOND) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        issue_a(P, rw, rx, rks);
+        if constexpr (KIND == STEP_FIRST) issue_scales(n0, m0);
+        read_w(p, IC(4));
+        read_w(p, IC(5));
+        mma(p, IC(3), fresh);
+        fence();
+        wait_w(p, IC(4), IC(2));
+        mma(p, IC(4), fresh);
+        read_w(p, IC(6));
+        fence();
+        wait_w(p, IC(5), IC(2));
+        mma(p, IC(5), fresh);
+        read_w(p, IC(7));
+        fence();
+        wait_w(p, IC(6), IC(2));
+        mma(p, IC(6), fresh);
+        read_w(p, IC(8));
+        fence();
+        wait_w(p, IC(7), IC(2));
+        mma(p, IC(7), fresh);
+        read_w(p, IC(9));
+        fence();
+        wait_w(p, IC(8), IC(2));
+        mma(p, IC(8), fresh);
+        fence();
+        // B: weight tiles 2..4 are in registers everywhere; X and tiles 0, 1 of the next step have landed
+        wait_w(p, IC(9), IC(0));
+        if constexpr (KIND != STEP_FIRST) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        issue_b(P, rw, rks);
+        if constexpr (KIND == STEP_LAST) {
+            fence();
+            mma(p, IC(9), fresh);
+            fence();
+        } else {
+            // the next step's first fragments (past the last step: a stale stage, nobody uses them);
+            // its quarters 2, 3 of X replace the ones this half group still multiplies, so they follow it
+            read_w(np, IC(0));
+            read_x(np, IC(0));
+            fence();
+            mma(p, IC(9), fresh);
+            fence();
+            read_w(np, IC(1));
+            read_x(np, IC(1));
+            fence();
+        }
+    };
+
     // Prologue: both stages requested in the order the steps request them (A then B).
-    issue_a(0, 0);
-    issue_b(0, 0);
-    issue_a(1, min(1, ksteps - 1));
-    issue_b(1, min(1, ksteps - 1));
-    asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    // The persistent kernel waits for all of it: its first tile then starts like every other, behind an
+    // epilogue that left no request in flight.
+    issue_a(0, wtile, xtile, 0);
+    issue_b(0, wtile, 0);
+    issue_a(1, wtile, xtile, min(1, ksteps - 1));
+    issue_b(1, wtile, min(1, ksteps - 1));
+    if constexpr (PERSIST) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    read_w(IC(0), IC(0));
-    read_x(IC(0), IC(0));
-    read_w(IC(0), IC(1));
-    read_x(IC(0), IC(1));
-    fence();
-    int ks = 0;
-    for (; ks + 1 < ksteps; ks += 2) {
-        step(IC(0), ks);
-        step(IC(1), ks + 1);
-    }
-    if (ks < ksteps) step(IC(0), ks);
-    // the stale fragment reads and the repeated requests of the last steps must be over before their
-    // registers and the stages are used for anything else
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    fence();
-#undef IC
+    read_first();
 
-    epilogue<TN, TM, 1>(a, acc, lds, wave, lane, n0 + wn * 32 * TN, m0 + wm * 32 * TM, scales + wn * 32 * TN,
-                        scales + BN + wm * 32 * TM);
+    if constexpr (!PERSIST) {
+        int ks = 0;
+        for (; ks + 1 < ksteps; ks += 2) {
+            step(IC(0), IC(STEP_PLAIN), wtile, xtile, min(ks + 2, ksteps - 1));
+            step(IC(1), IC(STEP_PLAIN), wtile, xtile, min(ks + 3, ksteps - 1));
+        }
+        if (ks < ksteps) step(IC(0), IC(STEP_PLAIN), wtile, xtile, ksteps - 1);
+        // the stale fragment reads and the repeated requests of the last steps must be over before their
+        // registers and the stages are used for anything else
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        fence();
+        epilogue<TN, TM, 1>(a, acc, lds, wave, lane, n0 + wn * 32 * TN, m0 + wm * 32 * TM, scales + wn * 32 * TN,
+                            scales + BN + wm * 32 * TM);
+    } else {
+        // Tiles blockIdx.x, + gridDim.x, ...: an even number (>= 4) of K steps each, so that a tile
+        // starts in stage 0.  The last two steps of a tile request the first two of the next, the
+        // epilogue touches no operand stage (results go from registers to memory, scales from
+        // their own corner of LDS), so the pipeline runs on across the boundary.
+        const __amdgpu_buffer_rsrc_t yres = __builtin_amdgcn_make_buffer_rsrc(
+            a.y, 0, (int)((((size_t)a.M - 1) * a.ldy + a.N) * 2), 0x00020000);
+        int tile = blockIdx.x;
+        while (true) {
+            const int next = tile + gridDim.x;
+            const bool more = next < tiles;
+            int m1 = m0, n1 = n0;
+            if (more) {
+                tile_coords(a, tm, tn, next);
+                m1 = tm * BM, n1 = tn * BN;
+            }
+            const uint32_t wnext = (uint32_t)n1 * (uint32_t)a.K, xnext = (uint32_t)m1 * (uint32_t)a.K;
+            step(IC(0), IC(STEP_FIRST), wtile, xtile, 2);
+            step(IC(1), IC(STEP_SECOND), wtile, xtile, 3);
+            for (int ks = 2; ks < ksteps - 2; ks += 2) {
+                step(IC(0), IC(STEP_PLAIN), wtile, xtile, ks + 2);
+                step(IC(1), IC(STEP_PLAIN), wtile, xtile, ks + 3);
+            }
+            step(IC(0), IC(STEP_PLAIN), wnext, xnext, more ? 0 : ksteps - 1);
+            step(IC(1), IC(STEP_LAST), wnext, xnext, more ? 1 : ksteps - 1);
+            epilogue_direct(a, acc, yres, lds_offset(scales), wave, n0, m0);
+            if (!more) break;
+            tile = next, m0 = m1, n0 = n1, wtile = wnext, xtile = xnext;
+            read_first();
+        }
+    }
+#undef IC
 }
 
 int launch_wide(Args &a, hipStream_t st);
+
+int wide_tiles(int M, int N) { return ((M + wide::BM - 1) / wide::BM) * ((N + wide::BN - 1) / wide::BN); }
 
 int launch_wide_tilewise(Args &a, hipStream_t st) {
     // buffer offsets are 32 bits: matrices (and the tile rows past their end) must stay below 2 GiB
@@ -1107,10 +1284,32 @@ int launch_wide_tilewise(Args &a, hipStream_t st) {
     a.tiles_m = (a.M + wide::BM - 1) / wide::BM;
     a.tiles_n = (a.N + wide::BN - 1) / wide::BN;
     static std::atomic<uint64_t> devices{0};
-    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_wide_tilewise_kernel),
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_wide_tilewise_kernel<false>),
                                    wide::LDS_BYTES, devices, "cmi_gemm_w8a8"))
         return rc;
-    gemm_w8a8_wide_tilewise_kernel<<<dim3(a.tiles_m * a.tiles_n), dim3(512), wide::LDS_BYTES, st>>>(a);
+    gemm_w8a8_wide_tilewise_kernel<false><<<dim3(a.tiles_m * a.tiles_n), dim3(512), wide::LDS_BYTES, st>>>(a);
+    return check_launch("cmi_gemm_w8a8");
+}
+
+// The persistent form: one workgroup per CU walks tiles blockIdx.x, + grid, ...  Takes what the
+// direct epilogue can write (bf16 rows of 16-byte pieces, no int32 dump) and an even number of K
+// steps; anything else goes to the one-tile-per-workgroup kernel.
+int launch_wide_persistent(Args &a, hipStream_t st) {
+    const int ksteps = a.K / BK;
+    const bool fits = !a.acc_out && a.N % 8 == 0 && a.ldy % 8 == 0 && aligned(a.y, 16) && ksteps >= 4 && ksteps % 2 == 0 &&
+                      ((size_t)a.M + wide::BM) * a.ldy * 2 < ((size_t)1 << 31) &&
+                      (size_t)(a.N + wide::BN) * a.K < ((size_t)1 << 31) && (size_t)(a.M + wide::BM) * a.K < ((size_t)1 << 31);
+    if (!fits) return launch_wide_tilewise(a, st);
+    a.tiles_m = (a.M + wide::BM - 1) / wide::BM;
+    a.tiles_n = (a.N + wide::BN - 1) / wide::BN;
+    constexpr int LDS = wide::OPERAND_BYTES + tilewise::SCALE_SLOTS * 256;
+    static std::atomic<uint64_t> devices{0};
+    if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemm_w8a8_wide_tilewise_kernel<true>), LDS, devices,
+                                   "cmi_gemm_w8a8"))
+        return rc;
+    const int tiles = a.tiles_m * a.tiles_n, cus = compute_units();
+    CMI_REQUIRE(cus > 0, CMI_E_HIP, "cmi_gemm_w8a8: cannot read the device's compute unit count");
+    gemm_w8a8_wide_tilewise_kernel<true><<<dim3(tiles < cus ? tiles : cus), dim3(512), LDS, st>>>(a);
     return check_launch("cmi_gemm_w8a8");
 }
 
@@ -1298,6 +1497,12 @@ int cmi::gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, co
     }
     // the 256 x 320 tile: the tile-wise kernel (1..3 % faster than the two-stage one on every shape
     // tried, 7 % at 2048 x 4096 x 2560); a forced 320 still names the two-stage kernel
+    // The persistent form (322) keeps its pipeline running from tile to tile.  At the clock the power
+    // limit leaves a launch of this size, closing the gaps between tiles buys little: measured -2.4 %
+    // at 7.6 tiles per CU (8192 x 19456 x 2560, 372.9 -> 363.8 us, cold and warm weights alike),
+    // -2 % cold / +0.5 % warm at 3.9, and a single tile is 3 % slower than the one-tile kernel
+    // (its epilogue writes 32 bytes per row and store instead of whole rows).  From four tiles per CU.
+    if (pick == 322 || (pick == 320 && !force && wide_tiles(a.M, a.N) > 4 * compute_units())) return launch_wide_persistent(a, st);
     if (pick == 321 || (pick == 320 && !force)) return launch_wide_tilewise(a, st);
     if (pick == 320) return launch_wide(a, st);
     if (pick == 256) return launch_big(a, st);

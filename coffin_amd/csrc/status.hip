@@ -44,6 +44,17 @@ int reserve_lds(const void *kernel, int bytes, std::atomic<uint64_t> &devices, c
     return CMI_OK;
 }
 
+int compute_units() {
+    static std::atomic<int> count[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    int n = count[dev & 63].load(std::memory_order_relaxed);
+    if (n > 0) return n;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+    count[dev & 63].store(n, std::memory_order_relaxed);
+    return n;
+}
+
 // ------------------------------------------------------------------ options
 // Kernel-selection overrides for tests and tuning.  Each is read from its environment variable
 // once, when first asked for, and validated there; afterwards only cmi_set_option changes it, so
@@ -55,7 +66,7 @@ std::atomic<int> g_gemv_wholerow{UNREAD};  // -1 = the library chooses, 0 = neve
 std::atomic<int> g_w4_decode_waves{0};     // 0 = the library chooses, 4 or 16 wavefronts per workgroup
 std::atomic<int> g_w4_decode_chain{0};     // 0 = the library chooses, 1 = never, else a variant code
 
-bool valid_gemm_tile(int v) { return v == 0 || v == 64 || v == 128 || v == 256 || v == 192 || v == 320 || v == 321 || v == 6464 || v == 128192; }
+bool valid_gemm_tile(int v) { return v == 0 || v == 64 || v == 128 || v == 256 || v == 192 || v == 320 || v == 321 || v == 322 || v == 6464 || v == 128192; }
 bool valid_wholerow(int v) { return v >= -1 && v <= 1; }
 
 int from_env(const char *name, int fallback, bool (*valid)(int)) {
@@ -99,7 +110,7 @@ extern "C" int cmi_set_option(const char *name, int value) {
     CMI_REQUIRE(name, CMI_E_ARG, "cmi_set_option: null name");
     if (!strcmp(name, "gemm_tile")) {
         CMI_REQUIRE(valid_gemm_tile(value), CMI_E_ARG,
-                    "cmi_set_option: gemm_tile=%d, expected 0 (library's choice), 64, 128, 192, 256, 320, 321, 6464 or 128192", value);
+                    "cmi_set_option: gemm_tile=%d, expected 0 (library's choice), 64, 128, 192, 256, 320, 321, 322, 6464 or 128192", value);
         g_gemm_tile.store(value, std::memory_order_relaxed);
         return CMI_OK;
     }

@@ -40,7 +40,9 @@ int cmi_abi_version(void);
  *   "gemm_tile"     0 (the library chooses) | 64 | 128 | 192 | 256 | 320 (tile along n) | 6464 (64 x 64)
  *                   | 128192 (128 n x 192 m) | 321 (the 256 x 320 tile walked weight tile by weight
  *                   tile: what the library runs where it chooses that tile; 320 names the older
- *                   two-stage kernel): block tile of cmi_gemm_w8a8 / cmi_gemm_w4a8 (non-zero also
+ *                   two-stage kernel) | 322 (321 as one workgroup per CU that walks its tiles one
+ *                   after the other: the library's choice where that tile gives more than four
+ *                   tiles per CU): block tile of cmi_gemm_w8a8 / cmi_gemm_w4a8 (non-zero also
  *                   bypasses their few-row routes);
  *   "gemv_wholerow" -1 (the library chooses) | 0 (never) | 1: the one-wavefront-per-weight-row
  *                   kernel of cmi_gemv_w8a16;

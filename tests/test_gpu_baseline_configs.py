@@ -26,7 +26,7 @@ from tests import gpu_util as G
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=["auto", "64", "128", "192", "128192", "256", "320", "321"])
+@pytest.fixture(params=["auto", "64", "128", "192", "128192", "256", "320", "321", "322"])
 def gemm_tile(request):
     if request.param != "auto":
         G.set_option("gemm_tile", int(request.param))

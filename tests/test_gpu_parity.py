@@ -290,7 +290,7 @@ def test_sixteen_row_kernels_at_lm_head_size_sampled_columns(orc):
 
 # ------------------------------------------------------------------ W8A8 GEMM
 
-@pytest.fixture(params=["auto", "64", "128", "192", "128192", "256", "320", "321", "6464"])
+@pytest.fixture(params=["auto", "64", "128", "192", "128192", "256", "320", "321", "322", "6464"])
 def gemm_tile(request):
     """Force the 128 x 64, 128 x 128, 128 x 192, 192 x 128, 256 x 256, 256 x 320 or 64 x 64 (m x n) block-tile kernel through
     cmi_set_option, or leave the choice to the library (conftest resets it after each test)."""
@@ -380,6 +380,31 @@ def test_gemm_w8a8_full_size_sampled_and_blockwise(orc, gemm_tile, m, n):
     # every element: checksum of the int32 accumulators against an fp64 matmul on the device
     total = (xq.double().sum(0) @ q.wq.double().t()).sum()
     assert float(acc.double().sum()) == float(total)
+
+
+@pytest.mark.parametrize("m,n,k", [(4100, 6408, 512), (8192, 9728, 2560), (2100, 12808, 1024), (600, 45000, 768),
+                                   (8200, 19456, 512)])
+def test_gemm_w8a8_workgroups_walking_several_tiles_give_the_one_tile_bits(orc, m, n, k):
+    """More 256 x 320 tiles than CUs: a workgroup of the persistent kernel (tile code 322, and the
+    library's own choice at the last shape, more than four tiles per CU) takes several, its requests running on from one tile
+    into the next and its results going from registers to memory.  Ragged last tiles in both
+    directions, a row pitch above N; bits of the 128 x 128 tile kernel and of the oracle."""
+    g = synth.generator(99, G.DEV)
+    q = synth.int8_weight(n, k, g)
+    x = synth.activations(m, k, g, outliers=True)
+    xq, xs = G.quant(x)
+    G.set_option("gemm_tile", 128)
+    _, y_t = G.gemm_w8a8(xq, q.wq, xs, q.scale, want_acc=False)
+    rows = torch.randint(0, m, (6,), generator=torch.Generator().manual_seed(5)).tolist() + [0, m - 1]
+    ridx = torch.tensor(rows, device=G.DEV)
+    _, y_ref = orc.gemm_w8a8(xq[ridx].cpu().numpy(), q.wq.cpu().numpy(), xs[ridx].cpu().numpy(), q.scale.cpu().numpy())
+    assert (G.bits(y_t[ridx]) == y_ref).all()
+    for tile in (322, 0):
+        G.set_option("gemm_tile", tile)
+        _, y = G.gemm_w8a8(xq, q.wq, xs, q.scale, want_acc=False, ldy=n + 24)
+        assert (y[:, :n].contiguous().view(torch.int16) == y_t.view(torch.int16)).all(), tile
+        assert (y[:, n:].float() == 0).all(), tile
+    G.set_option("gemm_tile", 0)
 
 
 @pytest.mark.parametrize("n,k", [(9728, 2560), (2560, 9728), (6144, 2560)])
@@ -614,7 +639,7 @@ def test_random_shapes_and_forced_tiles_against_the_oracle(orc):
         k = step * pick((1, 9), (9, 41), (41, 11008 // step + 1))
         while m * n * k > 2e9:
             m = max(1, m // 2)
-        tile = int(rnd.choice([0, 0, 0, 64, 128, 192, 128192, 256, 320, 321, 6464]))
+        tile = int(rnd.choice([0, 0, 0, 64, 128, 192, 128192, 256, 320, 321, 322, 6464]))
         want_acc = bool(rnd.randint(2))
         what = (case, kind, m, n, k, tile, want_acc)
         x = synth.activations(m, k, g, outliers=bool(rnd.randint(2)))
