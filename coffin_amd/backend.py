@@ -75,11 +75,12 @@ W8A8_VERIFY = os.environ.get("COFFIN_AMD_W8A8_VERIFY", "0").strip() == "1"
 BATCH_MFMA = os.environ.get("COFFIN_AMD_BATCH_MFMA", "0").strip() == "1"
 #: int4 weights are answered with W4A8 arithmetic (per-token int8 activations), which is what coffin
 #: runs on its native backends.  ``COFFIN_AMD_W4A16=1`` keeps the activations unquantised instead for
-#: decode-sized calls (up to ``W4A16_MAX_ROWS`` rows, K <= 10240): the int4 weight-only GEMV, i.e. the
+#: decode-sized calls (up to ``W4A16_MAX_ROWS`` rows, K <= ``W4A16_MAX_K``): the int4 weight-only GEMV, i.e. the
 #: arithmetic of the reference's torch path for an int4 weight (backends/reference/__init__.py:93-95)
 #: up to fp32 summation order; one launch per row, so it is meant for single-stream decode.
 W4A16 = os.environ.get("COFFIN_AMD_W4A16", "0").strip() == "1"
 W4A16_MAX_ROWS = 4
+W4A16_MAX_K = 32768
 #: Rows from which the matrix-pipe GEMV beats the dot-product one (measured on every layer shape).
 MFMA_MIN_ROWS = 3
 #: ``rms_norm`` / ``add_rms_norm`` / ``silu_mul`` also leave their output rows quantised (int8 +
@@ -472,7 +473,7 @@ def _gemv_q8(rec: _Record, act: torch.Tensor, rows: int, out: torch.Tensor, mfma
     or a process whose family is "mfma" uses it for every call, single rows included."""
     n, k = rec.n, rec.k
     whole = rec.family == "mfma" if rec.family is not None else BATCH_MFMA
-    fast = (whole or (mfma and rows >= MFMA_MIN_ROWS)) and k % 128 == 0 and k <= 10240
+    fast = (whole or (mfma and rows >= MFMA_MIN_ROWS)) and k % 128 == 0
     rc = _native.load().cmi_linear_w8a16(rec.a, rec.b, act.data_ptr(), out.data_ptr(), rows, n, k,
                                          1 if fast else 0, _stream())
     if rc:
@@ -582,7 +583,7 @@ def _project(w, x: torch.Tensor, prefill: bool, min_rows: int = PREFILL_MIN_ROWS
     out = torch.empty((rec.n,) if nd == 1 else (rows, rec.n), dtype=torch.bfloat16, device=dev)
     if rows == 0:
         return out
-    w4a16 = rec.kind == 4 and W4A16 and rows <= W4A16_MAX_ROWS and rec.k <= 10240 and rec.gs == 128 and rec.kd == rec.k
+    w4a16 = rec.kind == 4 and W4A16 and rows <= W4A16_MAX_ROWS and rec.k <= W4A16_MAX_K and rec.gs == 128 and rec.kd == rec.k
     quantising = (rec.kind == 4 and not w4a16) or (rec.kind == 8 and prefill and rows >= min_rows)
     if quantising and _HANDED is not None and rec.kd == rec.k:
         # the rows a producer of this backend left behind for exactly this tensor

@@ -25,7 +25,8 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int GS = 128;
 constexpr int WAVES = 4;
-constexpr int MAX_K = 10240;  // five passes of 2048 k
+constexpr int MAX_PASSES = 16;
+constexpr int MAX_K = MAX_PASSES * 2048;  // a wavefront keeps its whole row in registers: 4 per pass
 
 struct Args {
     const uint8_t *w4;
@@ -69,7 +70,7 @@ gemv_w4a16_kernel(const Args a) {
     const int nchunks = a.K / 32, xvecs = a.K / 8;
 
     // activations first (memory answers in request order), then every weight byte of the row
-    constexpr int XV = MAX_K / 8 / (64 * WAVES);  // 5 vectors per thread
+    constexpr int XV = NP;  // NP * 2048 k / 8 per vector / 256 threads
     uint4 xstage[XV];
     const uint4 *xg = reinterpret_cast<const uint4 *>(a.x);
 #pragma unroll
@@ -137,6 +138,12 @@ gemv_w4a16_kernel(const Args a) {
 template <int NP>
 int launch(const Args &a, hipStream_t st) {
     const size_t lds = (size_t)a.K * 2 + sizeof(float) * a.G;
+    if (NP * 2048 * 2 > 60 * 1024) {  // beyond what a launch may ask for without saying so first
+        static std::atomic<uint64_t> devices{0};
+        if (const int rc = reserve_lds(reinterpret_cast<const void *>(gemv_w4a16_kernel<NP>),
+                                       NP * 2048 * 2 + (int)sizeof(float) * (NP * 2048 / GS), devices, "cmi_gemv_w4a16"))
+            return rc;
+    }
     gemv_w4a16_kernel<NP><<<dim3((a.N + WAVES - 1) / WAVES), dim3(64 * WAVES), lds, st>>>(a);
     return check_launch("cmi_gemv_w4a16");
 }
@@ -154,12 +161,22 @@ extern "C" int cmi_gemv_w4a16(const uint8_t *w4, const float *ws, const void *x,
                 "cmi_gemv_w4a16: w4 and x must be 16-byte aligned");
     Args a{w4, ws, static_cast<const uint16_t *>(x), static_cast<uint16_t *>(y), N, K, K / GS};
     hipStream_t st = static_cast<hipStream_t>(stream);
+    // one instantiation per pass count up to 5 (K <= 10240: the decode shapes), then steps of 2 and 3
     const int passes = (K / 32 + 63) / 64;
     switch (passes) {
         case 1: return launch<1>(a, st);
         case 2: return launch<2>(a, st);
         case 3: return launch<3>(a, st);
         case 4: return launch<4>(a, st);
-        default: return launch<5>(a, st);
+        case 5: return launch<5>(a, st);
+        case 6:
+        case 7: return launch<7>(a, st);
+        case 8:
+        case 9: return launch<9>(a, st);
+        case 10:
+        case 11: return launch<11>(a, st);
+        case 12:
+        case 13: return launch<13>(a, st);
+        default: return launch<16>(a, st);
     }
 }

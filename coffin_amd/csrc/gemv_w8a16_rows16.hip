@@ -60,7 +60,7 @@ __device__ __forceinline__ void widen4(uint32_t w, uint32_t &lo, uint32_t &hi) {
 // NLP: lines per wavefront and round.  WAVES: wavefronts per workgroup.  ROUNDS: 1, or 2 for
 // K above 128*NLP*WAVES (the second round's bytes are requested line by line as the first
 // round frees their registers; asking for all weight bytes at the start took 179 registers
-// and measured slower).
+// and measured slower), or 0: as many rounds as K takes, counted at run time (K above 10240).
 // T: 16-row tiles of weight rows per workgroup (the activation tiles a wavefront fetched and
 // rearranged serve all of them: at 16 rows they are two thirds of the bytes a wavefront asks for).
 template <int NLP, int WAVES, int ROUNDS, int T = 1>
@@ -128,8 +128,10 @@ gemv_w8a16_rows16_kernel(const Args a) {
     v4f32 acc[T];
 #pragma unroll
     for (int t = 0; t < T; ++t) acc[t] = v4f32{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int r = 0; r < ROUNDS; ++r) {
+    const int rounds = ROUNDS > 0 ? ROUNDS : (lines + NLP * WAVES - 1) / (NLP * WAVES);
+    constexpr int UNROLL = ROUNDS > 0 ? ROUNDS : 1;
+#pragma unroll UNROLL
+    for (int r = 0; r < rounds; ++r) {
         // activations into the MFMA arrangement: row lane%16, bytes 64*kq .. +63 of the line
 #pragma unroll
         for (int i = 0; i < NLP; ++i) {
@@ -162,7 +164,7 @@ gemv_w8a16_rows16_kernel(const Args a) {
                                                                      __builtin_bit_cast(bf16x8, bw), acc[t], 0, 0, 0);
                 }
             }
-            if (r + 1 < ROUNDS) {
+            if (r + 1 < rounds) {
                 request_x(r + 1, i);
                 request_w(r + 1, i);
             }
@@ -354,8 +356,7 @@ extern "C" int cmi_gemv_w8a16_mfma(const int8_t *wq, const float *ws, const void
     CMI_REQUIRE(wq && ws && x && y, CMI_E_ARG, "cmi_gemv_w8a16_mfma: null pointer");
     CMI_REQUIRE(M >= 1 && M <= MAX_CHUNKS * ROWS, CMI_E_UNSUPPORTED, "cmi_gemv_w8a16_mfma: M=%d outside 1..64", M);
     CMI_REQUIRE(N >= 1 && K >= 1, CMI_E_ARG, "cmi_gemv_w8a16_mfma: bad shape N=%d K=%d", N, K);
-    CMI_REQUIRE(K % LINE == 0 && K <= 80 * LINE, CMI_E_UNSUPPORTED,
-                "cmi_gemv_w8a16_mfma: K=%d is not a multiple of 128 up to 10240 (use cmi_gemv_w8a16)", K);
+    CMI_REQUIRE(K % LINE == 0, CMI_E_UNSUPPORTED, "cmi_gemv_w8a16_mfma: K=%d is not a multiple of 128 (use cmi_gemv_w8a16)", K);
     CMI_REQUIRE(aligned(wq, 16) && aligned(x, 16) && aligned(y, 2) && aligned(ws, 4), CMI_E_ARG,
                 "cmi_gemv_w8a16_mfma: wq and x must be 16-byte aligned");
     Args a;
@@ -368,6 +369,19 @@ extern "C" int cmi_gemv_w8a16_mfma(const int8_t *wq, const float *ws, const void
     a.K = K;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int lines = K / LINE;
+    if (lines > 80) {
+        // rows longer than two rounds of registers hold: the 16-row kernel with a round count read at
+        // run time, 16 activation rows per launch (a row's bits are those of a 16-row call, as in the
+        // 64-row kernel; the weight is read once per 16 rows)
+        for (int lo = 0; lo < M; lo += ROWS) {
+            Args part = a;
+            part.x = a.x + (size_t)lo * K;
+            part.y = a.y + (size_t)lo * N;
+            part.M = M - lo < ROWS ? M - lo : ROWS;
+            if (const int rc = launch<5, 8, 0>(part, st)) return rc;
+        }
+        return CMI_OK;
+    }
     if (M > ROWS) {
         if (lines <= 8) return launch64<2, 4>(a, st);
         if (lines <= 20 && (N + ROWS - 1) / ROWS > 2048) return launch64<5, 4>(a, st);

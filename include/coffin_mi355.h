@@ -82,9 +82,9 @@ int cmi_gemv_w8a16(const int8_t *wq, const float *ws, const void *x, void *y,
 
 /* The same product for a batch with the sums on the matrix pipe
  * (v_mfma_f32_16x16x32_bf16; int8 -> bf16 is exact), 1 <= M <= 16,
- * K % 128 == 0, K <= 10240 (else CMI_E_UNSUPPORTED: use cmi_gemv_w8a16); also
- * up to 64 rows (the weight is still read once, the rows go through in chunks
- * of 16 with the 16-row arithmetic).
+ * K % 128 == 0 (else CMI_E_UNSUPPORTED: use cmi_gemv_w8a16); also
+ * up to 64 rows (up to K = 10240 the weight is still read once, the rows go through in chunks
+ * of 16 with the 16-row arithmetic; longer weight rows are read once per 16 activation rows).
  * 2-3 times faster than cmi_gemv_w8a16 at 8-16 rows.  A row's bits depend on K
  * only, not on the rows it travels with, but differ from cmi_gemv_w8a16's in
  * the last place (fp32 summation order): for callers without the
@@ -99,7 +99,7 @@ int cmi_gemv_w8a16_mfma(const int8_t *wq, const float *ws, const void *x, void *
 /* int8 weight-only projection of any number of rows, with the kernel family named by the caller:
  *   CMI_FAMILY_DOT   cmi_gemv_w8a16, 16 rows per launch: row m carries the bits of the single-row call
  *                    (what static-batch decode owes its users, models/qwen35/batch.py:19-22);
- *   CMI_FAMILY_MFMA  cmi_gemv_w8a16_mfma, 64 rows per launch (K % 128 == 0, K <= 10240, else
+ *   CMI_FAMILY_MFMA  cmi_gemv_w8a16_mfma, 64 rows per launch (K % 128 == 0, else
  *                    CMI_E_UNSUPPORTED and nothing is launched): 1.5-2.8 times faster at 4-16 rows,
  *                    slower at one row; a row's bits depend on K only.
  * The rule holds inside either family as long as every call on a weight -- single rows included --
@@ -148,7 +148,8 @@ int cmi_gemv_w4a8(const uint8_t *w4, const float *ws, const int8_t *xq, const fl
 /* int4 weight-only GEMV on *unquantised* bf16 activations (W4A16), one activation row, on the
  * re-laid-out weight:
  *   y[n] = bf16( sum_g ws[n,g] * sum_{k in g} (code - 8) * x[k] ),  fp32 sums in an order that
- * depends on K only.  K % 128 == 0, gs == 128, K <= 10240.  This is what the reference's torch
+ * depends on K only.  K % 128 == 0, gs == 128, K <= 32768 (a wavefront keeps its weight row in
+ * registers).  This is what the reference's torch
  * path computes for an int4 weight (backends/reference/__init__.py:93-95 with
  * w4a8_weights.py:96-99: no activation quantisation) up to fp32 summation order, and stands where
  * gemv_kn_w4 is bound (backends/corex/kernels/gemv.cu:1918-1930, 1935-1975). */

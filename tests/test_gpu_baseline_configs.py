@@ -152,7 +152,9 @@ def test_w4a8_kernels_stay_within_quantisation_error_of_the_unquantised_referenc
 # ------------------------------------------------------------- W4A16 (int4 weight-only) GEMV
 
 @pytest.mark.parametrize("n,k", [(9728, 2560), (2560, 9728), (2560, 4096), (6144, 2560), (37, 128), (1001, 384),
-                                 (300, 2048), (64, 10240), (5, 6272)])
+                                 (300, 2048), (64, 10240), (5, 6272),
+                                 # rows longer than 10240: 6..16 passes (config 5's 25600 -> 5120 among them)
+                                 (5120, 25600), (100, 12288), (33, 16384), (17, 20480), (40, 32768), (9, 28672)])
 def test_gemv_w4a16_against_the_exact_sum_and_the_unquantised_reference(orc, n, k):
     """The int4 weight-only GEMV is a floating-point path (fp32 sums in the kernel's own order):
     held to the exact value of sum_k (code - 8) * scale * x within its final bf16 rounding plus

@@ -153,10 +153,12 @@ def test_gemv_w8a16_whole_row_kernel_gives_the_general_kernels_bits(orc, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(16, 9728, 2560), (5, 2560, 9728), (7, 37, 128), (9, 100, 384),
                                    (16, 64, 10240), (6, 530, 1152), (1, 333, 2560), (3, 2560, 4096),
-                                   (16, 1024, 5120), (12, 640, 3072), (2, 96, 8192), (16, 300, 6656)])
+                                   (16, 1024, 5120), (12, 640, 3072), (2, 96, 8192), (16, 300, 6656),
+                                   # rows longer than two rounds of registers: the round count read at run time
+                                   (16, 64, 10368), (5, 5120, 25600), (16, 100, 12800), (1, 77, 16384), (9, 40, 65536)])
 def test_gemv_w8a16_mfma_within_tolerance(orc, m, n, k):
     """The matrix-pipe GEMV: same tolerance bars as the dot-product kernel, every
-    lines-per-wavefront variant, one and two rounds, ragged N."""
+    lines-per-wavefront variant, one, two and more rounds, ragged N."""
     wq, ws, x, y = _w8a16_case(orc, m, n, k, seeded(), mfma=True)
     _assert_weight_only_tolerance(orc, wq, ws, x, y)
 
@@ -164,7 +166,9 @@ def test_gemv_w8a16_mfma_within_tolerance(orc, m, n, k):
 @pytest.mark.parametrize("n,k", [(9728, 2560), (300, 5120), (70, 1024), (33000, 2560), (2560, 4096),
                                  (2560, 9728), (100, 10240), (77, 6656),
                                  # two and three weight tiles per workgroup, both 8-wavefront line counts, ragged N
-                                 (6144, 2560), (6100, 2560), (9000, 3200), (5120, 5120), (11008, 4096)])
+                                 (6144, 2560), (6100, 2560), (9000, 3200), (5120, 5120), (11008, 4096),
+                                 # long weight rows: one launch per 16 activation rows
+                                 (300, 12800), (5120, 25600)])
 def test_gemv_w8a16_mfma_wide_batches_carry_the_16_row_bits(n, k):
     """17..64 rows in one launch (one, two or three 16-row weight tiles per workgroup): every row
     has the bits of a 16-row call."""
@@ -202,7 +206,7 @@ def test_gemv_w8a16_batched_row_equals_single_row(n, k):
         assert (y.view(torch.int16) == single[:m].view(torch.int16)).all(), m
 
 
-@pytest.mark.parametrize("n,k", [(4096, 2560), (2560, 9728), (512, 5120), (300, 6656), (64, 128)])
+@pytest.mark.parametrize("n,k", [(4096, 2560), (2560, 9728), (512, 5120), (300, 6656), (64, 128), (200, 25600)])
 def test_gemv_w8a16_mfma_rows_do_not_depend_on_the_batch(n, k):
     """The matrix-pipe GEMV makes the weaker promise: a row's bits depend on K only, not on
     the rows it travels with (also one row alone); against the dot-product kernel the

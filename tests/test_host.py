@@ -375,7 +375,6 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     assert "null pointer" in _native.last_error()
     assert lib.cmi_gemv_w8a16_mfma(one, one, one, one, 65, 8, 128, null) == _native.E_UNSUPPORTED
     assert lib.cmi_gemv_w8a16_mfma(one, one, one, one, 4, 8, 64, null) == _native.E_UNSUPPORTED
-    assert lib.cmi_gemv_w8a16_mfma(one, one, one, one, 4, 8, 10368, null) == _native.E_UNSUPPORTED
     assert "multiple of 128" in _native.last_error()
     assert lib.cmi_gemv_w8a16_mfma(null, one, one, one, 4, 8, 128, null) == _native.E_ARG
     assert lib.cmi_gemv_w8a16(one, one, one, one, 17, 8, 16, null) == _native.E_UNSUPPORTED
