@@ -141,7 +141,9 @@ def parse_args():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawTextHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    # 20 untimed steps (16 ms): with 3 the clocks have not settled and the timed steps read 0.816-0.826 ms
+    # from run to run instead of 0.810-0.811
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--rows", type=int, default=1, help="activation rows M of the headline workload")
     ap.add_argument("--mfma", action="store_true",
                     help="headline workload through cmi_gemv_w8a16_mfma (the verify / short-prefill kernel) "
