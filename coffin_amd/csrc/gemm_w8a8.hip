@@ -1275,8 +1275,6 @@ gemm_w8a8_wide_tilewise_kernel(const Args a) {
 
 int launch_wide(Args &a, hipStream_t st);
 
-int wide_tiles(int M, int N) { return ((M + wide::BM - 1) / wide::BM) * ((N + wide::BN - 1) / wide::BN); }
-
 int launch_wide_tilewise(Args &a, hipStream_t st) {
     // buffer offsets are 32 bits: matrices (and the tile rows past their end) must stay below 2 GiB
     if ((size_t)(a.N + wide::BN) * a.K >= ((size_t)1 << 31) || (size_t)(a.M + wide::BM) * a.K >= ((size_t)1 << 31))
@@ -1495,14 +1493,17 @@ int cmi::gemm_w8a8_split(const int8_t *xq, const int8_t *wq, const float *xs, co
             }
         }
     }
-    // the 256 x 320 tile: the tile-wise kernel (1..3 % faster than the two-stage one on every shape
-    // tried, 7 % at 2048 x 4096 x 2560); a forced 320 still names the two-stage kernel
-    // The persistent form (322) keeps its pipeline running from tile to tile.  At the clock the power
-    // limit leaves a launch of this size, closing the gaps between tiles buys little: measured -2.4 %
-    // at 7.6 tiles per CU (8192 x 19456 x 2560, 372.9 -> 363.8 us, cold and warm weights alike),
-    // -2 % cold / +0.5 % warm at 3.9, and a single tile is 3 % slower than the one-tile kernel
-    // (its epilogue writes 32 bytes per row and store instead of whole rows).  From four tiles per CU.
-    if (pick == 322 || (pick == 320 && !force && wide_tiles(a.M, a.N) > 4 * compute_units())) return launch_wide_persistent(a, st);
+    // the 256 x 320 tile: the tile-wise kernel (within 1 % of the two-stage one on the large shapes,
+    // 7 % faster at 2048 x 4096 x 2560); a forced 320 still names the two-stage kernel
+    // The persistent form (322) keeps its pipeline running from tile to tile -- and takes the same time
+    // as the one-tile kernel: at the clock the power limit leaves these launches, closing the gaps
+    // between tiles is paid back in clock.  Alternating replays of the two, cold weights, medians:
+    // 8192 x 9728 x 2560 (3.9 tiles per CU) 178.0 / 177.9 us, 8192 x 19456 x 2560 (7.6) 372.4 / 371.5 and,
+    // in the other order, 359.3 / 356.4; 4096 x 9728 92.5 / 93.5; a single tile 49.3 / 51.1.  (A first
+    // comparison read -2 %: there the persistent kernel always ran behind the one-tile kernel and that
+    // one behind the slower 256 x 256 kernel, and what a launch follows moves it by more than that.)
+    // Kept for study under its code; the library's choice stays the one-tile kernel.
+    if (pick == 322) return launch_wide_persistent(a, st);
     if (pick == 321 || (pick == 320 && !force)) return launch_wide_tilewise(a, st);
     if (pick == 320) return launch_wide(a, st);
     if (pick == 256) return launch_big(a, st);

@@ -41,8 +41,8 @@ int cmi_abi_version(void);
  *                   | 128192 (128 n x 192 m) | 321 (the 256 x 320 tile walked weight tile by weight
  *                   tile: what the library runs where it chooses that tile; 320 names the older
  *                   two-stage kernel) | 322 (321 as one workgroup per CU that walks its tiles one
- *                   after the other: the library's choice where that tile gives more than four
- *                   tiles per CU): block tile of cmi_gemm_w8a8 / cmi_gemm_w4a8 (non-zero also
+ *                   after the other; measures the same as 321 and is never the library's choice):
+ *                   block tile of cmi_gemm_w8a8 / cmi_gemm_w4a8 (non-zero also
  *                   bypasses their few-row routes);
  *   "gemv_wholerow" -1 (the library chooses) | 0 (never) | 1: the one-wavefront-per-weight-row
  *                   kernel of cmi_gemv_w8a16;

@@ -389,10 +389,10 @@ def test_gemm_w8a8_full_size_sampled_and_blockwise(orc, gemm_tile, m, n):
 @pytest.mark.parametrize("m,n,k", [(4100, 6408, 512), (8192, 9728, 2560), (2100, 12808, 1024), (600, 45000, 768),
                                    (8200, 19456, 512)])
 def test_gemm_w8a8_workgroups_walking_several_tiles_give_the_one_tile_bits(orc, m, n, k):
-    """More 256 x 320 tiles than CUs: a workgroup of the persistent kernel (tile code 322, and the
-    library's own choice at the last shape, more than four tiles per CU) takes several, its requests running on from one tile
-    into the next and its results going from registers to memory.  Ragged last tiles in both
-    directions, a row pitch above N; bits of the 128 x 128 tile kernel and of the oracle."""
+    """More 256 x 320 tiles than CUs: a workgroup of the persistent kernel (tile code 322) takes
+    several, its requests running on from one tile into the next and its results going from
+    registers to memory.  Ragged last tiles in both directions, a row pitch above N; bits of the
+    128 x 128 tile kernel, of the library's own choice and of the oracle."""
     g = synth.generator(99, G.DEV)
     q = synth.int8_weight(n, k, g)
     x = synth.activations(m, k, g, outliers=True)
