@@ -1003,8 +1003,8 @@ def main() -> int:
         torch.cuda.empty_cache()
 
         w16 = {}
-        for n_, k_ in ((9728, 2560), (2560, 9728)):
-            copies = 16
+        for n_, k_ in ((9728, 2560), (2560, 9728), (5120, 25600)):
+            copies = 16 if k_ <= 10240 else 6
             ws4 = []
             for _ in range(copies):
                 w = synth.int4_weight(n_, k_, gen)
@@ -1028,6 +1028,28 @@ def main() -> int:
             w16[f"{k_}->{n_}"] = hbm_line(t, synth.w4_gemv_bytes(1, n_, k_))
             del ws4, gr
         extra["w4a16_gemv_M1_hipgraph"] = w16
+        torch.cuda.empty_cache()
+
+        # weight rows longer than two rounds of registers (K = 25600, the long side of the int4 model,
+        # as an int8 weight): both weight-only families at 1..64 rows, cold weights (4 x 131 MB)
+        n_, k_ = 5120, 25600
+        long_w = [synth.int8_weight(n_, k_, gen) for _ in range(4)]
+        long_rows = {}
+        for m in (1, 4, 16, 64):
+            xv = synth.activations(m, k_, gen)
+            yv = torch.empty((m, n_), dtype=torch.bfloat16, device=dev)
+            turn = [0]
+            def mfma_family():
+                c = long_w[turn[0] % 4]
+                turn[0] += 1
+                _native.check(lib.cmi_linear_w8a16(ptr(c.wq), ptr(c.scale), ptr(xv), ptr(yv), m, n_, k_, 1, cur_stream()), "linear_w8a16")
+            def dot_family():
+                c = long_w[turn[0] % 4]
+                turn[0] += 1
+                _native.check(lib.cmi_linear_w8a16(ptr(c.wq), ptr(c.scale), ptr(xv), ptr(yv), m, n_, k_, 0, cur_stream()), "linear_w8a16")
+            long_rows[f"M{m}"] = {"mfma_us": round(timed(mfma_family, 8) * 1e6, 1), "dot_us": round(timed(dot_family, 8) * 1e6, 1)}
+        extra["w8a16_long_rows_25600_to_5120_by_family"] = long_rows
+        del long_w
         result["extra"] = extra
 
     # ------------------------------------------------------------------ CPU baseline leg
